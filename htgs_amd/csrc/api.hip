@@ -1,0 +1,76 @@
+// C ABI glue: error reporting, size helpers and the two-call frame driver.
+// The launch order restates <mode>::inference (R/src/hybrid_blend/inference.cu:57-183 and its
+// siblings); the reference's single blocking read of the instance count (:118-119) is the seam
+// between htgs_render_front and htgs_render_back.
+#include "common.h"
+#include <cstdarg>
+#include <cstdio>
+
+namespace htgs {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char *what)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HTGS_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+    return HTGS_OK;
+}
+
+// extract_end_bit, R/include/rasterization_utils.h:3-13: bit width of n
+static int bit_width(uint32_t n)
+{
+    int b = 0;
+    while (n) { ++b; n >>= 1; }
+    return b;
+}
+
+}  // namespace htgs
+
+using namespace htgs;
+
+extern "C" const char *htgs_last_error(void) { return g_error; }
+
+extern "C" int htgs_tile_size(int mode) { return tile_size(mode); }
+
+extern "C" int htgs_end_bit(int mode, int width, int height)
+{
+    const int tile = tile_size(mode);
+    const uint32_t n_tiles = (uint32_t)div_up(width, tile) * (uint32_t)div_up(height, tile);
+    const int bits = bit_width(n_tiles - 1);
+    return mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING ? bits + 32 : bits;
+}
+
+extern "C" int htgs_key_bytes(int mode, int width, int height)
+{
+    if (mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING) return 8;
+    return htgs_end_bit(mode, width, height) <= 16 ? 2 : 4;
+}
+
+extern "C" int htgs_render_front(const htgs_frame *f)
+{
+    int rc = htgs_preprocess(f);
+    if (rc != HTGS_OK) return rc;
+    return htgs_scan_offsets(f);
+}
+
+extern "C" int htgs_render_back(const htgs_frame *f)
+{
+    int selector = 0;
+    int rc = htgs_create_instances(f);
+    if (rc != HTGS_OK) return rc;
+    rc = htgs_sort_instances(f, &selector);
+    if (rc != HTGS_OK) return rc;
+    rc = htgs_extract_ranges(f, selector);
+    if (rc != HTGS_OK) return rc;
+    return htgs_blend(f, selector);
+}

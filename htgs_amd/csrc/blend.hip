@@ -1,0 +1,362 @@
+// Per-tile blend kernels of the four modes (inference: image + depth).
+// Restates blend_cu of R/include/hybrid_blend/kernels/inference.cuh:78-216,
+// R/include/alpha_blend_first_k/kernels/inference.cuh:78-206,
+// R/include/alpha_blend_global_ordering/kernels/inference.cuh:78-176 and
+// R/include/oit_blend/kernels/inference.cuh:78-177.
+//
+// An 8x8 tile is exactly one wave64: one workgroup = one wave, Gaussian records are staged 64 at a
+// time in LDS (every lane then reads the same address, a broadcast), the K-buffer lives in VGPRs.
+// The 16x16 tiles of the global-ordering mode use four waves and a workgroup barrier.
+#include "common.h"
+
+namespace htgs {
+
+template <int N>
+struct Stage {
+    float4 v1[N], v2[N], v4[N], mt3[N], col[N];
+};
+
+template <int N>
+__device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
+                                           uint32_t fetch, uint32_t last, int slot, uint32_t *idx_out)
+{
+    if (fetch < last) {
+        const uint32_t g = inst[fetch];
+        const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
+        st.v1[slot] = rec[0];
+        st.v2[slot] = rec[1];
+        st.v4[slot] = rec[2];
+        st.mt3[slot] = rec[3];
+        st.col[slot] = rec[4];
+        if (idx_out) idx_out[slot] = g;
+    }
+}
+
+__device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__restrict__ depths, uint32_t w, uint32_t h,
+                                            uint32_t x, uint32_t y, bool chw, float r, float g, float b, float depth)
+{
+    const size_t pix = (size_t)w * y + x, np = (size_t)w * h;
+    r = saturate(r); g = saturate(g); b = saturate(b);
+    if (chw) { image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b; }
+    else { image[3 * pix] = r; image[3 * pix + 1] = g; image[3 * pix + 2] = b; }
+    depths[pix] = depth;
+}
+
+// ---------------------------------------------------------------------------------------------
+// HYBRID_BLEND: K nearest fragments with alpha >= 1/20 are alpha-blended in depth order, everything
+// else is merged order-independently into one tail fragment behind them.
+// ---------------------------------------------------------------------------------------------
+template <int K>
+__global__ void __launch_bounds__(64) blend_hybrid_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+{
+    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    __shared__ Stage<64> st;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+
+    float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f, depth_tail = 0.0f;
+    float c0[K], c1[K], c2[K], c3[K], cd[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) { c0[i] = c1[i] = c2[i] = c3[i] = 0.0f; cd[i] = __FLT_MAX__; }
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, nullptr);
+        __syncthreads();
+        if (inside) {
+            const int nb = last - base < 64u ? (int)(last - base) : 64;
+            for (int j = 0; j < nb; ++j) {
+                Frag f;
+                if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+                f.den_rcp = 1.0f / f.den;
+                const float4 col = st.col[j];
+                if (!frag_alpha<MODE>(col.w, f)) continue;
+                float depth = frag_depth(st.mt3[j], f);
+                float p0 = col.x * f.alpha, p1 = col.y * f.alpha, p2 = col.z * f.alpha, p3 = f.alpha;
+                if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
+#pragma unroll
+                    for (int i = 0; i < K; ++i) {
+                        if (depth < cd[i]) {
+                            float t;
+                            t = depth; depth = cd[i]; cd[i] = t;
+                            t = p0; p0 = c0[i]; c0[i] = t;
+                            t = p1; p1 = c1[i]; c1[i] = t;
+                            t = p2; p2 = c2[i]; c2[i] = t;
+                            t = p3; p3 = c3[i]; c3[i] = t;
+                        }
+                    }
+                }
+                tail0 += p0; tail1 += p1; tail2 += p2; tail3 += p3;
+                if (!median) depth_tail = __builtin_fmaf(depth, p3, depth_tail);
+                T_tail *= 1.0f - p3;
+            }
+        }
+    }
+    if (!inside) return;
+
+    float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T_core = 1.0f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        if (T_core >= kTransmittanceThreshold) {
+            r = __builtin_fmaf(T_core, c0[i], r);
+            g = __builtin_fmaf(T_core, c1[i], g);
+            b = __builtin_fmaf(T_core, c2[i], b);
+            if (median) depth_pixel = (T_core > 0.5f && cd[i] < __FLT_MAX__) ? cd[i] : depth_pixel;
+            else depth_pixel = __builtin_fmaf(T_core * c3[i], cd[i], depth_pixel);
+            T_core *= 1.0f - c3[i];
+        }
+    }
+    float total_alpha = 0.0f;
+    if (!median) total_alpha = 1.0f - T_core;
+    if (T_core >= kTransmittanceThreshold && tail3 >= ModeCfg<MODE>::min_alpha) {
+        const float weight_tail = T_core * (1.0f - T_tail);
+        const float wn = weight_tail * (1.0f / tail3);
+        r = __builtin_fmaf(wn, tail0, r);
+        g = __builtin_fmaf(wn, tail1, g);
+        b = __builtin_fmaf(wn, tail2, b);
+        if (!median) { depth_pixel = __builtin_fmaf(wn, depth_tail, depth_pixel); total_alpha += weight_tail; }
+    }
+    if (!median) depth_pixel = total_alpha > 0.0f ? depth_pixel / total_alpha : 0.0f;
+    store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
+}
+
+// ---------------------------------------------------------------------------------------------
+// ALPHA_BLEND_FIRST_K: the K nearest fragments with alpha >= 1/20, alpha-blended; no tail.
+// ---------------------------------------------------------------------------------------------
+template <int K>
+__global__ void __launch_bounds__(64) blend_first_k_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
+    __shared__ Stage<64> st;
+    __shared__ uint32_t st_idx[64];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+
+    float ca[K], cd[K];
+    uint32_t ci[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) { ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        __syncthreads();
+        if (inside) {
+            const int nb = last - base < 64u ? (int)(last - base) : 64;
+            for (int j = 0; j < nb; ++j) {
+                Frag f;
+                if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+                f.den_rcp = 1.0f / f.den;
+                float depth = frag_depth(st.mt3[j], f);
+                if (depth >= cd[K - 1]) continue;                      // depth test before the exponential (:151)
+                if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+                float alpha = f.alpha;
+                uint32_t idx = st_idx[j];
+#pragma unroll
+                for (int i = 0; i < K; ++i) {
+                    if (depth < cd[i]) {
+                        float t;
+                        t = depth; depth = cd[i]; cd[i] = t;
+                        t = alpha; alpha = ca[i]; ca[i] = t;
+                        const uint32_t ti = idx; idx = ci[i]; ci[i] = ti;
+                    }
+                }
+            }
+        }
+    }
+    if (!inside) return;
+
+    float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T = 1.0f;
+    bool open = true;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        open = open && T >= kTransmittanceThreshold && ci[i] != 0xffffffffu;
+        if (open) {
+            const float wgt = T * ca[i];
+            const float4 col = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS / 4) + 4];
+            r = __builtin_fmaf(wgt, col.x, r);
+            g = __builtin_fmaf(wgt, col.y, g);
+            b = __builtin_fmaf(wgt, col.z, b);
+            if (median) depth_pixel = T > 0.5f ? cd[i] : depth_pixel;
+            else depth_pixel = __builtin_fmaf(wgt, cd[i], depth_pixel);
+            T *= 1.0f - ca[i];
+        }
+    }
+    if (!median) depth_pixel = T < 1.0f ? depth_pixel / (1.0f - T) : 0.0f;
+    store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
+}
+
+// ---------------------------------------------------------------------------------------------
+// OIT_BLEND: weighted-sum order-independent transparency over all fragments.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(64) blend_oit_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw)
+{
+    constexpr int MODE = HTGS_MODE_OIT_BLEND;
+    __shared__ Stage<64> st;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, nullptr);
+        __syncthreads();
+        if (inside) {
+            const int nb = last - base < 64u ? (int)(last - base) : 64;
+            for (int j = 0; j < nb; ++j) {
+                Frag f;
+                if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+                f.den_rcp = 1.0f / f.den;
+                const float4 col = st.col[j];
+                if (!frag_alpha<MODE>(col.w, f)) continue;
+                const float depth = frag_depth(st.mt3[j], f);
+                a0 = __builtin_fmaf(f.alpha, col.x, a0);
+                a1 = __builtin_fmaf(f.alpha, col.y, a1);
+                a2 = __builtin_fmaf(f.alpha, col.z, a2);
+                a3 = __builtin_fmaf(f.alpha, depth, a3);
+                alpha_sum += f.alpha;
+                T *= 1.0f - f.alpha;
+            }
+        }
+    }
+    if (!inside) return;
+    float r = 0.0f, g = 0.0f, b = 0.0f, d = 0.0f;
+    if (alpha_sum >= ModeCfg<MODE>::min_alpha) {
+        const float alpha = 1.0f - T;
+        const float s = alpha * (1.0f / alpha_sum);
+        r = s * a0; g = s * a1; b = s * a2;
+        d = (s * a3) / alpha;
+    }
+    store_pixel(image, depths, width, height, x, y, chw, r, g, b, d);
+}
+
+// ---------------------------------------------------------------------------------------------
+// ALPHA_BLEND_GLOBAL_ORDERING: instances arrive sorted by (tile, depth of the Gaussian centre);
+// classic front-to-back blending, a pixel stops at T < 1e-4, the workgroup stops when all have.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) blend_global_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
+    __shared__ Stage<256> st;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t t = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+    float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T = 1.0f;
+    bool done = !inside;
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 256) {
+        if (__syncthreads_count(done) == 256) break;
+        stage_load(st, prim, inst, base + t, last, t, nullptr);
+        __syncthreads();
+        const int nb = last - base < 256u ? (int)(last - base) : 256;
+        for (int j = 0; !done && j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            const float4 col = st.col[j];
+            if (!frag_alpha<MODE>(col.w, f)) continue;
+            const float wgt = T * f.alpha;
+            r = __builtin_fmaf(wgt, col.x, r);
+            g = __builtin_fmaf(wgt, col.y, g);
+            b = __builtin_fmaf(wgt, col.z, b);
+            const float depth = st.mt3[j].w;
+            if (median) depth_pixel = T > 0.5f ? depth : depth_pixel;
+            else depth_pixel = __builtin_fmaf(wgt, depth, depth_pixel);
+            T *= 1.0f - f.alpha;
+            if (T < kTransmittanceThreshold) done = true;
+        }
+    }
+    if (!inside) return;
+    if (!median) depth_pixel = T < 1.0f ? depth_pixel / (1.0f - T) : 0.0f;
+    store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
+}
+
+template <int K>
+static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
+{
+    hipLaunchKernelGGL((blend_hybrid_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                       (const float4 *)f->prim, f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+}
+template <int K>
+static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
+{
+    hipLaunchKernelGGL((blend_first_k_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                       (const float4 *)f->prim, f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+}
+
+}  // namespace htgs
+
+using namespace htgs;
+
+extern "C" int htgs_effective_k(int K)
+{
+    return K >= 32 ? 32 : K >= 16 ? 16 : K >= 8 ? 8 : K >= 4 ? 4 : K >= 2 ? 2 : 1;
+}
+
+extern "C" int htgs_blend(const htgs_frame *f, int selector)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: null frame");
+    if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
+    if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: bad argument");
+    if (!f->ranges || !f->image || !f->depth || (f->n_instances > 0 && (!f->vals[selector] || !f->prim)))
+        return fail(HTGS_ERR_ARGUMENT, "htgs_blend: null pointer");
+    const int tile = tile_size(f->mode);
+    const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
+    const uint32_t n_tiles = grid_w * grid_h;
+    const int K = htgs_effective_k(f->K);
+    hipStream_t s = (hipStream_t)f->stream;
+    switch (f->mode) {
+        case HTGS_MODE_HYBRID_BLEND:
+            switch (K) {
+                case 32: launch_hybrid<32>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_hybrid<16>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_hybrid<8>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_hybrid<4>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_hybrid<2>(f, selector, grid_w, n_tiles); break;
+                default: launch_hybrid<1>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_ALPHA_BLEND_FIRST_K:
+            switch (K) {
+                case 32: launch_first_k<32>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_first_k<16>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_first_k<8>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_first_k<4>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_first_k<2>(f, selector, grid_w, n_tiles); break;
+                default: launch_first_k<1>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING:
+            hipLaunchKernelGGL(blend_global_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
+                               f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+            break;
+        default:
+            hipLaunchKernelGGL(blend_oit_kernel, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
+                               f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw);
+            break;
+    }
+    return check_launch("blend");
+}

@@ -1,0 +1,199 @@
+// Stable least-significant-digit radix sort of (key, primitive index) pairs, 8 bits per pass, for
+// 16-, 32- and 64-bit keys.  Replaces cub::DeviceRadixSort::SortPairs(begin_bit = 0, end_bit)
+// at R/src/hybrid_blend/inference.cu:145-153 (64-bit tile|depth keys:
+// R/src/alpha_blend_global_ordering/inference.cu:117-124).
+//
+// One pass = three launches and no inter-block waiting:
+//   digit_histogram : per-block digit counts, stored digit-major   hist[digit][block]
+//   digit_row_scan  : one block per digit: exclusive scan along its row, row total
+//   digit_scatter   : re-reads the block's items, ranks them stably with wave64 ballots, scatters
+// Item order inside a block is (wave, round, lane); every rank below is computed in that order,
+// which is what keeps equal keys in their input order.
+#include "common.h"
+
+namespace htgs {
+
+constexpr int kSortThreads = 256;
+constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kSortItems = 16;                              // rounds per wave
+constexpr int kSortTile = kSortThreads * kSortItems;        // 4096 items per block
+constexpr int kRadix = 256;
+
+template <typename KeyT>
+__device__ __forceinline__ uint32_t digit_of(KeyT k, int shift, uint32_t mask) { return (uint32_t)(k >> shift) & mask; }
+
+template <typename KeyT>
+__global__ void __launch_bounds__(kSortThreads) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
+                                                                     uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
+{
+    __shared__ uint32_t counts[kRadix];
+    counts[threadIdx.x] = 0;
+    __syncthreads();
+    const uint64_t base = (uint64_t)blockIdx.x * kSortTile;
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const uint64_t i = base + (uint64_t)r * kSortThreads + threadIdx.x;
+        if (i < n) atomicAdd(&counts[digit_of(keys[i], shift, mask)], 1u);
+    }
+    __syncthreads();
+    hist[(size_t)threadIdx.x * n_blocks + blockIdx.x] = counts[threadIdx.x];
+}
+
+// block d scans row d of hist in place (exclusive) and writes the row total to totals[d]
+__global__ void __launch_bounds__(kSortThreads) digit_row_scan_kernel(uint32_t *__restrict__ hist, uint32_t *__restrict__ totals, uint32_t n_blocks)
+{
+    __shared__ uint32_t wave_sums[kSortWaves];
+    uint32_t *row = hist + (size_t)blockIdx.x * n_blocks;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    uint32_t carry = 0;
+    for (uint32_t start = 0; start < n_blocks; start += kSortThreads) {
+        const uint32_t i = start + threadIdx.x;
+        const uint32_t v = i < n_blocks ? row[i] : 0u;
+        uint32_t inc = v;
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            const uint32_t t = __shfl_up(inc, d, kWave);
+            if (lane >= d) inc += t;
+        }
+        if (lane == kWave - 1) wave_sums[wave] = inc;
+        __syncthreads();
+        uint32_t before = 0, all = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) {
+            const uint32_t s = wave_sums[w];
+            if (w < wave) before += s;
+            all += s;
+        }
+        __syncthreads();
+        if (i < n_blocks) row[i] = carry + before + inc - v;
+        carry += all;
+    }
+    if (threadIdx.x == 0) totals[blockIdx.x] = carry;
+}
+
+template <typename KeyT>
+__global__ void __launch_bounds__(kSortThreads) digit_scatter_kernel(
+    const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
+    const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
+{
+    __shared__ uint32_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the output base
+    __shared__ uint32_t wave_sums[kSortWaves];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; ++w) counts[w][threadIdx.x] = 0;
+    __syncthreads();
+
+    const uint64_t wave_base = (uint64_t)blockIdx.x * kSortTile + (uint64_t)wave * (kWave * kSortItems);
+    KeyT key[kSortItems];
+    uint32_t rank[kSortItems];
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const uint64_t i = wave_base + (uint64_t)r * kWave + lane;
+        const bool valid = i < n;
+        key[r] = valid ? keys_in[i] : (KeyT)0;
+        const uint32_t d = digit_of(key[r], shift, mask);
+        // lanes of this wave holding the same digit
+        uint64_t peers = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t vote = __ballot(bit);
+            peers &= bit ? vote : ~vote;
+        }
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+        uint32_t seen = 0;
+        if (valid) {
+            seen = counts[wave][d];
+            if (below == 0) counts[wave][d] = seen + (uint32_t)__builtin_popcountll(peers);
+        }
+        rank[r] = seen + below;
+    }
+    __syncthreads();
+
+    // output base of (wave, digit): global digit base + this block's offset inside the digit + earlier waves
+    {
+        const uint32_t d = threadIdx.x;
+        const uint32_t total = totals[d];
+        uint32_t inc = total;
+#pragma unroll
+        for (int s = 1; s < kWave; s <<= 1) {
+            const uint32_t t = __shfl_up(inc, s, kWave);
+            if (lane >= s) inc += t;
+        }
+        if (lane == kWave - 1) wave_sums[wave] = inc;
+        __syncthreads();
+        uint32_t before = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w)
+            if (w < wave) before += wave_sums[w];
+        uint32_t run = before + inc - total + hist[(size_t)d * n_blocks + blockIdx.x];
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) {
+            const uint32_t c = counts[w][d];
+            counts[w][d] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const uint64_t i = wave_base + (uint64_t)r * kWave + lane;
+        if (i < n) {
+            const uint32_t pos = counts[wave][digit_of(key[r], shift, mask)] + rank[r];
+            keys_out[pos] = key[r];
+            vals_out[pos] = vals_in[i];
+        }
+    }
+}
+
+template <typename KeyT>
+static int sort_pairs(const htgs_frame *f, int end_bit, int *selector)
+{
+    hipStream_t s = (hipStream_t)f->stream;
+    const uint64_t n = f->n_instances;
+    const uint32_t n_blocks = (uint32_t)((n + kSortTile - 1) / kSortTile);
+    uint32_t *hist = f->sort_tmp;
+    uint32_t *totals = f->sort_tmp + (size_t)kRadix * n_blocks;
+    int cur = 0;
+    for (int shift = 0; shift < end_bit; shift += 8) {
+        const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+        const uint32_t mask = (1u << bits) - 1u;
+        const KeyT *kin = (const KeyT *)f->keys[cur];
+        KeyT *kout = (KeyT *)f->keys[cur ^ 1];
+        hipLaunchKernelGGL((digit_histogram_kernel<KeyT>), dim3(n_blocks), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
+        hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kSortThreads), 0, s, hist, totals, n_blocks);
+        hipLaunchKernelGGL((digit_scatter_kernel<KeyT>), dim3(n_blocks), dim3(kSortThreads), 0, s, kin, f->vals[cur], kout, f->vals[cur ^ 1],
+                           hist, totals, n, n_blocks, shift, mask);
+        cur ^= 1;
+    }
+    *selector = cur;
+    return check_launch("sort");
+}
+
+}  // namespace htgs
+
+using namespace htgs;
+
+extern "C" size_t htgs_sort_tmp_words(uint64_t n_instances)
+{
+    const uint64_t n_blocks = (n_instances + kSortTile - 1) / kSortTile;
+    return (size_t)(kRadix * (n_blocks > 0 ? n_blocks : 1) + kRadix);
+}
+
+extern "C" int htgs_sort_instances(const htgs_frame *f, int *selector)
+{
+    if (!f || !selector) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: null argument");
+    if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
+    *selector = 0;
+    if (f->n_instances == 0) return HTGS_OK;
+    if (f->n_instances > 0xffffffffull) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: more than 2^32-1 instances");
+    if (!f->keys[0] || !f->keys[1] || !f->vals[0] || !f->vals[1] || !f->sort_tmp)
+        return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: null pointer");
+    const int end_bit = htgs_end_bit(f->mode, f->width, f->height);
+    switch (htgs_key_bytes(f->mode, f->width, f->height)) {
+        case 8: return sort_pairs<uint64_t>(f, end_bit, selector);
+        case 4: return sort_pairs<uint32_t>(f, end_bit, selector);
+        default: return sort_pairs<uint16_t>(f, end_bit, selector);
+    }
+}

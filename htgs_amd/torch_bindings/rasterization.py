@@ -1,0 +1,220 @@
+"""Operator API of the rasterizer on PyTorch-ROCm.
+
+Same names, argument order, shapes and error behaviour as the reference's
+``HTGSCudaBackend/HTGSCudaBackend/torch_bindings/rasterization.py`` (``RasterizerMode`` :9-13,
+``RasterizerSettings`` :16-42, ``rasterize`` :140-163), implemented on the C ABI of ``libhtgs_amd.so``:
+torch only owns the device memory and the stream, every kernel is hand-written HIP.
+"""
+from __future__ import annotations
+
+import ctypes
+from enum import Enum
+from typing import NamedTuple, Optional
+
+import torch
+
+from .. import _native
+
+
+class RasterizerMode(Enum):
+    HYBRID_BLEND = 0
+    ALPHA_BLEND_FIRST_K = 1
+    ALPHA_BLEND_GLOBAL_ORDERING = 2
+    OIT_BLEND = 3
+
+
+class RasterizerSettings(NamedTuple):
+    M: torch.Tensor  # [4,4] world -> camera
+    VPM: torch.Tensor  # [4,4] world -> screen (pixel coordinates with the half-pixel shift, NDC depth)
+    cam_position: torch.Tensor  # [3] world space
+    mode: RasterizerMode
+    K: int  # core size of HYBRID_BLEND / ALPHA_BLEND_FIRST_K
+    active_sh_bases: int
+    width: int
+    height: int
+    near_plane: float
+    far_plane: float
+    scale_modifier: float
+
+    def as_tuple(self) -> tuple:
+        return (self.M, self.VPM, self.cam_position, self.mode.value, self.K, self.active_sh_bases,
+                self.width, self.height, self.near_plane, self.far_plane, self.scale_modifier)
+
+
+def _mode_value(mode) -> int:
+    return int(mode.value) if isinstance(mode, Enum) else int(mode)
+
+
+def _dev_f32(t: torch.Tensor, name: str, device: Optional[torch.device] = None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device})")
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be float32 (got {t.dtype})")
+    if device is not None and t.device != device:
+        raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+    return t.contiguous()
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None or t.numel() == 0 else t.data_ptr()
+
+
+class FrameBuffers:
+    """One frame on the C ABI: validated inputs, caller-owned scratch, outputs.
+
+    Scratch mirrors the reference's PerPrimitive / PerTile / PerInstance blobs
+    (R/include/hybrid_blend/buffer_utils.h:22-94) as individual torch tensors.  The methods map one to
+    one onto the entry points of ``include/htgs_amd.h`` so that tests and the benchmark can run and time
+    single stages; ``rasterize`` runs ``front`` / ``back``.
+    """
+
+    def __init__(self, positions, scales, rotations, opacities, sh_0, sh_rest, settings: RasterizerSettings,
+                 to_chw: bool = True, use_median_depth: bool = False, train: bool = False):
+        mode = _mode_value(settings.mode)
+        if mode not in (0, 1, 2, 3):
+            raise RuntimeError("unsupported rasterizer mode")
+        self.lib = _native.lib()
+        positions = _dev_f32(positions, "positions")
+        dev = positions.device
+        self.device = dev
+        self.positions = positions
+        self.scales = _dev_f32(scales, "scales", dev)
+        self.rotations = _dev_f32(rotations, "rotations", dev)
+        self.opacities = _dev_f32(opacities, "opacities", dev)
+        self.sh_0 = _dev_f32(sh_0, "sh_0", dev)
+        self.sh_rest = _dev_f32(sh_rest, "sh_rest", dev)
+        self.M = _dev_f32(settings.M, "settings.M", dev)
+        self.VPM = _dev_f32(settings.VPM, "settings.VPM", dev)
+        self.cam_position = _dev_f32(settings.cam_position, "settings.cam_position", dev)
+        n = positions.shape[0]
+        if positions.shape != (n, 3) or self.scales.shape != (n, 3) or self.rotations.shape != (n, 4) \
+                or self.opacities.numel() != n or self.sh_0.numel() != 3 * n or self.sh_rest.dim() != 3 \
+                or self.sh_rest.shape[0] != n or self.sh_rest.shape[2] != 3:
+            raise RuntimeError("inconsistent Gaussian tensor shapes")
+        if self.M.numel() != 16 or self.VPM.numel() != 16 or self.cam_position.numel() != 3:
+            raise RuntimeError("settings.M / VPM must be 4x4 and cam_position must have 3 elements")
+        self.n = n
+        self.mode = mode
+        self.width, self.height = int(settings.width), int(settings.height)
+        self.tile = self.lib.htgs_tile_size(mode)
+        self.grid_w = (self.width + self.tile - 1) // self.tile
+        self.grid_h = (self.height + self.tile - 1) // self.tile
+        self.n_tiles = self.grid_w * self.grid_h
+        self.key_bytes = self.lib.htgs_key_bytes(mode, self.width, self.height)
+        self.end_bit = self.lib.htgs_end_bit(mode, self.width, self.height)
+        self.to_chw = bool(to_chw)
+
+        u32 = dict(dtype=torch.int32, device=dev)
+        self.n_touched = torch.empty(n, **u32)
+        self.offsets = torch.empty(n, **u32)
+        self.bounds = torch.empty((n, 4), dtype=torch.int16, device=dev)
+        self.prim = torch.empty((n, _native.PRIM_FLOATS), dtype=torch.float32, device=dev)
+        self.clamp_info = torch.empty((3, n), dtype=torch.uint8, device=dev) if train else None
+        self.scan_tmp = torch.empty(self.lib.htgs_scan_tmp_words(n), **u32)
+        self.n_instances_dev = torch.zeros(1, **u32)
+        self.ranges = torch.empty((self.n_tiles, 2), **u32)
+        self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
+                                 dtype=torch.float32, device=dev)
+        self.depth = torch.empty((self.height, self.width), dtype=torch.float32, device=dev)
+        self.keys = [None, None]
+        self.vals = [None, None]
+        self.sort_tmp = None
+        self.n_instances = 0
+        self.selector = 0
+
+        f = _native.Frame()
+        f.positions, f.scales, f.rotations = _ptr(self.positions), _ptr(self.scales), _ptr(self.rotations)
+        f.opacities, f.sh_0, f.sh_rest = _ptr(self.opacities), _ptr(self.sh_0), _ptr(self.sh_rest)
+        f.M, f.VPM, f.cam_position = _ptr(self.M), _ptr(self.VPM), _ptr(self.cam_position)
+        f.n_primitives = n
+        f.total_sh_bases = int(self.sh_rest.shape[1])
+        f.active_sh_bases = int(settings.active_sh_bases)
+        f.mode, f.K = mode, int(settings.K)
+        f.width, f.height = self.width, self.height
+        f.near_plane, f.far_plane = float(settings.near_plane), float(settings.far_plane)
+        f.scale_modifier = float(settings.scale_modifier)
+        f.n_touched, f.offsets, f.bounds, f.prim = _ptr(self.n_touched), _ptr(self.offsets), _ptr(self.bounds), _ptr(self.prim)
+        f.clamp_info = _ptr(self.clamp_info)
+        f.scan_tmp, f.n_instances_dev = _ptr(self.scan_tmp), _ptr(self.n_instances_dev)
+        f.ranges = _ptr(self.ranges)
+        f.image, f.depth = _ptr(self.image), _ptr(self.depth)
+        f.to_chw, f.use_median_depth = int(bool(to_chw)), int(bool(use_median_depth))
+        f.stream = torch.cuda.current_stream(dev).cuda_stream
+        self.frame = f
+        self._ref = ctypes.byref(f)
+
+    # ---- stages -----------------------------------------------------------------------------
+    def preprocess(self):
+        _native.check(self.lib.htgs_preprocess(self._ref))
+
+    def scan(self):
+        _native.check(self.lib.htgs_scan_offsets(self._ref))
+
+    def front(self):
+        _native.check(self.lib.htgs_render_front(self._ref))
+
+    def read_instance_count(self) -> int:
+        """The frame's only host/device synchronisation (the reference's cudaMemcpy at
+        R/src/hybrid_blend/inference.cu:118-119)."""
+        return int(self.n_instances_dev.item()) & 0xffffffff if self.n > 0 else 0
+
+    def alloc_instances(self, n_instances: int):
+        dev = self.device
+        self.n_instances = int(n_instances)
+        key_dtype = {2: torch.int16, 4: torch.int32, 8: torch.int64}[self.key_bytes]
+        m = max(self.n_instances, 1)
+        self.keys = [torch.empty(m, dtype=key_dtype, device=dev) for _ in range(2)]
+        self.vals = [torch.empty(m, dtype=torch.int32, device=dev) for _ in range(2)]
+        self.sort_tmp = torch.empty(self.lib.htgs_sort_tmp_words(self.n_instances), dtype=torch.int32, device=dev)
+        f = self.frame
+        f.n_instances = self.n_instances
+        f.keys[0], f.keys[1] = _ptr(self.keys[0]), _ptr(self.keys[1])
+        f.vals[0], f.vals[1] = _ptr(self.vals[0]), _ptr(self.vals[1])
+        f.sort_tmp = _ptr(self.sort_tmp)
+
+    def create_instances(self):
+        _native.check(self.lib.htgs_create_instances(self._ref))
+
+    def sort(self) -> int:
+        sel = ctypes.c_int(0)
+        _native.check(self.lib.htgs_sort_instances(self._ref, ctypes.byref(sel)))
+        self.selector = sel.value
+        return self.selector
+
+    def extract_ranges(self):
+        _native.check(self.lib.htgs_extract_ranges(self._ref, self.selector))
+
+    def blend(self):
+        _native.check(self.lib.htgs_blend(self._ref, self.selector))
+
+    def back(self):
+        _native.check(self.lib.htgs_render_back(self._ref))
+        self.selector = ((self.end_bit + 7) // 8) & 1 if self.n_instances > 0 else 0
+
+    def run(self):
+        self.front()
+        self.alloc_instances(self.read_instance_count())
+        self.back()
+        return self.image, self.depth
+
+
+def rasterize(
+    positions: torch.Tensor,
+    scales: torch.Tensor,
+    rotations: torch.Tensor,
+    opacities: torch.Tensor,
+    sh_0: torch.Tensor,
+    sh_rest: torch.Tensor,
+    settings: RasterizerSettings,
+    to_chw: bool,
+    use_median_depth: bool,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Inference render: ``(image, depth)`` with ``image`` ``[3,H,W]`` (``to_chw``) or ``[H,W,3]`` clamped to
+    [0,1] and ``depth`` ``[1,H,W]`` / ``[H,W,1]`` (reference: rasterization.py:140-163)."""
+    with torch.no_grad():
+        image, depth = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, settings,
+                                    to_chw, use_median_depth).run()
+    depth = depth.unsqueeze(0) if to_chw else depth.unsqueeze(-1)
+    return image, depth

@@ -1,0 +1,53 @@
+"""Helpers shared by the tests: oracle frames from synthetic scenes, GPU stage runner."""
+import numpy as np
+import torch
+
+import oracle
+from htgs_amd.synthetic import Scene
+from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode
+
+
+def oracle_frame(scene: Scene, mode: int, K=None, scale_modifier: float = 1.0, tile=None) -> oracle.Frame:
+    return oracle.Frame(scene.M.cpu().numpy(), scene.VPM.cpu().numpy(), scene.cam_position.cpu().numpy(), int(mode),
+                        scene.K if K is None else K, scene.active_sh_bases, scene.width, scene.height,
+                        scene.near_plane, scene.far_plane, scale_modifier, tile)
+
+
+def oracle_render(scene: Scene, mode: int, K=None, to_chw=True, median=False, scale_modifier=1.0) -> dict:
+    fr = oracle_frame(scene, mode, K, scale_modifier)
+    return oracle.render(fr, *[t.cpu().numpy() for t in scene.gaussians()], to_chw=to_chw, use_median_depth=median)
+
+
+def u32(t: torch.Tensor) -> np.ndarray:
+    """int32 / int16 / int64 tensor holding unsigned data -> unsigned numpy array"""
+    a = t.detach().cpu().numpy()
+    return a.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
+
+
+def gpu_stages(scene_gpu: Scene, mode: int, K=None, to_chw=True, median=False, scale_modifier=1.0) -> dict:
+    """Runs the frame stage by stage through the C ABI and returns every intermediate as numpy."""
+    settings = scene_gpu.settings(RasterizerMode(int(mode)), K, scale_modifier)
+    fb = FrameBuffers(*scene_gpu.gaussians(), settings, to_chw, median)
+    fb.n_touched.fill_(-1)
+    fb.bounds.zero_()
+    fb.prim.zero_()
+    fb.preprocess()
+    fb.scan()
+    n_inst = fb.read_instance_count()
+    fb.alloc_instances(n_inst)
+    fb.create_instances()
+    keys0 = u32(fb.keys[0])[:n_inst].astype(np.uint64)
+    vals0 = u32(fb.vals[0])[:n_inst].copy()
+    sel = fb.sort()
+    fb.extract_ranges()
+    fb.blend()
+    torch.cuda.synchronize()
+    prim = fb.prim.cpu().numpy()
+    return {
+        "fb": fb, "n_instances": n_inst,
+        "n_touched": u32(fb.n_touched), "offsets": u32(fb.offsets), "bounds": u32(fb.bounds).astype(np.uint32),
+        "VPMT1": prim[:, 0:4], "VPMT2": prim[:, 4:8], "VPMT4": prim[:, 8:12], "MT3": prim[:, 12:16], "rgba": prim[:, 16:20],
+        "keys": keys0, "vals": vals0,
+        "sorted_keys": u32(fb.keys[sel])[:n_inst].astype(np.uint64), "sorted_vals": u32(fb.vals[sel])[:n_inst].copy(),
+        "ranges": u32(fb.ranges), "image": fb.image.cpu().numpy(), "depth": fb.depth.cpu().numpy(),
+    }
