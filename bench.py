@@ -1,0 +1,164 @@
+#!/usr/bin/env python3
+"""Headline benchmark: frames per second of the inference rasterizer on one MI355X.
+
+One "step" is one full ``rasterize()`` call (preprocess -> scan -> host read of the instance count ->
+duplication -> radix sort -> ranges -> blend) on a seeded synthetic scene whose tensors are already resident
+in HBM.  Default workload: 3 M Gaussians, 1920x1080, HYBRID_BLEND K=16 (the configuration the metric is quoted
+on).  Prints ONE JSON line.
+
+The per-stage breakdown and the roofline figures are measured in the same process with HIP events on the
+stream the kernels are launched on (torch's current stream, which is the stream handed to the C ABI).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MODE_NAMES = {0: "HYBRID_BLEND", 1: "ALPHA_BLEND_FIRST_K", 2: "ALPHA_BLEND_GLOBAL_ORDERING", 3: "OIT_BLEND"}
+HBM_PEAK_GBS = 8000.0
+# fp32 vector peak as published (157.3 TFLOP/s counts packed FP32; plain FMA issue is half of it)
+FP32_PEAK_TFLOPS = 157.3
+# flops of the mandatory part of one pixel/instance evaluation (the two planes, m, d, |m|^2, |d|^2, cut-off test)
+FLOPS_PER_EVAL = 46
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2, help="scene: 1 = 1M/720p, 2 = 3M/1080p, 3 = 6M stress")
+    ap.add_argument("--n", type=int, default=None, help="override the number of Gaussians")
+    ap.add_argument("--mode", type=int, default=0)
+    ap.add_argument("--K", type=int, default=16)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def event_ms(fn, reps):
+    import torch
+    out = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        out.append(a.elapsed_time(b))
+    return out
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build renders one frame on one GPU; --gpus must be 1 "
+              "(sharding is described in DESIGN.md, not implemented)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from htgs_amd.synthetic import make_scene
+    from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode, rasterize
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    scene_cpu = make_scene(args.config, args.n)
+    scene = scene_cpu.to(dev)
+    mode = RasterizerMode(args.mode)
+    settings = scene.settings(mode, args.K)
+    gauss = scene.gaussians()
+
+    def step():
+        return rasterize(*gauss, settings, True, False)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-stage breakdown (HIP events on the launch stream), median over reps -------------------
+    reps = max(5, min(30, args.steps))
+    fb = FrameBuffers(*gauss, settings, True, False)
+    fb.front()
+    n_inst = fb.read_instance_count()
+    fb.alloc_instances(n_inst)
+    fb.back()
+    torch.cuda.synchronize()
+    n_vis = int((fb.n_touched != 0).sum().item())
+    N, P, T = fb.n, fb.width * fb.height, fb.n_tiles
+    B, kb = settings.active_sh_bases, fb.key_bytes
+    passes = (fb.end_bit + 7) // 8
+    stages = {}
+    for name, fn in (("preprocess", fb.preprocess), ("scan", fb.scan), ("create_instances", fb.create_instances),
+                     ("sort", fb.sort), ("extract_ranges", fb.extract_ranges), ("blend", fb.blend)):
+        for _ in range(3):
+            fn()
+        stages[name] = statistics.median(event_ms(fn, reps))
+    blend_all = event_ms(fb.blend, reps)
+    blend_avg_ms = sum(blend_all) / len(blend_all)
+    algo_bytes = {
+        "preprocess": N * (56 + 12 * (B - 1) * (B > 1)) + 4 * N + 88 * n_vis,   # 80 B record + 8 B bounds per visible Gaussian
+        "scan": 8 * N,
+        "create_instances": 16 * n_vis + (kb + 4) * n_inst,
+        "sort": passes * 2 * (kb + 4) * n_inst + passes * kb * n_inst,
+        "extract_ranges": kb * n_inst + 8 * T,
+        "blend": 84 * n_inst + 16 * P,
+    }
+    stage_report = {
+        k: {"ms": round(v, 4), "algo_GB": round(algo_bytes[k] / 1e9, 4),
+            "GBps": round(algo_bytes[k] / 1e9 / (v / 1e3), 1), "frac_hbm": round(algo_bytes[k] / 1e9 / (v / 1e3) / HBM_PEAK_GBS, 4)}
+        for k, v in stages.items()
+    }
+    tile_px = fb.tile * fb.tile
+    blend_flops = FLOPS_PER_EVAL * tile_px * n_inst
+    achieved_tflops = blend_flops / (blend_avg_ms / 1e3) / 1e12
+    roofline = {
+        "kernel": "blend", "bound": "valu_fp32", "achieved": round(achieved_tflops, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved_tflops / FP32_PEAK_TFLOPS, 4), "traffic": None,
+        "launch_ms": round(blend_avg_ms, 4), "evals_per_launch": tile_px * n_inst,
+    }
+
+    # ---- CPU baseline: the C oracle on this box's host cores, one whole frame of the same workload ----
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        import oracle
+        fr = oracle.Frame(scene_cpu.M.numpy(), scene_cpu.VPM.numpy(), scene_cpu.cam_position.numpy(), args.mode, args.K,
+                          scene_cpu.active_sh_bases, scene_cpu.width, scene_cpu.height, scene_cpu.near_plane, scene_cpu.far_plane)
+        arrays = [t.numpy() for t in scene_cpu.gaussians()]
+        t0 = time.perf_counter()
+        oracle.render(fr, *arrays)
+        cpu_s = time.perf_counter() - t0
+        cpu_baseline = {"value": round(1.0 / cpu_s, 4), "unit": "FPS", "cores": oracle.num_threads(), "kind": "port",
+                        "sample": f"one whole frame of the same workload, C oracle with OpenMP, {cpu_s:.2f} s"}
+
+    line = {
+        "metric": "FPS HYBRID_BLEND K=16 fwd @1080p, 3M Gaussians" if (args.config, args.mode, args.K) == (2, 0, 16)
+        else f"FPS {MODE_NAMES[args.mode]} K={args.K} fwd",
+        "value": round(1e3 / ms_per_step, 2), "unit": "FPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{scene.name} {MODE_NAMES[args.mode]} K={args.K} forward (rasterize), {N} Gaussians, "
+                               f"{scene.width}x{scene.height}, SH bases {B}",
+                   "n_gaussians": N, "n_visible": n_vis, "n_instances": n_inst, "n_tiles": T, "key_bytes": kb, "sort_passes": passes},
+        "stages": stage_report,
+        "stage_sum_ms": round(sum(stages.values()), 4),
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
