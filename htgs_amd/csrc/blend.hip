@@ -32,6 +32,10 @@ __device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restric
     }
 }
 
+// exchange two VGPRs in the active lanes (one instruction instead of a select pair)
+__device__ __forceinline__ void vswap(float &a, float &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void vswap(uint32_t &a, uint32_t &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+
 __device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__restrict__ depths, uint32_t w, uint32_t h,
                                             uint32_t x, uint32_t y, bool chw, float r, float g, float b, float depth)
 {
@@ -83,12 +87,11 @@ __global__ void __launch_bounds__(64) blend_hybrid_kernel(
 #pragma unroll
                     for (int i = 0; i < K; ++i) {
                         if (depth < cd[i]) {
-                            float t;
-                            t = depth; depth = cd[i]; cd[i] = t;
-                            t = p0; p0 = c0[i]; c0[i] = t;
-                            t = p1; p1 = c1[i]; c1[i] = t;
-                            t = p2; p2 = c2[i]; c2[i] = t;
-                            t = p3; p3 = c3[i]; c3[i] = t;
+                            vswap(depth, cd[i]);
+                            vswap(p0, c0[i]);
+                            vswap(p1, c1[i]);
+                            vswap(p2, c2[i]);
+                            vswap(p3, c3[i]);
                         }
                     }
                 }
