@@ -16,6 +16,7 @@ struct Stage {
     float4 v1[N], v2[N], v4[N], mt3[N], col[N];
 };
 
+// Stages one Gaussian record per lane.
 template <int N>
 __device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                            uint32_t fetch, uint32_t last, int slot, uint32_t *idx_out)
@@ -51,7 +52,7 @@ __device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__
 // else is merged order-independently into one tail fragment behind them.
 // ---------------------------------------------------------------------------------------------
 template <int K>
-__global__ void __launch_bounds__(64) blend_hybrid_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 4 : 2))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
 {
@@ -73,7 +74,8 @@ __global__ void __launch_bounds__(64) blend_hybrid_kernel(
         __syncthreads();
         stage_load(st, prim, inst, base + lane, last, lane, nullptr);
         __syncthreads();
-        if (inside) {
+        {
+            // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
             const int nb = last - base < 64u ? (int)(last - base) : 64;
             for (int j = 0; j < nb; ++j) {
                 Frag f;
