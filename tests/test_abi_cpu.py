@@ -1,0 +1,111 @@
+"""CPU-side checks of the boundary: the shared library loads without a GPU and exports every symbol that
+include/htgs_amd.h declares, the ctypes mirror of ``htgs_frame`` has the C layout, the pure helper functions
+agree with the reference's definitions, and the Python operator validates its arguments like the reference
+(RuntimeError on an unsupported mode, R/src/rasterization_api.cu:171-172)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+import oracle
+from htgs_amd import _native
+from htgs_amd.synthetic import make_scene
+from htgs_amd.torch_bindings import RasterizerMode, RasterizerSettings, rasterize
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "htgs_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(htgs_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) >= 15
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    for name in names:
+        assert hasattr(handle, name), f"{name} is declared in include/htgs_amd.h but not exported"
+    assert sorted(_native.SYMBOLS) == names, "htgs_amd/_native.py must bind exactly the declared entry points"
+    _native.lib()
+
+
+def test_frame_struct_layout_matches_the_header(tmp_path):
+    fields = [name for name, _ in _native.Frame._fields_]
+    src = tmp_path / "layout.c"
+    prints = "\n".join(f'    printf("{f} %zu\\n", offsetof(htgs_frame, {f}));' for f in fields)
+    src.write_text(f'#include <stdio.h>\n#include <stddef.h>\n#include "{HEADER}"\nint main(void) {{\n'
+                   f'    printf("sizeof %zu\\n", sizeof(htgs_frame));\n{prints}\n    return 0;\n}}\n')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-o", str(exe), str(src)], check=True)
+    out = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    assert int(out["sizeof"]) == ctypes.sizeof(_native.Frame)
+    for f in fields:
+        assert int(out[f]) == getattr(_native.Frame, f).offset, f
+
+
+def test_helper_functions():
+    lib = _native.lib()
+    assert [lib.htgs_tile_size(m) for m in range(4)] == [8, 8, 16, 8]
+    # K is rounded down to a power of two, at most 32 (R/src/hybrid_blend/inference.cu:22-27)
+    assert [lib.htgs_effective_k(k) for k in (0, 1, 2, 3, 4, 7, 8, 15, 16, 31, 32, 33, 1000)] == [1, 1, 2, 2, 4, 4, 8, 8, 16, 16, 32, 32, 32]
+    for (w, h) in [(256, 256), (1280, 720), (1920, 1080), (1600, 1066), (8, 8), (9, 8), (4096, 4096), (16, 16)]:
+        for mode in range(4):
+            tile = 16 if mode == 2 else 8
+            n_tiles = -(-w // tile) * -(-h // tile)
+            bits = (n_tiles - 1).bit_length()           # extract_end_bit, R/include/rasterization_utils.h:3-13
+            assert lib.htgs_end_bit(mode, w, h) == bits + (32 if mode == 2 else 0)
+            assert lib.htgs_key_bytes(mode, w, h) == (8 if mode == 2 else (2 if bits <= 16 else 4))
+            fr = oracle.Frame(None, None, None, mode, 16, 16, w, h, 0.2, 1000.0)
+            assert oracle.end_bit(fr) == lib.htgs_end_bit(mode, w, h)
+    assert lib.htgs_scan_tmp_words(0) >= 1 and lib.htgs_scan_tmp_words(3_000_000) >= 3_000_000 // 2048
+    assert lib.htgs_sort_tmp_words(0) >= 256 and lib.htgs_sort_tmp_words(20_000_000) >= 256 * (20_000_000 // 4096)
+
+
+def test_entry_points_reject_bad_frames_without_touching_the_gpu():
+    lib = _native.lib()
+    f = _native.Frame()
+    f.mode = 7
+    f.width = f.height = 64
+    for fn in (lib.htgs_preprocess, lib.htgs_create_instances):
+        assert fn(ctypes.byref(f)) == 1
+        assert b"unsupported rasterizer mode" in lib.htgs_last_error()
+    sel = ctypes.c_int(0)
+    assert lib.htgs_sort_instances(ctypes.byref(f), ctypes.byref(sel)) == 1
+    assert lib.htgs_blend(ctypes.byref(f), 0) == 1
+    f.mode = 0
+    f.n_primitives = 10            # but every pointer is null
+    assert lib.htgs_preprocess(ctypes.byref(f)) == 2
+    assert lib.htgs_preprocess(None) == 2
+    f.n_primitives = -1
+    assert lib.htgs_preprocess(ctypes.byref(f)) == 2
+
+
+def test_python_api_surface_and_validation():
+    import HTGSCudaBackend.torch_bindings as alias
+    import htgs_amd
+    for name in ("rasterize", "RasterizerSettings", "RasterizerMode"):
+        assert getattr(alias, name) is getattr(htgs_amd, name)
+    assert [m.value for m in RasterizerMode] == [0, 1, 2, 3]
+    assert RasterizerSettings._fields == ("M", "VPM", "cam_position", "mode", "K", "active_sh_bases", "width", "height",
+                                          "near_plane", "far_plane", "scale_modifier")
+    sc = make_scene(0, 10)
+    s = sc.settings(RasterizerMode.OIT_BLEND, 4)
+    assert s.as_tuple()[3:] == (3, 4, 1, 256, 256, 0.2, 1000.0, 1.0)
+    with pytest.raises(RuntimeError, match="GPU"):
+        rasterize(*sc.gaussians(), s, True, False)          # CPU tensors: there is no CPU path
+    bad = s._replace(mode=5)
+    with pytest.raises(RuntimeError, match="unsupported rasterizer mode"):
+        rasterize(*sc.gaussians(), bad, True, False)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _native.lib()

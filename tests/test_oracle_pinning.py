@@ -1,0 +1,382 @@
+"""Pins the CPU oracle (oracle/htgs_oracle.c).  The reference ships no tests, fixtures or golden outputs, so each
+part of the oracle is checked against what the mathematics fixes: library routines (scipy rotations and
+spherical harmonics, numpy cumsum / stable argsort / searchsorted), closed forms (on-axis sphere extent,
+near/far culling of a sphere, single-fragment compositing), brute force (dense sampling of the cut-off
+ellipsoid, tile overlap of the continuous box) and an independent float64 evaluator that uses the textbook
+ray/Gaussian maximum instead of the reference's plane construction (oracle/bruteforce.py)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+from scipy.spatial.transform import Rotation
+from scipy.special import sph_harm_y
+
+import oracle
+from oracle import bruteforce as bf
+from htgs_amd.synthetic import Scene, make_scene, pinhole
+from util import oracle_frame, oracle_render
+
+
+def ulp_diff(a: float, b: float) -> float:
+    return abs(a - b) / np.spacing(np.float32(abs(b)))
+
+
+# ---------------------------------------------------------------------------------------------------------
+# elementary functions of the rounding convention
+# ---------------------------------------------------------------------------------------------------------
+def test_logf_matches_libm():
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([np.exp(rng.uniform(-80, 80, 4000)), rng.uniform(0.5, 2.0, 4000), [1.0, 255.0, 20.0, 1e-40, 3e38]])
+    worst = 0.0
+    for x in xs.astype(np.float32):
+        got, want = oracle.logf(float(x)), math.log(float(x))
+        worst = max(worst, abs(got - want) / max(float(np.spacing(np.float32(abs(want)))), 1e-45) if want != 0 else abs(got))
+    assert worst <= 2.5, worst
+    assert oracle.logf(1.0) == 0.0
+    assert oracle.logf(0.0) == -math.inf and math.isnan(oracle.logf(-1.0)) and oracle.logf(math.inf) == math.inf
+
+
+def test_expf_matches_libm():
+    xs = np.linspace(-20.0, 0.0, 20001).astype(np.float32)
+    worst = max(ulp_diff(oracle.expf(float(x)), math.exp(float(x))) for x in xs)
+    assert worst <= 2.0, worst
+    assert oracle.expf(0.0) == 1.0
+
+
+# ---------------------------------------------------------------------------------------------------------
+# per-Gaussian stage
+# ---------------------------------------------------------------------------------------------------------
+def small_scene(n=150, seed=7, width=48, height=40, focal=60.0, sh_degree=3, z_range=(2.0, 6.0), scale=(0.05, 0.3),
+                rotation=None, translation=(0.1, -0.2, 0.3)) -> Scene:
+    g = torch.Generator().manual_seed(seed)
+    pos = torch.rand(n, 3, generator=g) * 2 - 1
+    pos[:, 0] *= 1.8
+    pos[:, 1] *= 1.5
+    pos[:, 2] = z_range[0] + (z_range[1] - z_range[0]) * torch.rand(n, generator=g)
+    scales = scale[0] + (scale[1] - scale[0]) * torch.rand(n, 3, generator=g)
+    q = torch.randn(n, 4, generator=g)
+    q = q / q.norm(dim=1, keepdim=True)
+    opac = 0.02 + 0.97 * torch.rand(n, 1, generator=g)
+    sh_0 = (torch.rand(n, 1, 3, generator=g) - 0.5) / 0.28209479177387814
+    n_rest = (sh_degree + 1) ** 2 - 1
+    sh_rest = torch.randn(n, n_rest, 3, generator=g) * 0.3 if n_rest else torch.zeros(n, 0, 3)
+    if rotation is None:
+        rotation = Rotation.from_euler("xyz", [4.0, -6.0, 10.0], degrees=True).as_matrix()
+    M, VPM, cam = pinhole(width, height, focal, focal * 1.1, width / 2 + 0.7, height / 2 - 1.3, 0.2, 1000.0, translation, rotation)
+    # move the Gaussians (generated in camera space) into world space
+    Rc, tc = M[:3, :3].double(), M[:3, 3].double()
+    pos = ((pos.double() - tc) @ Rc).float()
+    return Scene("small", pos.contiguous(), scales, q, opac, sh_0, sh_rest, M, VPM, cam, width, height, 0.2, 1000.0,
+                 (sh_degree + 1) ** 2, 4)
+
+
+def test_vpmt_rows_match_matrix_product_with_scipy_rotation():
+    sc = small_scene()
+    fr = oracle_frame(sc, 0, scale_modifier=1.3)
+    pre = oracle.preprocess(fr, *[t.numpy() for t in sc.gaussians()])
+    q = sc.rotations.double().numpy()
+    R = Rotation.from_quat(q[:, [1, 2, 3, 0]]).as_matrix()             # scipy is scalar-last
+    S = sc.scales.double().numpy() * 1.3
+    VPM = sc.VPM.double().numpy()
+    M = sc.M.double().numpy()
+    vis = pre["n_touched"] > 0
+    assert vis.sum() > 50
+    for i in np.nonzero(vis)[0]:
+        T = np.eye(4)
+        T[:3, :3] = R[i] * S[i][None, :]
+        T[:3, 3] = sc.positions[i].double().numpy()
+        full = VPM @ T
+        np.testing.assert_allclose(pre["VPMT1"][i], full[0], rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(pre["VPMT2"][i], full[1], rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(pre["VPMT4"][i], full[3], rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(pre["MT3"][i], (M @ T)[2], rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(R[i] @ R[i].T, np.eye(3), atol=1e-6)
+
+
+def continuous_box(sc: Scene, i: int, rho: float, n_samples=200_000, seed=0):
+    """Brute force: sample the surface of the ellipsoid (x-mu)^T S^-1 (x-mu) = rho densely, project with VPM."""
+    rng = np.random.default_rng(seed)
+    d = rng.normal(size=(n_samples, 3))
+    d /= np.linalg.norm(d, axis=1, keepdims=True)
+    q = sc.rotations[i].double().numpy()
+    R = Rotation.from_quat(q[[1, 2, 3, 0]]).as_matrix()
+    pts = sc.positions[i].double().numpy() + (d * sc.scales[i].double().numpy() * math.sqrt(rho)) @ R.T
+    h = np.c_[pts, np.ones(len(pts))] @ sc.VPM.double().numpy().T
+    xy = h[:, :2] / h[:, 3:4]
+    return xy.min(0), xy.max(0)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_screen_bounds_are_tight_and_conservative(mode):
+    """The tile rectangle must be exactly the set of tiles overlapped by the projected cut-off ellipsoid's box."""
+    sc = small_scene(n=60, width=160, height=128, focal=200.0, scale=(0.05, 0.25))
+    fr = oracle_frame(sc, mode)
+    pre = oracle.preprocess(fr, *[t.numpy() for t in sc.gaussians()])
+    tile = fr.tile_edge()
+    gw, gh = fr.grid()
+    checked = 0
+    for i in range(60):
+        opacity = float(sc.opacities[i])
+        rho = 2.0 * math.log(opacity / bf.MIN_ALPHA[mode])
+        if rho <= 0.05 or pre["n_touched"][i] == 0:
+            continue
+        lo, hi = continuous_box(sc, i, rho)
+        b = pre["bounds"][i].astype(int)
+        # sampled extremes are inside the true box by at most ~1e-3 px; a Gaussian whose box edge is that close
+        # to a tile edge is ambiguous and skipped
+        edges = np.array([lo[0] + 0.5, hi[0] + 0.5, lo[1] + 0.5, hi[1] + 0.5]) / tile
+        if np.abs(edges - np.round(edges)).min() < 2e-3:
+            continue
+        want = [min(gw, max(0, math.floor(edges[0]))), min(gw, max(0, math.ceil(edges[1]))),
+                min(gh, max(0, math.floor(edges[2]))), min(gh, max(0, math.ceil(edges[3])))]
+        assert list(b) == want, (i, list(b), want)
+        checked += 1
+    assert checked >= 25
+
+
+def test_on_axis_sphere_extent_closed_form():
+    """Isotropic Gaussian of scale s on the optical axis at depth z: the cut-off sphere of radius r = s sqrt(rho)
+    projects to the half-extent f r / sqrt(z^2 - r^2) about cx - 0.5."""
+    f, z, s, opacity = 500.0, 5.0, 0.2, 0.8
+    M, VPM, cam = pinhole(1024, 1024, f, f, 512.0, 512.0, 0.2, 1000.0)
+    rho = 2.0 * math.log(255.0 * opacity)
+    r = s * math.sqrt(rho)
+    half = f * r / math.sqrt(z * z - r * r)
+    centre = 512.0 - 0.5 + f * 0.0
+    # the perspective centre of the projected sphere is shifted: c = f * z * x / (z^2 - r^2) = 0 on the axis
+    sc = Scene("axis", torch.tensor([[0.0, 0.0, z]]), torch.full((1, 3), s), torch.tensor([[1.0, 0, 0, 0]]), torch.tensor([[opacity]]),
+               torch.zeros(1, 1, 3), torch.zeros(1, 0, 3), M, VPM, cam, 1024, 1024, 0.2, 1000.0, 1, 4)
+    pre = oracle.preprocess(oracle_frame(sc, 0), *[t.numpy() for t in sc.gaussians()])
+    want = [math.floor((centre - half + 0.5) / 8), math.ceil((centre + half + 0.5) / 8)] * 2
+    assert list(pre["bounds"][0]) == want
+
+
+def test_near_far_culling_closed_form():
+    """A sphere at depth z with cut-off radius r survives iff near <= z - r and z + r <= far."""
+    f, s, opacity = 300.0, 0.1, 0.9
+    r = s * math.sqrt(2.0 * math.log(255.0 * opacity))
+    M, VPM, cam = pinhole(256, 256, f, f, 128.0, 128.0, 1.0, 10.0)
+    zs = [0.5, 1.0 + 0.5 * r, 1.0 + 0.99 * r, 1.0 + 1.01 * r, 5.0, 10.0 - 1.01 * r, 10.0 - 0.99 * r, 10.5]
+    want = [False, False, False, True, True, True, False, False]
+    n = len(zs)
+    sc = Scene("nf", torch.tensor([[0.0, 0.0, z] for z in zs]), torch.full((n, 3), s), torch.tensor([[1.0, 0, 0, 0]] * n),
+               torch.full((n, 1), opacity), torch.zeros(n, 1, 3), torch.zeros(n, 0, 3), M, VPM, cam, 256, 256, 1.0, 10.0, 1, 4)
+    pre = oracle.preprocess(oracle_frame(sc, 0), *[t.numpy() for t in sc.gaussians()])
+    assert [bool(v) for v in pre["n_touched"] > 0] == want
+
+
+def test_degenerate_and_low_opacity_gaussians():
+    """A flat Gaussian (one scale 0) still gets a finite box; opacity below the threshold gives rho < 0, a
+    zero-extent box with at most one tile; opacity 0 is culled (R/include/kernel_utils.cuh:104-137)."""
+    M, VPM, cam = pinhole(256, 256, 300.0, 300.0, 128.0, 128.0, 0.2, 1000.0)
+    pos = torch.tensor([[0.1, 0.1, 4.0], [0.3, -0.2, 4.0], [0.0, 0.0, 4.0]])
+    scales = torch.tensor([[0.2, 0.1, 0.0], [0.1, 0.1, 0.1], [0.1, 0.1, 0.1]])
+    opac = torch.tensor([[0.9], [0.003], [0.0]])
+    sc = Scene("deg", pos, scales, torch.tensor([[1.0, 0, 0, 0]] * 3), opac, torch.zeros(3, 1, 3), torch.zeros(3, 0, 3), M, VPM, cam,
+               256, 256, 0.2, 1000.0, 1, 4)
+    pre = oracle.preprocess(oracle_frame(sc, 0), *[t.numpy() for t in sc.gaussians()])
+    assert pre["n_touched"][0] > 1 and np.isfinite(pre["VPMT1"][0]).all()
+    assert pre["n_touched"][1] <= 1
+    assert pre["n_touched"][2] == 0
+
+
+def real_sh_from_scipy(dirs: np.ndarray) -> np.ndarray:
+    """Real spherical harmonics from scipy's complex ones, in the sign convention of 3-D Gaussian splatting:
+    the textbook real basis with (x, y, z) -> (-x, -y, z) for odd m... expressed directly: the Cartesian
+    polynomial of each textbook real harmonic evaluated at the direction, with the (-1)^m phase removed."""
+    x, y, z = dirs.T
+    theta = np.arctan2(y, x)                 # azimuth
+    phi = np.arccos(np.clip(z, -1, 1))       # polar
+    out = []
+    for l in range(4):
+        for m in range(-l, l + 1):
+            Y = sph_harm_y(l, abs(m), phi, theta)
+            if m < 0:
+                v = math.sqrt(2) * (-1) ** m * Y.imag
+            elif m == 0:
+                v = Y.real
+            else:
+                v = math.sqrt(2) * (-1) ** m * Y.real
+            # 3DGS convention: odd-m harmonics carry an extra minus sign (Condon-Shortley phase kept)
+            out.append(v * ((-1) ** m))
+    return np.stack(out, axis=-1)
+
+
+def test_sh_basis_against_scipy_and_oracle_colours():
+    rng = np.random.default_rng(3)
+    d = rng.normal(size=(500, 3))
+    d /= np.linalg.norm(d, axis=1, keepdims=True)
+    np.testing.assert_allclose(bf.sh_basis(torch.tensor(d)).numpy(), real_sh_from_scipy(d), atol=1e-12)
+    for degree in (0, 1, 2, 3):
+        sc = small_scene(sh_degree=3)
+        sc.active_sh_bases = (degree + 1) ** 2
+        pre = oracle.preprocess(oracle_frame(sc, 0), *[t.numpy() for t in sc.gaussians()])
+        want = bf.sh_colour(sc.positions.double(), sc.sh_0.double(), sc.sh_rest.double(), sc.cam_position.double(), sc.active_sh_bases)
+        vis = pre["n_touched"] > 0
+        np.testing.assert_allclose(pre["rgba"][vis, :3], want.numpy()[vis], atol=3e-6)
+        np.testing.assert_array_equal(pre["rgba"][vis, 3], sc.opacities.numpy()[vis, 0])
+    # degree 0 only: rgb = max(0, 0.5 + 0.28209479 sh0)
+    sc = small_scene(sh_degree=0)
+    pre = oracle.preprocess(oracle_frame(sc, 0), *[t.numpy() for t in sc.gaussians()])
+    vis = pre["n_touched"] > 0
+    np.testing.assert_allclose(pre["rgba"][vis, :3], np.maximum(0, 0.5 + 0.28209479177387814 * sc.sh_0.numpy()[vis, 0]), atol=1e-6)
+
+
+def test_clamp_flags():
+    sc = small_scene(sh_degree=1)
+    sc.sh_0 = sc.sh_0 * 3.0      # push many channels below zero
+    pre = oracle.preprocess(oracle_frame(sc, 0), *[t.numpy() for t in sc.gaussians()], train=True)
+    want = bf.sh_colour(sc.positions.double(), sc.sh_0.double(), sc.sh_rest.double(), sc.cam_position.double(), 4)
+    vis = pre["n_touched"] > 0
+    unclamped_negative = (pre["rgba"][vis, :3] == 0) & (want.numpy()[vis] == 0)
+    np.testing.assert_array_equal(pre["clamp_info"].T[vis].astype(bool), unclamped_negative)
+    assert unclamped_negative.any() and not unclamped_negative.all()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# scan, duplication, sort, ranges
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("mode", [0, 2])
+def test_integer_stages_against_numpy(mode):
+    sc = make_scene(1, 20_000)
+    fr = oracle_frame(sc, mode)
+    out = oracle.render(fr, *[t.numpy() for t in sc.gaussians()])
+    nt, b = out["pre"]["n_touched"], out["pre"]["bounds"].astype(np.int64)
+    np.testing.assert_array_equal(out["offsets"], np.cumsum(nt, dtype=np.uint64).astype(np.uint32))
+    np.testing.assert_array_equal(nt, ((b[:, 1] - b[:, 0]) * (b[:, 3] - b[:, 2])).astype(np.uint32) * (nt > 0))
+    # duplication: python loops, row-major tiles, ascending primitive index
+    gw, gh = fr.grid()
+    keys, vals = [], []
+    for i in np.nonzero(nt)[0][:3000]:
+        z = int(out["pre"]["MT3"][i, 3:4].view(np.uint32)[0])
+        for y in range(b[i, 2], b[i, 3]):
+            for x in range(b[i, 0], b[i, 1]):
+                t = y * gw + x
+                keys.append((t << 32) | z if mode == 2 else t)
+                vals.append(i)
+    np.testing.assert_array_equal(out["keys"][:len(keys)], np.array(keys, dtype=np.uint64))
+    np.testing.assert_array_equal(out["vals"][:len(vals)], np.array(vals, dtype=np.uint32))
+    # sort: stable ascending
+    order = np.argsort(out["keys"], kind="stable")
+    np.testing.assert_array_equal(out["sorted_keys"], out["keys"][order])
+    np.testing.assert_array_equal(out["sorted_vals"], out["vals"][order])
+    # ranges: searchsorted on the tile ids; untouched tiles are (0, 0)
+    tiles = out["sorted_keys"] >> np.uint64(32 if mode == 2 else 0)
+    first = np.searchsorted(tiles, np.arange(gw * gh), side="left")
+    last = np.searchsorted(tiles, np.arange(gw * gh), side="right")
+    touched = last > first
+    np.testing.assert_array_equal(out["ranges"][touched, 0], first[touched])
+    np.testing.assert_array_equal(out["ranges"][touched, 1], last[touched])
+    assert (out["ranges"][~touched] == 0).all()
+    assert int((last - first).sum()) == len(tiles) == int(nt.sum())
+
+
+def test_sort_respects_end_bit():
+    """Only the low end_bit bits take part in the comparison (cub::DeviceRadixSort semantics)."""
+    rng = np.random.default_rng(5)
+    keys = rng.integers(0, 1 << 40, size=5000, dtype=np.uint64)
+    vals = np.arange(5000, dtype=np.uint32)
+    for bits in (1, 7, 16, 17, 33, 40):
+        k, v = oracle.sort_pairs(keys, vals, bits)
+        order = np.argsort(keys & np.uint64((1 << bits) - 1), kind="stable")
+        np.testing.assert_array_equal(v, vals[order])
+        np.testing.assert_array_equal(k, keys[order])
+
+
+def test_empty_and_all_culled_scenes():
+    sc = small_scene(n=5)
+    sc.positions = sc.positions * 0 + torch.tensor([0.0, 0.0, -50.0])     # behind the camera
+    out = oracle_render(sc, 0, 4)
+    assert out["pre"]["n_touched"].sum() == 0 and len(out["keys"]) == 0
+    assert (out["ranges"] == 0).all() and (out["image"] == 0).all() and (out["depth"] == 0).all()
+
+
+# ---------------------------------------------------------------------------------------------------------
+# per-pixel stage against the independent float64 evaluator
+# ---------------------------------------------------------------------------------------------------------
+def brute(sc: Scene, mode: int, K: int, median=False, scale_modifier=1.0):
+    fr = bf.evaluate(*[t for t in sc.gaussians()], sc.M, sc.VPM, sc.cam_position, mode, sc.active_sh_bases,
+                     sc.width, sc.height, sc.near_plane, sc.far_plane, scale_modifier)
+    return bf.render(fr, mode, K, median)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("K,median", [(1, False), (4, False), (4, True), (16, False), (32, False)])
+def test_render_matches_float64_brute_force(mode, K, median):
+    if mode == 3 and median:
+        pytest.skip("OIT_BLEND has no median depth (R/src/oit_blend/inference.cu:37)")
+    sc = small_scene(n=160, seed=11 + mode)
+    ref = oracle_render(sc, mode, K, median=median)
+    img, dep, alpha, margin = brute(sc, mode, K, median)
+    ok = (margin > 1e-4).numpy()
+    assert ok.mean() > 0.97
+    assert (ref["image"].max(0) > 0.05).mean() > 0.5, "scene too empty to mean anything"
+    err_i = np.abs(ref["image"] - img.numpy())[:, ok].max()
+    err_d = np.abs(ref["depth"] - dep.numpy())[ok].max()
+    assert err_i < 2e-5, err_i
+    assert err_d < 2e-4, err_d          # depths are ~5 units: 2e-4 is ~40 float32 ulps of accumulated rounding
+    if not median:
+        assert np.abs(ref["alpha"] - alpha.numpy())[ok].max() < 2e-5
+
+
+def test_scale_modifier_and_off_axis_camera():
+    sc = small_scene(n=120, seed=3, rotation=Rotation.from_euler("xyz", [20.0, -30.0, 45.0], degrees=True).as_matrix())
+    ref = oracle_render(sc, 0, 8, scale_modifier=0.7)
+    img, dep, alpha, margin = brute(sc, 0, 8, scale_modifier=0.7)
+    ok = (margin > 1e-4).numpy()
+    assert np.abs(ref["image"] - img.numpy())[:, ok].max() < 2e-5
+
+
+def test_single_fragment_closed_forms():
+    """One Gaussian, K >= 1: every mode gives rgb = alpha * c, depth = depth of the fragment, where alpha and depth
+    follow the textbook ray maximum."""
+    M, VPM, cam = pinhole(32, 32, 40.0, 40.0, 16.0, 16.0, 0.2, 1000.0)
+    sc = Scene("one", torch.tensor([[0.05, -0.03, 3.0]]), torch.tensor([[0.3, 0.2, 0.25]]), torch.tensor([[0.9, 0.1, 0.3, -0.2]]) / 1.0,
+               torch.tensor([[0.7]]), torch.tensor([[[1.0, 0.2, -0.5]]]), torch.zeros(1, 0, 3), M, VPM, cam, 32, 32, 0.2, 1000.0, 1, 4)
+    sc.rotations = sc.rotations / sc.rotations.norm()
+    fr = bf.evaluate(*sc.gaussians(), sc.M, sc.VPM, sc.cam_position, 0, 1, 32, 32, 0.2, 1000.0)
+    a, d = fr.alpha.reshape(32, 32).numpy(), fr.depth.reshape(32, 32).numpy()
+    c = fr.rgb[0].numpy()
+    for mode in range(4):
+        ref = oracle_render(sc, mode, 4)
+        thr = bf.MIN_ALPHA[mode]
+        inside = a > thr * 1.001
+        outside = a < thr * 0.999
+        assert inside.sum() > 50
+        np.testing.assert_allclose(ref["image"][:, inside], (c[:, None] * a[inside][None, :]), atol=2e-6)
+        assert (ref["image"][:, outside] == 0).all()
+        want_depth = float(fr.z_centre[0]) if mode == 2 else d[inside]
+        np.testing.assert_allclose(ref["depth"][inside], want_depth, rtol=2e-5)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 3])
+def test_image_does_not_depend_on_tile_size(mode):
+    """Per-pixel fragment order is primitive-index order whatever the tiling, so 8x8 and 16x16 tiles must give the
+    very same image, bit for bit; per-tile counts of course differ."""
+    sc = make_scene(0, 3000)
+    arrays = [t.numpy() for t in sc.gaussians()]
+    a = oracle.render(oracle_frame(sc, mode, 4, tile=8), *arrays)
+    b = oracle.render(oracle_frame(sc, mode, 4, tile=16), *arrays)
+    np.testing.assert_array_equal(a["image"], b["image"])
+    np.testing.assert_array_equal(a["depth"], b["depth"])
+    assert len(a["keys"]) != len(b["keys"])
+
+
+def test_hybrid_with_large_k_equals_sorted_alpha_blending_of_core_plus_tail():
+    """K >= number of fragments and every alpha >= 1/20: HYBRID_BLEND = FIRST_K with the hybrid thresholds = exact
+    depth-sorted alpha blending (empty tail)."""
+    sc = small_scene(n=20, seed=5, scale=(0.1, 0.3))
+    sc.opacities = sc.opacities * 0 + 0.9
+    hyb = oracle_render(sc, 0, 32)
+    img, dep, alpha, margin = brute(sc, 0, 32)
+    fr = bf.evaluate(*sc.gaussians(), sc.M, sc.VPM, sc.cam_position, 0, sc.active_sh_bases, sc.width, sc.height, 0.2, 1000.0)
+    # pixels where no fragment sits between 1/255 and 1/20 have an empty tail
+    clean = (~((fr.alpha >= 1 / 255) & (fr.alpha < 1 / 20)).any(1)).reshape(sc.height, sc.width).numpy() & (margin > 1e-4).numpy()
+    assert clean.sum() > 200
+    order = torch.argsort(torch.where(fr.alpha >= 1 / 20, fr.depth, torch.full_like(fr.depth, 1e300)), dim=1)
+    a = torch.gather(fr.alpha * (fr.alpha >= 1 / 20), 1, order)
+    T = torch.cumprod(torch.cat([torch.ones_like(a[:, :1]), 1 - a[:, :-1]], 1), 1)
+    w = T * a * (T >= 1e-4)
+    want = (w[..., None] * fr.rgb[order]).sum(1).clamp(0, 1).T.reshape(3, sc.height, sc.width).numpy()
+    assert np.abs(hyb["image"] - want)[:, clean].max() < 2e-5
