@@ -225,3 +225,69 @@ def render(frame: Frame, positions, scales, rotations, opacities, sh_0, sh_rest,
         "pre": pre, "offsets": offsets, "keys": keys, "vals": vals, "sorted_keys": skeys, "sorted_vals": svals,
         "ranges": ranges, "image": image, "depth": depth, "alpha": alpha,
     }
+
+
+# ---------------------------------------------------------------------------------------------------------
+# training: forward with per-pixel records, backward
+# ---------------------------------------------------------------------------------------------------------
+def effective_k(K: int) -> int:
+    return 32 if K >= 32 else 16 if K >= 16 else 8 if K >= 8 else 4 if K >= 4 else 2 if K >= 2 else 1
+
+
+def forward(frame: Frame, positions, scales, rotations, opacities, sh_0, sh_rest) -> dict:
+    """``_C.forward`` of the reference (R/src/rasterization_api.cu:37-176): scale_modifier is ignored (the
+    training preprocess always uses 1, R/include/hybrid_blend/kernels/forward.cuh:10-76), the image is [3,H,W]
+    and not clamped, and the per-pixel records needed by backward are returned."""
+    import dataclasses
+    frame = dataclasses.replace(frame, scale_modifier=1.0)
+    pre = preprocess(frame, positions, scales, rotations, opacities, sh_0, sh_rest, train=True)
+    offsets = inclusive_scan(pre["n_touched"])
+    keys, vals = create_instances(frame, pre, offsets)
+    skeys, svals = sort_pairs(keys, vals, end_bit(frame))
+    ranges = extract_ranges(frame, skeys)
+    h, w = frame.height, frame.width
+    K = effective_k(frame.K)
+    image = np.zeros((3, h, w), np.float32)
+    core_idx = np.full((K, h * w), 0xFFFFFFFF, np.uint32)
+    core_info = np.zeros((K, h * w, 4), np.float32)
+    tail_info = np.zeros((6, h * w), np.float32)
+    cam = frame.c_struct(0)
+    lib().oracle_blend_forward(ctypes.byref(cam), _p(ranges), _p(svals), _p(pre["VPMT1"]), _p(pre["VPMT2"]), _p(pre["VPMT4"]),
+                               _p(pre["MT3"]), _p(pre["rgba"]), _p(image), _p(core_idx), _p(core_info), _p(tail_info))
+    return {"frame": frame, "pre": pre, "offsets": offsets, "sorted_keys": skeys, "sorted_vals": svals, "ranges": ranges,
+            "image": image, "core_idx": core_idx, "core_info": core_info, "tail_info": tail_info}
+
+
+def backward(fwd: dict, grad_image, positions, scales, rotations, opacities, sh_0, sh_rest,
+             densification_info: Optional[np.ndarray] = None, use_distance_scaling: bool = False) -> dict:
+    """``_C.backward`` of the reference (R/src/rasterization_api.cu:178-363): gradients w.r.t. positions, scales,
+    rotations (no normalisation term), opacities, sh_0, sh_rest; ``densification_info`` ([2,N] or [3,N]) is updated
+    in place."""
+    frame: Frame = fwd["frame"]
+    positions, scales, rotations = _f32(positions), _f32(scales), _f32(rotations)
+    sh_rest = _f32(sh_rest)
+    grad_image = _f32(grad_image)
+    n = positions.shape[0]
+    total_sh = sh_rest.shape[1]
+    pre = fwd["pre"]
+    g_pos = np.zeros((n, 3), np.float32)
+    g_scale = np.zeros((n, 3), np.float32)
+    g_rot = np.zeros((n, 4), np.float32)
+    g_op = np.zeros((n, 1), np.float32)
+    g_sh0 = np.zeros((n, 1, 3), np.float32)
+    g_rest = np.zeros((n, total_sh, 3), np.float32)
+    vpmt_mode = frame.mode in (MODE_HYBRID, MODE_OIT)
+    g_vpmt = np.zeros((9, n), np.float32) if vpmt_mode else None
+    helper = np.zeros(n, np.float32) if densification_info is not None and densification_info.shape[0] == 3 else None
+    cam = frame.c_struct(total_sh)
+    lib().oracle_blend_backward(
+        ctypes.byref(cam), ctypes.c_int(n), _p(fwd["ranges"]), _p(fwd["sorted_vals"]), _p(pre["VPMT1"]), _p(pre["VPMT2"]),
+        _p(pre["VPMT4"]), _p(pre["rgba"]), _p(scales), _p(rotations), _p(fwd["image"]), _p(fwd["core_idx"]), _p(fwd["core_info"]),
+        _p(fwd["tail_info"]), _p(grad_image), _p(g_pos), _p(g_scale), _p(g_rot), _p(g_op), _p(g_sh0), _p(g_vpmt), _p(helper))
+    grad_rgb = g_sh0.reshape(n, 3).copy()
+    lib().oracle_preprocess_backward(
+        ctypes.byref(cam), ctypes.c_int(n), _p(positions), _p(scales), _p(rotations), _p(sh_rest), _p(pre["n_touched"]),
+        _p(pre["clamp_info"]), _p(g_vpmt), _p(helper), _p(g_pos), _p(g_scale), _p(g_rot), _p(g_sh0), _p(g_rest),
+        _p(densification_info), ctypes.c_int(bool(use_distance_scaling)))
+    return {"positions": g_pos, "scales": g_scale, "rotations": g_rot, "opacities": g_op, "sh_0": g_sh0, "sh_rest": g_rest,
+            "grad_rgb": grad_rgb, "grad_VPMT": g_vpmt}

@@ -93,9 +93,10 @@ def evaluate(positions, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam
 
     R = quat_to_rot(rotations)
     s = scales * scale_modifier
-    # S^-1 = R diag(1/s^2) R^T
-    Sinv = R @ torch.diag_embed(1.0 / (s * s)) @ R.transpose(-1, -2)          # [G,3,3]
-    Sigma = R @ torch.diag_embed(s * s) @ R.transpose(-1, -2)
+    # S = (R diag(s)) (R diag(s))^T.  Inverted numerically rather than as R diag(1/s^2) R^T so that derivatives
+    # with respect to the quaternion are those of the matrix formula even off the unit sphere.
+    Sigma = R @ torch.diag_embed(s * s) @ R.transpose(-1, -2)                 # [G,3,3]
+    Sinv = torch.linalg.inv(Sigma)
     delta = positions - origin                                                # [G,3]
     Sd = torch.einsum("gij,gj->gi", Sinv, delta)                              # S^-1 (mu - o)
     rSr = torch.einsum("pi,gij,pj->pg", dir_w, Sinv, dir_w)

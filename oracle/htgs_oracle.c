@@ -652,3 +652,567 @@ O_EXPORT void oracle_blend(
             }
     }
 }
+
+/* ========================================================================= */
+/* training: forward with per-pixel records, backward                        */
+/* ========================================================================= */
+
+/* Per-pixel records written by the training forward pass (PerPixelBuffers,
+ * R/include/hybrid_blend/buffer_utils.h:96-108 and siblings), all pixel-minor:
+ *   core_idx  [K][P]     primitive of each blended core slot, UINT32_MAX = empty or skipped
+ *   core_info [K][P][4]  (dC/dalpha of the slot, blending weight)
+ *   tail_info [6][P]     hybrid: sum alpha*rgb of the tail (3), 1/sum alpha, T_tail, T_core
+ *                        oit:    sum alpha*rgb (3), 1/sum alpha, T  (5 rows)
+ * The reference leaves tail_info unwritten where the alpha sum is below 1/255 and then reads it in
+ * backward (forward.cuh:193-204 vs backward.cuh:158-173); here such records are zero. */
+
+/* blend_cu (forward) of HYBRID_BLEND, R/include/hybrid_blend/kernels/forward.cuh:108-233 */
+static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, size_t pix, size_t np,
+                                 float rgb_out[3], uint32_t *core_idx_out, float *core_info_out, float *tail_info_out)
+{
+    const float fx = (float)x, fy = (float)y;
+    const float cutoff = mode_cutoff_sq(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
+    float T_tail = 1.0f, tail[4] = { 0, 0, 0, 0 };
+    float core[KMAX][4], core_depth[KMAX];
+    uint32_t core_idx[KMAX];
+    for (int i = 0; i < K; ++i) { core[i][0] = core[i][1] = core[i][2] = core[i][3] = 0.0f; core_depth[i] = FLT_MAX; core_idx[i] = UINT32_MAX; }
+    fragment f;
+    for (uint32_t j = first; j < last; ++j) {
+        const size_t g = in->inst[j];
+        const float *col = in->rgba + 4 * g;
+        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
+                           fx, fy, cutoff, min_alpha, 1, NULL, &f)) continue;
+        float depth = f.depth;
+        float c[4] = { col[0], col[1], col[2], f.alpha };                                      /* :160 */
+        if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {
+            uint32_t idx = (uint32_t)g;
+            for (int i = 0; i < K; ++i) {
+                if (depth < core_depth[i]) {
+                    float t = depth; depth = core_depth[i]; core_depth[i] = t;
+                    for (int k = 0; k < 4; ++k) { t = c[k]; c[k] = core[i][k]; core[i][k] = t; }
+                    uint32_t ti = idx; idx = core_idx[i]; core_idx[i] = ti;
+                }
+            }
+        }
+        tail[0] += c[0] * c[3]; tail[1] += c[1] * c[3]; tail[2] += c[2] * c[3]; tail[3] += c[3];   /* :173 */
+        T_tail *= 1.0f - c[3];
+    }
+    float rgb[3] = { 0, 0, 0 }, T_core = 1.0f;
+    for (int i = 0; i < K && T_core >= TRANSMITTANCE_THRESHOLD; ++i) {                         /* :184-190 */
+        const float bw = T_core * core[i][3];
+        for (int k = 0; k < 3; ++k) rgb[k] = fmaf(bw, core[i][k], rgb[k]);
+        T_core *= 1.0f - core[i][3];
+        if (T_core < TRANSMITTANCE_THRESHOLD) T_core = 0.0f;
+    }
+    float wtail[3] = { 0, 0, 0 };
+    float ti[6] = { 0, 0, 0, 0, 0, 0 };
+    if (tail[3] >= min_alpha) {                                                                /* :193 */
+        const float asr = 1.0f / tail[3];
+        const float s = (T_core * (1.0f - T_tail)) * asr;
+        for (int k = 0; k < 3; ++k) wtail[k] = s * tail[k];
+        ti[0] = tail[0]; ti[1] = tail[1]; ti[2] = tail[2]; ti[3] = asr; ti[4] = T_tail; ti[5] = T_core;
+    }
+    for (int r = 0; r < 6; ++r) tail_info_out[r * np + pix] = ti[r];
+    float rgb_new[3] = { 0, 0, 0 };
+    T_core = 1.0f;
+    for (int i = 0; i < K; ++i) {                                                              /* :209-227 */
+        const int skip = core_idx[i] == UINT32_MAX || T_core < TRANSMITTANCE_THRESHOLD;
+        core_idx_out[i * np + pix] = skip ? UINT32_MAX : core_idx[i];
+        float *info = core_info_out + 4 * (i * np + pix);
+        if (skip) { info[0] = info[1] = info[2] = info[3] = 0.0f; continue; }
+        const float bw = T_core * core[i][3];
+        for (int k = 0; k < 3; ++k) rgb_new[k] = fmaf(bw, core[i][k], rgb_new[k]);
+        const float oma = 1.0f - core[i][3];
+        const float omar = 1.0f / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS);
+        for (int k = 0; k < 3; ++k) {
+            const float behind = ((rgb[k] - rgb_new[k]) + wtail[k]) * omar;
+            info[k] = fmaf(core[i][k], T_core, -behind);
+        }
+        info[3] = bw;
+        T_core *= oma;
+    }
+    for (int k = 0; k < 3; ++k) rgb_out[k] = rgb[k] + wtail[k];                                /* :229 */
+}
+
+/* blend_cu (forward) of ALPHA_BLEND_FIRST_K, R/include/alpha_blend_first_k/kernels/forward.cuh:108-213 */
+static void first_k_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, size_t pix, size_t np,
+                                  float rgb_out[3], uint32_t *core_idx_out, float *core_info_out)
+{
+    const float fx = (float)x, fy = (float)y;
+    const float cutoff = mode_cutoff_sq(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
+    float core_alpha[KMAX], core_depth[KMAX];
+    uint32_t core_idx[KMAX];
+    for (int i = 0; i < K; ++i) { core_alpha[i] = 0.0f; core_depth[i] = FLT_MAX; core_idx[i] = UINT32_MAX; }
+    fragment f;
+    for (uint32_t j = first; j < last; ++j) {
+        const size_t g = in->inst[j];
+        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
+                           fx, fy, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
+        float depth = f.depth, alpha = f.alpha;
+        uint32_t idx = (uint32_t)g;
+        for (int i = 0; i < K; ++i) {
+            if (depth < core_depth[i]) {
+                float t = depth; depth = core_depth[i]; core_depth[i] = t;
+                t = alpha; alpha = core_alpha[i]; core_alpha[i] = t;
+                uint32_t ti = idx; idx = core_idx[i]; core_idx[i] = ti;
+            }
+        }
+    }
+    float rgb[3] = { 0, 0, 0 }, T = 1.0f;
+    float cols[KMAX][3];
+    for (int i = 0; i < K && T >= TRANSMITTANCE_THRESHOLD; ++i) {                              /* :175-186 */
+        if (core_idx[i] == UINT32_MAX) break;
+        const float bw = T * core_alpha[i];
+        const float *col = in->rgba + 4 * (size_t)core_idx[i];
+        for (int k = 0; k < 3; ++k) { cols[i][k] = col[k]; rgb[k] = fmaf(bw, col[k], rgb[k]); }
+        T *= 1.0f - core_alpha[i];
+    }
+    float rgb_new[3] = { 0, 0, 0 };
+    T = 1.0f;
+    for (int i = 0; i < K; ++i) {                                                              /* :189-209 */
+        const int skip = core_idx[i] == UINT32_MAX || T < TRANSMITTANCE_THRESHOLD;
+        core_idx_out[i * np + pix] = skip ? UINT32_MAX : core_idx[i];
+        float *info = core_info_out + 4 * (i * np + pix);
+        if (skip) { info[0] = info[1] = info[2] = info[3] = 0.0f; continue; }
+        const float bw = T * core_alpha[i];
+        for (int k = 0; k < 3; ++k) rgb_new[k] = fmaf(bw, cols[i][k], rgb_new[k]);
+        const float oma = 1.0f - core_alpha[i];
+        const float omar = 1.0f / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS);
+        for (int k = 0; k < 3; ++k) info[k] = fmaf(cols[i][k], T, -((rgb[k] - rgb_new[k]) * omar));
+        info[3] = bw;
+        T *= oma;
+    }
+    for (int k = 0; k < 3; ++k) rgb_out[k] = rgb[k];
+}
+
+/* blend_cu (forward) of ALPHA_BLEND_GLOBAL_ORDERING, R/include/alpha_blend_global_ordering/kernels/forward.cuh:103-153 */
+static void global_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, float rgb_out[3])
+{
+    const float fx = (float)x, fy = (float)y;
+    const float cutoff = mode_cutoff_sq(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
+    float rgb[3] = { 0, 0, 0 }, T = 1.0f;
+    fragment f;
+    for (uint32_t j = first; j < last; ++j) {
+        const size_t g = in->inst[j];
+        const float *col = in->rgba + 4 * g;
+        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
+                           fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+        const float bw = T * f.alpha;
+        for (int k = 0; k < 3; ++k) rgb[k] = fmaf(bw, col[k], rgb[k]);
+        T *= 1.0f - f.alpha;
+        if (T < TRANSMITTANCE_THRESHOLD) break;
+    }
+    for (int k = 0; k < 3; ++k) rgb_out[k] = rgb[k];
+}
+
+/* blend_cu (forward) of OIT_BLEND, R/include/oit_blend/kernels/forward.cuh:101-162 */
+static void oit_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, size_t pix, size_t np,
+                              float rgb_out[3], float *tail_info_out)
+{
+    const float fx = (float)x, fy = (float)y;
+    const float cutoff = mode_cutoff_sq(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
+    float acc[3] = { 0, 0, 0 }, alpha_sum = 0.0f, T = 1.0f;
+    fragment f;
+    for (uint32_t j = first; j < last; ++j) {
+        const size_t g = in->inst[j];
+        const float *col = in->rgba + 4 * g;
+        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
+                           fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+        for (int k = 0; k < 3; ++k) acc[k] = fmaf(f.alpha, col[k], acc[k]);
+        alpha_sum += f.alpha;
+        T *= 1.0f - f.alpha;
+    }
+    float ti[5] = { 0, 0, 0, 0, 0 };
+    rgb_out[0] = rgb_out[1] = rgb_out[2] = 0.0f;
+    if (alpha_sum >= min_alpha) {                                                              /* :147 */
+        const float asr = 1.0f / alpha_sum;
+        const float s = (1.0f - T) * asr;
+        for (int k = 0; k < 3; ++k) rgb_out[k] = s * acc[k];
+        ti[0] = acc[0]; ti[1] = acc[1]; ti[2] = acc[2]; ti[3] = asr; ti[4] = T;
+    }
+    for (int r = 0; r < 5; ++r) tail_info_out[r * np + pix] = ti[r];
+}
+
+/* forward blend of the frame's mode: image is [3][H][W], not clamped (forward.cuh:231-233) */
+O_EXPORT void oracle_blend_forward(
+    const oracle_cam *c, const uint32_t *ranges, const uint32_t *inst,
+    const float *VPMT1, const float *VPMT2, const float *VPMT4, const float *MT3, const float *rgba,
+    float *image, uint32_t *core_idx, float *core_info, float *tail_info)
+{
+    const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
+    const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
+    const blend_in in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba };
+    const int K = round_k(c->K);
+    const size_t np = (size_t)c->width * c->height;
+    #pragma omp parallel for schedule(dynamic, 4)
+    for (int t = 0; t < grid_w * grid_h; ++t) {
+        const int tx = t % grid_w, ty = t / grid_w;
+        const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        for (int ly = 0; ly < c->tile_h; ++ly)
+            for (int lx = 0; lx < c->tile_w; ++lx) {
+                const int x = tx * c->tile_w + lx, y = ty * c->tile_h + ly;
+                if (x >= c->width || y >= c->height) continue;
+                const size_t pix = (size_t)c->width * y + x;
+                float rgb[3];
+                switch (c->mode) {
+                    case MODE_HYBRID: hybrid_pixel_forward(&in, first, last, x, y, K, pix, np, rgb, core_idx, core_info, tail_info); break;
+                    case MODE_FIRST_K: first_k_pixel_forward(&in, first, last, x, y, K, pix, np, rgb, core_idx, core_info); break;
+                    case MODE_GLOBAL: global_pixel_forward(&in, first, last, x, y, rgb); break;
+                    default: oit_pixel_forward(&in, first, last, x, y, pix, np, rgb, tail_info); break;
+                }
+                image[pix] = rgb[0]; image[np + pix] = rgb[1]; image[2 * np + pix] = rgb[2];
+            }
+    }
+}
+
+/* dL/dalpha of one fragment -> dL/dopacity and the gradients of the three VPMT rows.
+ * R/include/hybrid_blend/kernels/backward.cuh:260-289 (identical in the other modes). */
+typedef struct { float opacity; float dV1[4], dV2[4], dV4[4]; } frag_grads;
+
+static void fragment_backward(const fragment *f, float opacity, float dL_dalpha, float fx, float fy, frag_grads *o)
+{
+    const float *px = f->px, *py = f->py, *m = f->m, *d = f->d;
+    o->opacity = dL_dalpha * f->G;
+    const float dL_dG = dL_dalpha * opacity;
+    const float dL_drho2 = dL_dG * -0.5f * f->G;
+    const float dL_dnum = dL_drho2 * f->den_rcp;
+    const float dL_dden = dL_drho2 * -f->num * f->den_rcp * f->den_rcp;
+    float dm[3], dd[3];
+    for (int k = 0; k < 3; ++k) { dm[k] = dL_dnum * 2.0f * m[k]; dd[k] = dL_dden * 2.0f * d[k]; }
+    float dpx[4], dpy[4];
+    dpx[0] = -py[3] * dm[0] - py[2] * dd[1] + py[1] * dd[2];
+    dpx[1] = -py[3] * dm[1] + py[2] * dd[0] - py[0] * dd[2];
+    dpx[2] = -py[3] * dm[2] - py[1] * dd[0] + py[0] * dd[1];
+    dpx[3] = py[0] * dm[0] + py[1] * dm[1] + py[2] * dm[2];
+    dpy[0] = px[3] * dm[0] + px[2] * dd[1] - px[1] * dd[2];
+    dpy[1] = px[3] * dm[1] - px[2] * dd[0] + px[0] * dd[2];
+    dpy[2] = px[3] * dm[2] + px[1] * dd[0] - px[0] * dd[1];
+    dpy[3] = -(px[0] * dm[0] + px[1] * dm[1] + px[2] * dm[2]);
+    for (int k = 0; k < 4; ++k) {
+        o->dV1[k] = dpx[k];
+        o->dV2[k] = dpy[k];
+        o->dV4[k] = -fx * dpx[k] - fy * dpy[k];
+    }
+}
+
+/* recomputes G and alpha of a fragment exactly as the forward pass did; 0 if it was rejected */
+static inline int reeval_fragment(const blend_in *in, size_t g, float fx, float fy, int mode, fragment *f)
+{
+    return eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
+                         fx, fy, mode_cutoff_sq(mode), mode_min_alpha(mode), 0, NULL, f);
+}
+
+/* position gradient of one fragment from the fourth column of dL/dVPMT, backward.cuh:292-305 */
+static inline void position_grad(const oracle_cam *c, const frag_grads *g, float out[3])
+{
+    const float *V = c->VPM;
+    const float c4[3] = { g->dV1[3], g->dV2[3], g->dV4[3] };
+    for (int k = 0; k < 3; ++k) out[k] = V[0 + k] * c4[0] + V[4 + k] * c4[1] + V[12 + k] * c4[2];
+}
+
+/* convert_quaternion_to_rotation_matrix_backward, R/include/kernel_utils.cuh:44-61 */
+static void quat_backward(const float *q, const float dR[9], float out[4])
+{
+    const float r = q[0], x = q[1], y = q[2], z = q[3];
+    const float s21 = dR[3] - dR[1], a21 = dR[3] + dR[1];
+    const float s13 = dR[2] - dR[6], a13 = dR[2] + dR[6];
+    const float s32 = dR[7] - dR[5], a32 = dR[7] + dR[5];
+    out[0] = 2.0f * (x * s32 + y * s13 + z * s21);
+    out[1] = 2.0f * (r * s32 - 2.0f * x * (dR[4] + dR[8]) + y * a21 + z * a13);
+    out[2] = 2.0f * (r * s13 + x * a21 - 2.0f * y * (dR[0] + dR[8]) + z * a32);
+    out[3] = 2.0f * (r * s21 + x * a13 + y * a32 - 2.0f * z * (dR[0] + dR[4]));
+}
+
+/* dL/dscale and dL/dquaternion from dL/dVPMT[:, :3] (rows 1, 2, 4; columns c1..c3),
+ * R/include/hybrid_blend/kernels/backward.cuh:39-70 = alpha_blend_first_k/kernels/backward.cuh:161-190 */
+static void scale_rotation_grad(const oracle_cam *c, const float *scale, const float *quat,
+                                const float c1[3], const float c2[3], const float c3[3], float dscale[3], float dquat[4])
+{
+    float R[9];
+    quat_to_rot(quat, R);
+    const float *V1 = c->VPM, *V2 = c->VPM + 4, *V4 = c->VPM + 12;
+    const float Rc[3][3] = { { R[0], R[3], R[6] }, { R[1], R[4], R[7] }, { R[2], R[5], R[8] } };
+    const float *cols[3] = { c1, c2, c3 };
+    for (int k = 0; k < 3; ++k) {
+        const float t[3] = { dot3(V1, Rc[k]), dot3(V2, Rc[k]), dot3(V4, Rc[k]) };
+        dscale[k] = dot3(t, cols[k]);
+    }
+    float dR[9];
+    for (int row = 0; row < 3; ++row) {
+        const float vc[3] = { V1[row], V2[row], V4[row] };
+        for (int k = 0; k < 3; ++k) dR[3 * row + k] = dot3(vc, cols[k]) * scale[k];
+    }
+    quat_backward(quat, dR, dquat);
+}
+
+/* Backward blend of every mode.  Accumulates, per Gaussian:
+ *   grad_rgb [N][3]  dL/d(clamped colour)   (the reference keeps it in grad_sh_0)
+ *   grad_opacities [N], grad_positions [N][3] (ray part only)
+ *   hybrid / oit: grad_VPMT [9][N] (rows 1, 2, 4 x columns 1..3; backward.cuh:319-327)
+ *   first_k / global: grad_scales [N][3], grad_rotations [N][4] directly, per fragment
+ *   helper [N]: sum over fragments of |dL/dposition|_1, or NULL
+ * hybrid, oit:  R/include/hybrid_blend/kernels/backward.cuh:104-331, R/include/oit_blend/kernels/backward.cuh:104-290
+ * first_k:      R/include/alpha_blend_first_k/kernels/backward.cuh:60-206
+ * global:       R/include/alpha_blend_global_ordering/kernels/backward.cuh:60-251
+ * Sums are formed in a fixed order (tile by tile, the reference uses atomics). */
+O_EXPORT void oracle_blend_backward(
+    const oracle_cam *c, int n, const uint32_t *ranges, const uint32_t *inst,
+    const float *VPMT1, const float *VPMT2, const float *VPMT4, const float *rgba,
+    const float *scales, const float *rotations, const float *image,
+    const uint32_t *core_idx, const float *core_info, const float *tail_info, const float *grad_image,
+    float *grad_positions, float *grad_scales, float *grad_rotations, float *grad_opacities, float *grad_rgb,
+    float *grad_VPMT, float *helper)
+{
+    const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
+    const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
+    const blend_in in = { ranges, inst, VPMT1, VPMT2, VPMT4, VPMT1 /* MT3 unused */, rgba };
+    const int K = round_k(c->K);
+    const size_t np = (size_t)c->width * c->height;
+    const int mode = c->mode;
+
+    if (mode == MODE_FIRST_K) {
+        /* one stored fragment at a time, backward.cuh:81-205 */
+        for (size_t frag = 0; frag < np * (size_t)K; ++frag) {
+            const size_t pix = frag / K, slot = frag % K;
+            const uint32_t g = core_idx[slot * np + pix];
+            if (g == UINT32_MAX) continue;
+            const float fx = (float)(pix % c->width), fy = (float)(pix / c->width);
+            const float gp[3] = { grad_image[pix], grad_image[np + pix], grad_image[2 * np + pix] };
+            const float *info = core_info + 4 * (slot * np + pix);
+            for (int k = 0; k < 3; ++k) grad_rgb[3 * (size_t)g + k] += info[3] * gp[k];
+            const float dL_dalpha = dot3(info, gp);
+            if (dL_dalpha == 0.0f) continue;
+            fragment f;
+            /* no cut-off / threshold test here: the fragment is known to be in the core (backward.cuh:104-115) */
+            for (int k = 0; k < 4; ++k) {
+                f.px[k] = fmaf(-VPMT4[4 * (size_t)g + k], fx, VPMT1[4 * (size_t)g + k]);
+                f.py[k] = fmaf(-VPMT4[4 * (size_t)g + k], fy, VPMT2[4 * (size_t)g + k]);
+            }
+            for (int k = 0; k < 3; ++k) f.m[k] = fmaf(f.px[3], f.py[k], -(f.px[k] * f.py[3]));
+            f.d[0] = fmaf(f.px[1], f.py[2], -(f.px[2] * f.py[1]));
+            f.d[1] = fmaf(f.px[2], f.py[0], -(f.px[0] * f.py[2]));
+            f.d[2] = fmaf(f.px[0], f.py[1], -(f.px[1] * f.py[0]));
+            f.num = fmaf(f.m[2], f.m[2], fmaf(f.m[1], f.m[1], f.m[0] * f.m[0]));
+            f.den = fmaf(f.d[2], f.d[2], fmaf(f.d[1], f.d[1], f.d[0] * f.d[0]));
+            f.den_rcp = 1.0f / f.den;
+            f.G = o_expf((-0.5f * f.num) * f.den_rcp);
+            frag_grads fg;
+            fragment_backward(&f, rgba[4 * (size_t)g + 3], dL_dalpha, fx, fy, &fg);
+            grad_opacities[g] += fg.opacity;
+            float dp[3];
+            position_grad(c, &fg, dp);
+            for (int k = 0; k < 3; ++k) grad_positions[3 * (size_t)g + k] += dp[k];
+            const float c1[3] = { fg.dV1[0], fg.dV2[0], fg.dV4[0] }, c2[3] = { fg.dV1[1], fg.dV2[1], fg.dV4[1] }, c3[3] = { fg.dV1[2], fg.dV2[2], fg.dV4[2] };
+            float ds[3], dq[4];
+            scale_rotation_grad(c, scales + 3 * (size_t)g, rotations + 4 * (size_t)g, c1, c2, c3, ds, dq);
+            for (int k = 0; k < 3; ++k) grad_scales[3 * (size_t)g + k] += ds[k];
+            for (int k = 0; k < 4; ++k) grad_rotations[4 * (size_t)g + k] += dq[k];
+            if (helper) helper[g] += fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]);
+        }
+        return;
+    }
+
+    for (int t = 0; t < grid_w * grid_h; ++t) {
+        const int tx = t % grid_w, ty = t / grid_w;
+        const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        if (mode == MODE_GLOBAL) {
+            /* per pixel front to back, with the final colour of the pixel, backward.cuh:97-249 */
+            for (int l = 0; l < c->tile_w * c->tile_h; ++l) {
+                const int x = tx * c->tile_w + l % c->tile_w, y = ty * c->tile_h + l / c->tile_w;
+                if (x >= c->width || y >= c->height) continue;
+                const size_t pix = (size_t)c->width * y + x;
+                const float fx = (float)x, fy = (float)y;
+                const float gp[3] = { grad_image[pix], grad_image[np + pix], grad_image[2 * np + pix] };
+                const float fin[3] = { image[pix], image[np + pix], image[2 * np + pix] };
+                float rgb_new[3] = { 0, 0, 0 }, T = 1.0f;
+                for (uint32_t j = first; j < last; ++j) {
+                    const size_t g = inst[j];
+                    fragment f;
+                    if (!reeval_fragment(&in, g, fx, fy, mode, &f)) continue;
+                    const float bw = T * f.alpha;
+                    const float *col = rgba + 4 * g;
+                    for (int k = 0; k < 3; ++k) grad_rgb[3 * g + k] += bw * gp[k];
+                    for (int k = 0; k < 3; ++k) rgb_new[k] = fmaf(bw, col[k], rgb_new[k]);
+                    const float oma = 1.0f - f.alpha;
+                    const float omar = 1.0f / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS);
+                    float v[3];
+                    for (int k = 0; k < 3; ++k) v[k] = T * col[k] - (fin[k] - rgb_new[k]) * omar;
+                    const float dL_dalpha = dot3(v, gp);
+                    if (dL_dalpha != 0.0f) {
+                        frag_grads fg;
+                        fragment_backward(&f, col[3], dL_dalpha, fx, fy, &fg);
+                        grad_opacities[g] += fg.opacity;
+                        float dp[3];
+                        position_grad(c, &fg, dp);
+                        for (int k = 0; k < 3; ++k) grad_positions[3 * g + k] += dp[k];
+                        const float c1[3] = { fg.dV1[0], fg.dV2[0], fg.dV4[0] }, c2[3] = { fg.dV1[1], fg.dV2[1], fg.dV4[1] }, c3[3] = { fg.dV1[2], fg.dV2[2], fg.dV4[2] };
+                        float ds[3], dq[4];
+                        scale_rotation_grad(c, scales + 3 * g, rotations + 4 * g, c1, c2, c3, ds, dq);
+                        for (int k = 0; k < 3; ++k) grad_scales[3 * g + k] += ds[k];
+                        for (int k = 0; k < 4; ++k) grad_rotations[4 * g + k] += dq[k];
+                        if (helper) helper[g] += fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]);
+                    }
+                    T *= oma;
+                    if (T < TRANSMITTANCE_THRESHOLD) break;
+                }
+            }
+            continue;
+        }
+        /* hybrid / oit: one Gaussian of the tile at a time, all 64 pixels, then one addition per accumulator */
+        for (uint32_t j = first; j < last; ++j) {
+            const size_t g = inst[j];
+            const float *col = rgba + 4 * g;
+            float a_rgb[3] = { 0, 0, 0 }, a_op = 0, a_pos[3] = { 0, 0, 0 }, a_V1[3] = { 0, 0, 0 }, a_V2[3] = { 0, 0, 0 }, a_V4[3] = { 0, 0, 0 }, a_help = 0;
+            for (int l = 0; l < c->tile_w * c->tile_h; ++l) {
+                const int x = tx * c->tile_w + l % c->tile_w, y = ty * c->tile_h + l / c->tile_w;
+                if (x >= c->width || y >= c->height) continue;
+                const size_t pix = (size_t)c->width * y + x;
+                const float fx = (float)x, fy = (float)y;
+                fragment f;
+                if (!reeval_fragment(&in, g, fx, fy, mode, &f)) continue;
+                const float gp[3] = { grad_image[pix], grad_image[np + pix], grad_image[2 * np + pix] };
+                int slot = -1;
+                if (mode == MODE_HYBRID)
+                    for (int i = 0; i < K; ++i) if (core_idx[i * np + pix] == (uint32_t)g) slot = i;   /* backward.cuh:231-235 */
+                float dL_dalpha;
+                if (slot >= 0) {
+                    const float *info = core_info + 4 * (slot * np + pix);
+                    for (int k = 0; k < 3; ++k) a_rgb[k] += info[3] * gp[k];                        /* :154, :241 */
+                    dL_dalpha = dot3(info, gp);                                                    /* :155 */
+                } else {
+                    const float rt[3] = { tail_info[pix], tail_info[np + pix], tail_info[2 * np + pix] };
+                    const float asr = tail_info[3 * np + pix], T_tail = tail_info[4 * np + pix];
+                    const float T_core = mode == MODE_HYBRID ? tail_info[5 * np + pix] : 1.0f;
+                    const float w_tail = T_core * asr;                                             /* :166 */
+                    const float full = w_tail * (1.0f - T_tail);                                   /* :168 */
+                    const float rdg = dot3(rt, gp);
+                    for (int k = 0; k < 3; ++k) a_rgb[k] += (full * gp[k]) * f.alpha;              /* :170, :244 */
+                    const float common = -full * asr * rdg;                                        /* :171 */
+                    const float cg[3] = { full * gp[0], full * gp[1], full * gp[2] };              /* :172 */
+                    const float a_term = w_tail * T_tail * rdg;                                    /* :173 */
+                    const float oma = 1.0f - f.alpha;
+                    dL_dalpha = common + dot3(col, cg) + a_term / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS);   /* :253-255 */
+                }
+                if (dL_dalpha == 0.0f) continue;                                                   /* :258 */
+                frag_grads fg;
+                fragment_backward(&f, col[3], dL_dalpha, fx, fy, &fg);
+                a_op += fg.opacity;
+                for (int k = 0; k < 3; ++k) { a_V1[k] += fg.dV1[k]; a_V2[k] += fg.dV2[k]; a_V4[k] += fg.dV4[k]; }
+                float dp[3];
+                position_grad(c, &fg, dp);
+                for (int k = 0; k < 3; ++k) a_pos[k] += dp[k];
+                a_help += fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]);
+            }
+            for (int k = 0; k < 3; ++k) {
+                grad_rgb[3 * g + k] += a_rgb[k];
+                grad_positions[3 * g + k] += a_pos[k];
+                grad_VPMT[(size_t)(0 + k) * n + g] += a_V1[k];
+                grad_VPMT[(size_t)(3 + k) * n + g] += a_V2[k];
+                grad_VPMT[(size_t)(6 + k) * n + g] += a_V4[k];
+            }
+            grad_opacities[g] += a_op;
+            if (helper) helper[g] += a_help;
+        }
+    }
+}
+
+/* convert_sh_to_rgb_backward, R/include/kernel_utils.cuh:190-281.  grad_sh0 holds dL/drgb on entry and
+ * dL/dsh_0 on exit; returns the colour's contribution to dL/dposition in dpos. */
+static void sh_backward(const oracle_cam *c, const float *rest, const uint8_t clamp[3], const float *p,
+                        float *grad_sh0, float *grad_rest, float dpos[3])
+{
+    float g[3];
+    for (int k = 0; k < 3; ++k) g[k] = clamp[k] ? 0.0f : grad_sh0[k];
+    for (int k = 0; k < 3; ++k) grad_sh0[k] = 0.28209479177387814f * g[k];
+    dpos[0] = dpos[1] = dpos[2] = 0.0f;
+    if (c->active_sh <= 1) return;
+    const float xr = p[0] - c->cam[0], yr = p[1] - c->cam[1], zr = p[2] - c->cam[2];
+    const float inv = 1.0f / sqrtf(xr * xr + yr * yr + zr * zr);
+    const float x = xr * inv, y = yr * inv, z = zr * inv;
+    float b[15] = { 0 }, dx[3] = { 0, 0, 0 }, dy[3] = { 0, 0, 0 }, dz[3] = { 0, 0, 0 };
+    int nb = 3;
+    b[0] = -0.48860251190291987f * y; b[1] = 0.48860251190291987f * z; b[2] = -0.48860251190291987f * x;
+    for (int k = 0; k < 3; ++k) {
+        dx[k] = -0.48860251190291987f * rest[2 * 3 + k];
+        dy[k] = -0.48860251190291987f * rest[0 * 3 + k];
+        dz[k] = 0.48860251190291987f * rest[1 * 3 + k];
+    }
+    if (c->active_sh > 4) {
+        nb = 8;
+        const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, xz = x * z, yz = y * z;
+        b[3] = 1.0925484305920792f * xy; b[4] = -1.0925484305920792f * yz; b[5] = 0.94617469575755997f * zz - 0.31539156525251999f;
+        b[6] = -1.0925484305920792f * xz; b[7] = 0.54627421529603959f * xx - 0.54627421529603959f * yy;
+        for (int k = 0; k < 3; ++k) {
+            dx[k] = dx[k] + (1.0925484305920792f * y) * rest[3 * 3 + k] + (-1.0925484305920792f * z) * rest[6 * 3 + k] + (1.0925484305920792f * x) * rest[7 * 3 + k];
+            dy[k] = dy[k] + (1.0925484305920792f * x) * rest[3 * 3 + k] + (-1.0925484305920792f * z) * rest[4 * 3 + k] + (-1.0925484305920792f * y) * rest[7 * 3 + k];
+            dz[k] = dz[k] + (-1.0925484305920792f * y) * rest[4 * 3 + k] + (1.8923493915151202f * z) * rest[5 * 3 + k] + (-1.0925484305920792f * x) * rest[6 * 3 + k];
+        }
+        if (c->active_sh > 9) {
+            nb = 15;
+            b[8] = 0.59004358992664352f * y * (-3.0f * xx + yy); b[9] = 2.8906114426405538f * xy * z;
+            b[10] = 0.45704579946446572f * y * (1.0f - 5.0f * zz); b[11] = 0.3731763325901154f * z * (5.0f * zz - 3.0f);
+            b[12] = 0.45704579946446572f * x * (1.0f - 5.0f * zz); b[13] = 1.4453057213202769f * z * (xx - yy);
+            b[14] = 0.59004358992664352f * x * (-xx + 3.0f * yy);
+            for (int k = 0; k < 3; ++k) {
+                dx[k] = dx[k] + (-3.5402615395598609f * xy) * rest[8 * 3 + k] + (2.8906114426405538f * yz) * rest[9 * 3 + k]
+                              + (0.45704579946446572f - 2.2852289973223288f * zz) * rest[12 * 3 + k] + (2.8906114426405538f * xz) * rest[13 * 3 + k]
+                              + (-1.7701307697799304f * xx + 1.7701307697799304f * yy) * rest[14 * 3 + k];
+                dy[k] = dy[k] + (-1.7701307697799304f * xx + 1.7701307697799304f * yy) * rest[8 * 3 + k] + (2.8906114426405538f * xz) * rest[9 * 3 + k]
+                              + (0.45704579946446572f - 2.2852289973223288f * zz) * rest[10 * 3 + k] + (-2.8906114426405538f * yz) * rest[13 * 3 + k]
+                              + (3.5402615395598609f * xy) * rest[14 * 3 + k];
+                dz[k] = dz[k] + (2.8906114426405538f * xy) * rest[9 * 3 + k] + (-4.5704579946446566f * yz) * rest[10 * 3 + k]
+                              + (5.597644988851731f * zz - 1.1195289977703462f) * rest[11 * 3 + k] + (-4.5704579946446566f * xz) * rest[12 * 3 + k]
+                              + (1.4453057213202769f * xx - 1.4453057213202769f * yy) * rest[13 * 3 + k];
+            }
+        }
+    }
+    for (int i = 0; i < nb; ++i)
+        for (int k = 0; k < 3; ++k) grad_rest[3 * i + k] = b[i] * g[k];
+    const float gd[3] = { dot3(dx, g), dot3(dy, g), dot3(dz, g) };
+    const float xx = xr * xr, yy = yr * yr, zz = zr * zr, xy = xr * yr, xz = xr * zr, yz = yr * zr;
+    const float n2 = xx + yy + zz;
+    const float s = 1.0f / sqrtf(n2 * n2 * n2);
+    dpos[0] = ((yy + zz) * gd[0] - xy * gd[1] - xz * gd[2]) * s;
+    dpos[1] = (-xy * gd[0] + (xx + zz) * gd[1] - yz * gd[2]) * s;
+    dpos[2] = (-xz * gd[0] - yz * gd[1] + (xx + yy) * gd[2]) * s;
+}
+
+/* preprocess_cu (backward): R/include/hybrid_blend/kernels/backward.cuh:10-102 (grad_VPMT != NULL: also scale and
+ * rotation gradients) and R/include/alpha_blend_first_k/kernels/backward.cuh:10-58 (grad_VPMT == NULL).
+ * densification_info is [2 or 3][N] or NULL (R/src/rasterization_api.cu:219-223). */
+O_EXPORT void oracle_preprocess_backward(
+    const oracle_cam *c, int n, const float *positions, const float *scales, const float *rotations, const float *sh_rest,
+    const uint32_t *n_touched, const uint8_t *clamp_info, const float *grad_VPMT, const float *helper,
+    float *grad_positions, float *grad_scales, float *grad_rotations, float *grad_sh_0, float *grad_sh_rest,
+    float *densification_info, int use_distance_scaling)
+{
+    #pragma omp parallel for schedule(static)
+    for (int i = 0; i < n; ++i) {
+        if (n_touched[i] == 0) continue;
+        if (grad_VPMT) {
+            float col[3][3];
+            for (int k = 0; k < 3; ++k) {
+                col[k][0] = grad_VPMT[(size_t)(0 + k) * n + i];
+                col[k][1] = grad_VPMT[(size_t)(3 + k) * n + i];
+                col[k][2] = grad_VPMT[(size_t)(6 + k) * n + i];
+            }
+            scale_rotation_grad(c, scales + 3 * (size_t)i, rotations + 4 * (size_t)i, col[0], col[1], col[2],
+                                grad_scales + 3 * (size_t)i, grad_rotations + 4 * (size_t)i);
+        }
+        const float *p = positions + 3 * (size_t)i;
+        const uint8_t clamp[3] = { clamp_info[i], clamp_info[(size_t)n + i], clamp_info[2 * (size_t)n + i] };
+        float dpos[3];
+        sh_backward(c, sh_rest + 3 * (size_t)c->total_sh * i, clamp, p, grad_sh_0 + 3 * (size_t)i,
+                    grad_sh_rest + 3 * (size_t)c->total_sh * i, dpos);
+        float *gp = grad_positions + 3 * (size_t)i;
+        for (int k = 0; k < 3; ++k) gp[k] = gp[k] + dpos[k];
+        if (densification_info) {
+            float z_scale = 1.0f;
+            if (use_distance_scaling) z_scale = (dot3(c->M3, p) + c->M3[3]) * 0.5f;
+            const float v[3] = { gp[0] * z_scale, gp[1] * z_scale, gp[2] * z_scale };
+            densification_info[i] += 1.0f;
+            densification_info[(size_t)n + i] += sqrtf(dot3(v, v));
+            if (helper) densification_info[2 * (size_t)n + i] += z_scale * helper[i];
+        }
+    }
+}

@@ -1,0 +1,78 @@
+"""Pins the oracle's training path (forward records + backward): gradients against torch.autograd through the
+independent float64 evaluator (oracle/bruteforce.py), which knows nothing of the reference's hand-derived chain
+rule; linearity in the upstream gradient; zero gradients for culled Gaussians; the densification side outputs
+against their definition (R/include/hybrid_blend/kernels/backward.cuh:85-98,306)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import bruteforce as bf
+from test_oracle_pinning import small_scene
+from util import oracle_frame
+
+NAMES = ["positions", "scales", "rotations", "opacities", "sh_0", "sh_rest"]
+
+
+def autograd_reference(sc, mode, K, grad_image):
+    leaves = [t.double().clone().requires_grad_(True) for t in sc.gaussians()]
+    frags = bf.evaluate(*leaves, sc.M, sc.VPM, sc.cam_position, mode, sc.active_sh_bases, sc.width, sc.height,
+                        sc.near_plane, sc.far_plane)
+    img, _, _, margin = bf.render(frags, mode, K, False, clamp=False)
+    mask = (margin > 1e-4)
+    (img * grad_image.double() * mask.double()).sum().backward()
+    return img.detach(), mask, [l.grad for l in leaves]
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("K,sh_degree", [(4, 2), (16, 3), (1, 0)])
+def test_backward_matches_float64_autograd(mode, K, sh_degree):
+    sc = small_scene(n=70, seed=31 + mode + K, sh_degree=sh_degree)
+    arrays = [t.numpy() for t in sc.gaussians()]
+    fwd = oracle.forward(oracle_frame(sc, mode, K), *arrays)
+    gi = torch.randn(3, sc.height, sc.width, generator=torch.Generator().manual_seed(1))
+    img, mask, want = autograd_reference(sc, mode, K, gi)
+    assert mask.float().mean() > 0.97
+    assert np.abs(fwd["image"] - img.numpy())[:, mask.numpy()].max() < 2e-5
+    got = oracle.backward(fwd, (gi * mask.float()).numpy(), *arrays)
+    for name, w in zip(NAMES, want):
+        g = got[name]
+        if w is None or g.size == 0:          # sh_rest of an SH-degree-0 scene has no elements
+            continue
+        w = w.numpy().reshape(g.shape)
+        scale = max(np.abs(w).max(), 1e-12)
+        assert np.abs(g - w).max() / scale < 2e-5, (name, np.abs(g - w).max(), scale)
+
+
+def test_backward_is_linear_in_the_upstream_gradient_and_ignores_culled_gaussians():
+    sc = small_scene(n=80, seed=5)
+    sc.positions[:10] = sc.positions[:10] * 0 + torch.tensor([0.0, 0.0, -30.0])        # behind the camera
+    arrays = [t.numpy() for t in sc.gaussians()]
+    fwd = oracle.forward(oracle_frame(sc, 0, 4), *arrays)
+    g = torch.Generator().manual_seed(2)
+    a, b = torch.randn(3, sc.height, sc.width, generator=g).numpy(), torch.randn(3, sc.height, sc.width, generator=g).numpy()
+    ga, gb, gab = (oracle.backward(fwd, x, *arrays) for x in (a, b, 2 * a - 3 * b))
+    for name in NAMES:
+        np.testing.assert_allclose(gab[name], 2 * ga[name] - 3 * gb[name], rtol=0, atol=2e-4 * max(1.0, np.abs(gab[name]).max()))
+        assert (ga[name][:10] == 0).all()
+
+
+def test_densification_side_outputs():
+    sc = small_scene(n=60, seed=9)
+    arrays = [t.numpy() for t in sc.gaussians()]
+    fwd = oracle.forward(oracle_frame(sc, 0, 4), *arrays)
+    gi = torch.randn(3, sc.height, sc.width, generator=torch.Generator().manual_seed(3)).numpy()
+    n = 60
+    vis = fwd["pre"]["n_touched"] > 0
+    z = (sc.positions.numpy() @ sc.M.numpy()[2, :3] + sc.M.numpy()[2, 3])
+    for rows, scaling in [(2, False), (3, False), (3, True)]:
+        info = np.full((rows, n), 0.5, np.float32)
+        grads = oracle.backward(fwd, gi, *arrays, densification_info=info, use_distance_scaling=scaling)
+        zs = z * 0.5 if scaling else np.ones(n)
+        np.testing.assert_allclose(info[0], 0.5 + vis, rtol=0, atol=0)
+        np.testing.assert_allclose(info[1], 0.5 + vis * np.linalg.norm(grads["positions"] * zs[:, None], axis=1), rtol=1e-5, atol=1e-6)
+        if rows == 3:
+            assert (info[2][vis] >= 0.5).all() and (info[2][~vis] == 0.5).all()
+            # |.|_1 summed per fragment dominates the 1-norm of the summed ray-space gradient
+            ray_part = grads["positions"] - 0  # includes the (small) colour-direction term; allow for it
+            assert (info[2] - 0.5 + 1e-3 >= 0.2 * np.abs(ray_part).sum(1) * np.abs(zs) * vis).all()
