@@ -53,6 +53,21 @@ class Frame(ctypes.Structure):
         ("depth", ctypes.c_void_p),
         ("to_chw", ctypes.c_int32),
         ("use_median_depth", ctypes.c_int32),
+        ("core_idx", ctypes.c_void_p),
+        ("core_info", ctypes.c_void_p),
+        ("tail_info", ctypes.c_void_p),
+        ("grad_image", ctypes.c_void_p),
+        ("grad_acc", ctypes.c_void_p),
+        ("dens_helper", ctypes.c_void_p),
+        ("grad_positions", ctypes.c_void_p),
+        ("grad_scales", ctypes.c_void_p),
+        ("grad_rotations", ctypes.c_void_p),
+        ("grad_opacities", ctypes.c_void_p),
+        ("grad_sh_0", ctypes.c_void_p),
+        ("grad_sh_rest", ctypes.c_void_p),
+        ("densification_info", ctypes.c_void_p),
+        ("densification_rows", ctypes.c_int32),
+        ("use_distance_scaling", ctypes.c_int32),
         ("stream", ctypes.c_void_p),
     ]
 
@@ -75,6 +90,12 @@ SYMBOLS = {
     "htgs_blend": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
     "htgs_render_front": (ctypes.c_int, [_FRAME_P]),
     "htgs_render_back": (ctypes.c_int, [_FRAME_P]),
+    "htgs_forward_front": (ctypes.c_int, [_FRAME_P]),
+    "htgs_forward_back": (ctypes.c_int, [_FRAME_P, ctypes.POINTER(ctypes.c_int)]),
+    "htgs_blend_forward": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
+    "htgs_blend_backward": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
+    "htgs_preprocess_backward": (ctypes.c_int, [_FRAME_P]),
+    "htgs_backward": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
 }
 
 _lib = None

@@ -74,3 +74,26 @@ extern "C" int htgs_render_back(const htgs_frame *f)
     if (rc != HTGS_OK) return rc;
     return htgs_blend(f, selector);
 }
+
+extern "C" int htgs_forward_front(const htgs_frame *f)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_front: null frame");
+    if (!f->clamp_info && f->n_primitives > 0) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_front: clamp_info is required for training");
+    htgs_frame t = *f;
+    t.scale_modifier = 1.0f;   // the training preprocess has no scale modifier (R/include/hybrid_blend/kernels/forward.cuh:10-76)
+    int rc = htgs_preprocess(&t);
+    if (rc != HTGS_OK) return rc;
+    return htgs_scan_offsets(&t);
+}
+
+extern "C" int htgs_forward_back(const htgs_frame *f, int *selector)
+{
+    if (!f || !selector) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_back: null argument");
+    int rc = htgs_create_instances(f);
+    if (rc != HTGS_OK) return rc;
+    rc = htgs_sort_instances(f, selector);
+    if (rc != HTGS_OK) return rc;
+    rc = htgs_extract_ranges(f, *selector);
+    if (rc != HTGS_OK) return rc;
+    return htgs_blend_forward(f, *selector);
+}

@@ -1,0 +1,548 @@
+// Backward pass of the four blend modes.
+// Restates blend_cu / preprocess_cu of R/include/hybrid_blend/kernels/backward.cuh:10-331,
+// R/include/oit_blend/kernels/backward.cuh:104-290, R/include/alpha_blend_first_k/kernels/backward.cuh:10-206,
+// R/include/alpha_blend_global_ordering/kernels/backward.cuh:60-251 and the shared chain rule of
+// R/include/kernel_utils.cuh:44-61,190-281.
+//
+// Every mode accumulates the same 16 numbers per Gaussian with float atomics (grad_acc, row-major [16][N]):
+//   0-2 dL/drgb   3 dL/dopacity   4-7 dL/dVPMT1   8-11 dL/dVPMT2   12-15 dL/dVPMT4
+// and one per-Gaussian kernel turns them into the gradients of positions, scales, rotations, opacities and SH
+// coefficients.  The reference does this for HYBRID and OIT and applies the per-Gaussian part once per fragment
+// for FIRST_K and GLOBAL_ORDERING; the map from dL/dVPMT to the parameters is linear, so summing first is the
+// same function.  Sums are formed by atomics, so their rounding depends on the order of arrival.
+#include "blend_common.h"
+
+namespace htgs {
+
+struct FragGrads {
+    float opacity;
+    float dV1[4], dV2[4], dV4[4];
+};
+
+// dL/dalpha of one fragment -> dL/dopacity and dL/dVPMT rows, R/include/hybrid_blend/kernels/backward.cuh:260-289
+__device__ __forceinline__ void fragment_backward(const Frag &f, float opacity, float dL_dalpha, float fx, float fy, FragGrads &o)
+{
+    o.opacity = dL_dalpha * f.G;
+    const float dL_drho2 = dL_dalpha * opacity * -0.5f * f.G;
+    const float dL_dnum = dL_drho2 * f.den_rcp;
+    const float dL_dden = dL_drho2 * -f.num * f.den_rcp * f.den_rcp;
+    float dm[3], dd[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { dm[k] = dL_dnum * 2.0f * f.m[k]; dd[k] = dL_dden * 2.0f * f.d[k]; }
+    const float *px = f.px, *py = f.py;
+    float dpx[4], dpy[4];
+    dpx[0] = -py[3] * dm[0] - py[2] * dd[1] + py[1] * dd[2];
+    dpx[1] = -py[3] * dm[1] + py[2] * dd[0] - py[0] * dd[2];
+    dpx[2] = -py[3] * dm[2] - py[1] * dd[0] + py[0] * dd[1];
+    dpx[3] = py[0] * dm[0] + py[1] * dm[1] + py[2] * dm[2];
+    dpy[0] = px[3] * dm[0] + px[2] * dd[1] - px[1] * dd[2];
+    dpy[1] = px[3] * dm[1] - px[2] * dd[0] + px[0] * dd[2];
+    dpy[2] = px[3] * dm[2] + px[1] * dd[0] - px[0] * dd[1];
+    dpy[3] = -(px[0] * dm[0] + px[1] * dm[1] + px[2] * dm[2]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        o.dV1[k] = dpx[k];
+        o.dV2[k] = dpy[k];
+        o.dV4[k] = -fx * dpx[k] - fy * dpy[k];
+    }
+}
+
+// |VPM[:, :3]^T (dV1.w, dV2.w, dV4.w)|_1: 1-norm of the fragment's position gradient (backward.cuh:292-306)
+__device__ __forceinline__ float position_grad_l1(const float *__restrict__ VPM, const FragGrads &g)
+{
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) s += fabsf(VPM[k] * g.dV1[3] + VPM[4 + k] * g.dV2[3] + VPM[12 + k] * g.dV4[3]);
+    return s;
+}
+
+__device__ __forceinline__ void atomic_add_nonzero(float *p, float v)
+{
+    if (v != 0.0f) unsafeAtomicAdd(p, v);
+}
+
+// ---------------------------------------------------------------------------------------------
+// HYBRID_BLEND (K >= 1) and OIT_BLEND (K == 0): one lane per Gaussian of the staged batch, all lanes walk the
+// 64 pixels of the tile together (per-pixel terms are LDS broadcasts), 16 atomics per (Gaussian, tile).
+// ---------------------------------------------------------------------------------------------
+template <int K>
+__global__ void __launch_bounds__(64) blend_tail_backward_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
+    const float *__restrict__ grad_image, const float *__restrict__ VPM, float *__restrict__ grad_acc, float *__restrict__ helper,
+    uint32_t n, uint32_t width, uint32_t height, uint32_t grid_w)
+{
+    constexpr int MODE = K > 0 ? HTGS_MODE_HYBRID_BLEND : HTGS_MODE_OIT_BLEND;
+    constexpr int KS = K > 0 ? K : 1;
+    __shared__ uint32_t s_idx[64 * KS];      // [pixel][slot]
+    __shared__ float4 s_core[64 * KS];       // (weight * g, dC/dalpha . g)
+    __shared__ float4 s_tail[64];            // (full weight * g, common)
+    __shared__ float s_tail_a[64];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    const size_t np = (size_t)width * height;
+    {
+        const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
+        float4 tail = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float tail_a = 0.0f;
+        const bool inside = x < width && y < height;
+        const size_t pix = inside ? (size_t)width * y + x : 0;
+        float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f;
+        if (inside) {
+            g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix];
+            const float r0 = tail_info[pix], r1 = tail_info[np + pix], r2 = tail_info[2 * np + pix];
+            const float asr = tail_info[3 * np + pix], T_tail = tail_info[4 * np + pix], T_core = tail_info[5 * np + pix];
+            const float w_tail = T_core * asr;                                   // backward.cuh:166
+            const float full = w_tail * (1.0f - T_tail);                         // :168
+            const float rdg = r0 * g0 + r1 * g1 + r2 * g2;
+            tail = make_float4(full * g0, full * g1, full * g2, -full * asr * rdg);   // :170-172
+            tail_a = w_tail * T_tail * rdg;                                      // :173
+        }
+        s_tail[lane] = tail;
+        s_tail_a[lane] = tail_a;
+        if (K > 0) {
+#pragma unroll
+            for (int i = 0; i < KS; ++i) {
+                uint32_t idx = 0xffffffffu;
+                float4 c = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (inside) {
+                    idx = core_idx[(size_t)i * np + pix];
+                    const float4 info = core_info[(size_t)i * np + pix];
+                    c = make_float4(info.w * g0, info.w * g1, info.w * g2, info.x * g0 + info.y * g1 + info.z * g2);   // :154-155
+                }
+                s_idx[lane * KS + i] = idx;
+                s_core[lane * KS + i] = c;
+            }
+        }
+    }
+    __syncthreads();
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        const bool valid = base + lane < last;
+        const uint32_t g = valid ? inst[base + lane] : 0u;
+        const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
+        // a lane without a Gaussian evaluates a record that every pixel rejects (|m|^2 = 1 > cutoff * 0)
+        const float4 V1 = valid ? rec[0] : make_float4(0.0f, 0.0f, 0.0f, 1.0f);
+        const float4 V2 = valid ? rec[1] : make_float4(1.0f, 0.0f, 0.0f, 0.0f);
+        const float4 V4 = valid ? rec[2] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        const float4 col = valid ? rec[4] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        float acc[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) acc[k] = 0.0f;
+        float help = 0.0f;
+        for (uint32_t p = 0; p < 64; ++p) {
+            const uint32_t x = x0 + (p & 7), y = y0 + (p >> 3);
+            if (x >= width || y >= height) continue;                             // uniform
+            const float fx = (float)x, fy = (float)y;
+            Frag f;
+            if (!frag_cutoff<MODE>(V1, V2, V4, fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            if (!frag_alpha<MODE>(col.w, f)) continue;
+            int slot = -1;
+            if (K > 0 && f.alpha >= kMinAlphaCore) {
+#pragma unroll
+                for (int i = 0; i < KS; ++i)
+                    if (s_idx[p * KS + i] == g) slot = i;                        // :231-235
+            }
+            float dL_dalpha;
+            if (slot >= 0) {
+                const float4 c = s_core[p * KS + slot];
+                acc[0] += c.x; acc[1] += c.y; acc[2] += c.z;                     // :241
+                dL_dalpha = c.w;                                                 // :250
+            } else {
+                const float4 t = s_tail[p];
+                acc[0] += t.x * f.alpha; acc[1] += t.y * f.alpha; acc[2] += t.z * f.alpha;   // :244
+                const float oma = 1.0f - f.alpha;
+                dL_dalpha = t.w + (col.x * t.x + col.y * t.y + col.z * t.z)
+                          + s_tail_a[p] / (oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255
+            }
+            if (dL_dalpha == 0.0f) continue;                                     // :258
+            FragGrads fg;
+            fragment_backward(f, col.w, dL_dalpha, fx, fy, fg);
+            acc[3] += fg.opacity;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { acc[4 + k] += fg.dV1[k]; acc[8 + k] += fg.dV2[k]; acc[12 + k] += fg.dV4[k]; }
+            if (helper) help += position_grad_l1(VPM, fg);
+        }
+        if (valid) {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) atomic_add_nonzero(grad_acc + (size_t)k * n + g, acc[k]);
+            if (helper) atomic_add_nonzero(helper + g, help);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// ALPHA_BLEND_FIRST_K: one thread per stored core fragment (slot, pixel), backward.cuh:81-205
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) blend_first_k_backward_kernel(
+    const float4 *__restrict__ prim, const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info,
+    const float *__restrict__ grad_image, const float *__restrict__ VPM, float *__restrict__ grad_acc, float *__restrict__ helper,
+    uint32_t n, uint32_t width, size_t np, size_t n_fragments)
+{
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (tid >= n_fragments) return;
+    const uint32_t g = core_idx[tid];
+    if (g == 0xffffffffu) return;
+    const size_t pix = tid % np;
+    const float fx = (float)(uint32_t)(pix % width), fy = (float)(uint32_t)(pix / width);
+    const float g0 = grad_image[pix], g1 = grad_image[np + pix], g2 = grad_image[2 * np + pix];
+    const float4 info = core_info[tid];
+    atomic_add_nonzero(grad_acc + g, info.w * g0);
+    atomic_add_nonzero(grad_acc + (size_t)n + g, info.w * g1);
+    atomic_add_nonzero(grad_acc + 2 * (size_t)n + g, info.w * g2);
+    const float dL_dalpha = info.x * g0 + info.y * g1 + info.z * g2;
+    if (dL_dalpha == 0.0f) return;
+    const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
+    Frag f;
+    frag_cutoff<HTGS_MODE_ALPHA_BLEND_FIRST_K>(rec[0], rec[1], rec[2], fx, fy, f);   // stored fragments passed it in forward
+    f.den_rcp = 1.0f / f.den;
+    const float opacity = rec[4].w;
+    f.G = d_expf((-0.5f * f.num) * f.den_rcp);
+    FragGrads fg;
+    fragment_backward(f, opacity, dL_dalpha, fx, fy, fg);
+    atomic_add_nonzero(grad_acc + 3 * (size_t)n + g, fg.opacity);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        atomic_add_nonzero(grad_acc + (size_t)(4 + k) * n + g, fg.dV1[k]);
+        atomic_add_nonzero(grad_acc + (size_t)(8 + k) * n + g, fg.dV2[k]);
+        atomic_add_nonzero(grad_acc + (size_t)(12 + k) * n + g, fg.dV4[k]);
+    }
+    if (helper) atomic_add_nonzero(helper + g, position_grad_l1(VPM, fg));
+}
+
+// ---------------------------------------------------------------------------------------------
+// ALPHA_BLEND_GLOBAL_ORDERING: one lane per pixel walks the depth-sorted list front to back with the final
+// colour of the pixel (backward.cuh:97-249); each Gaussian's contributions are summed over the wave before
+// one lane issues the atomics.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+    return v;
+}
+
+__global__ void __launch_bounds__(256) blend_global_backward_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    const float *__restrict__ image, const float *__restrict__ grad_image, const float *__restrict__ VPM,
+    float *__restrict__ grad_acc, float *__restrict__ helper, uint32_t n, uint32_t width, uint32_t height, uint32_t grid_w)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
+    __shared__ Stage<256> st;
+    __shared__ uint32_t st_idx[256];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t t = threadIdx.x;
+    const uint32_t lane = t & (kWave - 1);
+    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+    const size_t np = (size_t)width * height, pix = inside ? (size_t)width * y + x : 0;
+    float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, e0 = 0.0f, e1 = 0.0f, e2 = 0.0f;
+    if (inside) {
+        g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix];
+        e0 = image[pix]; e1 = image[np + pix]; e2 = image[2 * np + pix];
+    }
+    float n0 = 0.0f, n1 = 0.0f, n2 = 0.0f, T = 1.0f;
+    bool done = !inside;
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 256) {
+        if (__syncthreads_count(done) == 256) break;
+        stage_load(st, prim, inst, base + t, last, t, st_idx);
+        __syncthreads();
+        const int nb = last - base < 256u ? (int)(last - base) : 256;
+        for (int j = 0; j < nb; ++j) {
+            float acc[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) acc[k] = 0.0f;
+            float help = 0.0f;
+            bool hit = false;
+            if (!done) {
+                Frag f;
+                const float4 col = st.col[j];
+                if (frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) {
+                    f.den_rcp = 1.0f / f.den;
+                    if (frag_alpha<MODE>(col.w, f)) {
+                        hit = true;
+                        const float bw = T * f.alpha;
+                        acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                    // :171-174
+                        n0 += bw * col.x; n1 += bw * col.y; n2 += bw * col.z;                    // :178
+                        const float oma = 1.0f - f.alpha;
+                        const float omar = 1.0f / (oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);
+                        const float dL_dalpha = (T * col.x - (e0 - n0) * omar) * g0 + (T * col.y - (e1 - n1) * omar) * g1
+                                              + (T * col.z - (e2 - n2) * omar) * g2;            // :181
+                        if (dL_dalpha != 0.0f) {
+                            FragGrads fg;
+                            fragment_backward(f, col.w, dL_dalpha, fx, fy, fg);
+                            acc[3] = fg.opacity;
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) { acc[4 + k] = fg.dV1[k]; acc[8 + k] = fg.dV2[k]; acc[12 + k] = fg.dV4[k]; }
+                            if (helper) help = position_grad_l1(VPM, fg);
+                        }
+                        T *= oma;                                                                // :245
+                        if (T < kTransmittanceThreshold) done = true;
+                    }
+                }
+            }
+            if (__any(hit)) {                                                                    // wave-uniform
+                const uint32_t g = st_idx[j];
+#pragma unroll
+                for (int k = 0; k < 16; ++k) {
+                    const float s = wave_sum(acc[k]);
+                    if (lane == 0) atomic_add_nonzero(grad_acc + (size_t)k * n + g, s);
+                }
+                if (helper) {
+                    const float s = wave_sum(help);
+                    if (lane == 0) atomic_add_nonzero(helper + g, s);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-Gaussian part: grad_acc -> gradients of the parameters; SH backward; densification statistics
+// (R/include/hybrid_blend/kernels/backward.cuh:10-102, R/include/kernel_utils.cuh:44-61,190-281)
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) preprocess_backward_kernel(
+    const float *__restrict__ positions, const float *__restrict__ scales, const float *__restrict__ rotations,
+    const float *__restrict__ sh_rest, const uint32_t *__restrict__ n_touched, const uint8_t *__restrict__ clamp_info,
+    const float *__restrict__ grad_acc, const float *__restrict__ helper, const float *__restrict__ M,
+    const float *__restrict__ VPM_in, const float *__restrict__ cam_position,
+    float *__restrict__ grad_positions, float *__restrict__ grad_scales, float *__restrict__ grad_rotations,
+    float *__restrict__ grad_opacities, float *__restrict__ grad_sh_0, float *__restrict__ grad_sh_rest,
+    float *__restrict__ densification_info, int n, int active_sh, int total_sh, int use_distance_scaling)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float *gsr = grad_sh_rest + 3 * (size_t)total_sh * i;
+    if (n_touched[i] == 0) {                                                     // backward.cuh:31: nothing flows to culled Gaussians
+#pragma unroll
+        for (int k = 0; k < 3; ++k) { grad_positions[3 * (size_t)i + k] = 0.0f; grad_scales[3 * (size_t)i + k] = 0.0f; grad_sh_0[3 * (size_t)i + k] = 0.0f; }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) grad_rotations[4 * (size_t)i + k] = 0.0f;
+        grad_opacities[i] = 0.0f;
+        for (int k = 0; k < 3 * total_sh; ++k) gsr[k] = 0.0f;
+        return;
+    }
+    float a[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) a[k] = grad_acc[(size_t)k * n + i];
+    float V1[4], V2[4], V4[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { V1[k] = VPM_in[k]; V2[k] = VPM_in[4 + k]; V4[k] = VPM_in[12 + k]; }
+
+    // columns of dL/dVPMT (rows 1, 2, 4)
+    const float c1[3] = { a[4], a[8], a[12] }, c2[3] = { a[5], a[9], a[13] }, c3[3] = { a[6], a[10], a[14] }, c4[3] = { a[7], a[11], a[15] };
+    const float sx = scales[3 * (size_t)i], sy = scales[3 * (size_t)i + 1], sz = scales[3 * (size_t)i + 2];
+    const float4 q = *reinterpret_cast<const float4 *>(rotations + 4 * (size_t)i);
+    const float r = q.x, x = q.y, y = q.z, z = q.w;
+    const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, xz = x * z, yz = y * z, rx = r * x, ry = r * y, rz = r * z;
+    const float R[3][3] = { { 1.0f - 2.0f * (yy + zz), 2.0f * (xy - rz), 2.0f * (xz + ry) },
+                            { 2.0f * (xy + rz), 1.0f - 2.0f * (xx + zz), 2.0f * (yz - rx) },
+                            { 2.0f * (xz - ry), 2.0f * (yz + rx), 1.0f - 2.0f * (xx + yy) } };
+    const float *cols[3] = { c1, c2, c3 };
+    const float s[3] = { sx, sy, sz };
+    float dscale[3], dR[3][3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {                                                // backward.cuh:56-60
+        const float t1 = V1[0] * R[0][k] + V1[1] * R[1][k] + V1[2] * R[2][k];
+        const float t2 = V2[0] * R[0][k] + V2[1] * R[1][k] + V2[2] * R[2][k];
+        const float t4 = V4[0] * R[0][k] + V4[1] * R[1][k] + V4[2] * R[2][k];
+        dscale[k] = t1 * cols[k][0] + t2 * cols[k][1] + t4 * cols[k][2];
+    }
+#pragma unroll
+    for (int row = 0; row < 3; ++row)                                            // :64-68
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+            dR[row][k] = (V1[row] * cols[k][0] + V2[row] * cols[k][1] + V4[row] * cols[k][2]) * s[k];
+    const float s21 = dR[1][0] - dR[0][1], a21 = dR[1][0] + dR[0][1];
+    const float s13 = dR[0][2] - dR[2][0], a13 = dR[0][2] + dR[2][0];
+    const float s32 = dR[2][1] - dR[1][2], a32 = dR[2][1] + dR[1][2];
+    float4 dq;                                                                   // kernel_utils.cuh:55-60
+    dq.x = 2.0f * (x * s32 + y * s13 + z * s21);
+    dq.y = 2.0f * (r * s32 - 2.0f * x * (dR[1][1] + dR[2][2]) + y * a21 + z * a13);
+    dq.z = 2.0f * (r * s13 + x * a21 - 2.0f * y * (dR[0][0] + dR[2][2]) + z * a32);
+    dq.w = 2.0f * (r * s21 + x * a13 + y * a32 - 2.0f * z * (dR[0][0] + dR[1][1]));
+#pragma unroll
+    for (int k = 0; k < 3; ++k) grad_scales[3 * (size_t)i + k] = dscale[k];
+    *reinterpret_cast<float4 *>(grad_rotations + 4 * (size_t)i) = dq;
+    grad_opacities[i] = a[3];
+
+    // position: ray part from the fourth column (backward.cuh:292-305), colour part below
+    float dpos[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) dpos[k] = V1[k] * c4[0] + V2[k] * c4[1] + V4[k] * c4[2];
+
+    // SH, kernel_utils.cuh:190-281
+    const float p[3] = { positions[3 * (size_t)i], positions[3 * (size_t)i + 1], positions[3 * (size_t)i + 2] };
+    float g[3];
+    g[0] = clamp_info[i] ? 0.0f : a[0];
+    g[1] = clamp_info[(size_t)n + i] ? 0.0f : a[1];
+    g[2] = clamp_info[2 * (size_t)n + i] ? 0.0f : a[2];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) grad_sh_0[3 * (size_t)i + k] = 0.28209479177387814f * g[k];
+    for (int k = 0; k < 3 * total_sh; ++k) gsr[k] = 0.0f;
+    if (active_sh > 1) {
+        const float *c = sh_rest + 3 * (size_t)total_sh * i;
+        const float xr = p[0] - cam_position[0], yr = p[1] - cam_position[1], zr = p[2] - cam_position[2];
+        const float inv = 1.0f / __builtin_sqrtf(xr * xr + yr * yr + zr * zr);
+        const float dx_ = xr * inv, dy_ = yr * inv, dz_ = zr * inv;
+        float b[15];
+        float gx[3], gy[3], gz[3];
+        int nb = 3;
+        b[0] = -0.48860251190291987f * dy_; b[1] = 0.48860251190291987f * dz_; b[2] = -0.48860251190291987f * dx_;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            gx[k] = -0.48860251190291987f * c[6 + k];
+            gy[k] = -0.48860251190291987f * c[0 + k];
+            gz[k] = 0.48860251190291987f * c[3 + k];
+        }
+        if (active_sh > 4) {
+            nb = 8;
+            const float X = dx_, Y = dy_, Z = dz_;
+            const float XX = X * X, YY = Y * Y, ZZ = Z * Z, XY = X * Y, XZ = X * Z, YZ = Y * Z;
+            b[3] = 1.0925484305920792f * XY; b[4] = -1.0925484305920792f * YZ; b[5] = 0.94617469575755997f * ZZ - 0.31539156525251999f;
+            b[6] = -1.0925484305920792f * XZ; b[7] = 0.54627421529603959f * XX - 0.54627421529603959f * YY;
+#pragma unroll
+            for (int k = 0; k < 3; ++k) {
+                gx[k] += (1.0925484305920792f * Y) * c[9 + k] + (-1.0925484305920792f * Z) * c[18 + k] + (1.0925484305920792f * X) * c[21 + k];
+                gy[k] += (1.0925484305920792f * X) * c[9 + k] + (-1.0925484305920792f * Z) * c[12 + k] + (-1.0925484305920792f * Y) * c[21 + k];
+                gz[k] += (-1.0925484305920792f * Y) * c[12 + k] + (1.8923493915151202f * Z) * c[15 + k] + (-1.0925484305920792f * X) * c[18 + k];
+            }
+            if (active_sh > 9) {
+                nb = 15;
+                b[8] = 0.59004358992664352f * Y * (-3.0f * XX + YY); b[9] = 2.8906114426405538f * XY * Z;
+                b[10] = 0.45704579946446572f * Y * (1.0f - 5.0f * ZZ); b[11] = 0.3731763325901154f * Z * (5.0f * ZZ - 3.0f);
+                b[12] = 0.45704579946446572f * X * (1.0f - 5.0f * ZZ); b[13] = 1.4453057213202769f * Z * (XX - YY);
+                b[14] = 0.59004358992664352f * X * (-XX + 3.0f * YY);
+#pragma unroll
+                for (int k = 0; k < 3; ++k) {
+                    gx[k] += (-3.5402615395598609f * XY) * c[24 + k] + (2.8906114426405538f * YZ) * c[27 + k]
+                           + (0.45704579946446572f - 2.2852289973223288f * ZZ) * c[36 + k] + (2.8906114426405538f * XZ) * c[39 + k]
+                           + (-1.7701307697799304f * XX + 1.7701307697799304f * YY) * c[42 + k];
+                    gy[k] += (-1.7701307697799304f * XX + 1.7701307697799304f * YY) * c[24 + k] + (2.8906114426405538f * XZ) * c[27 + k]
+                           + (0.45704579946446572f - 2.2852289973223288f * ZZ) * c[30 + k] + (-2.8906114426405538f * YZ) * c[39 + k]
+                           + (3.5402615395598609f * XY) * c[42 + k];
+                    gz[k] += (2.8906114426405538f * XY) * c[27 + k] + (-4.5704579946446566f * YZ) * c[30 + k]
+                           + (5.597644988851731f * ZZ - 1.1195289977703462f) * c[33 + k] + (-4.5704579946446566f * XZ) * c[36 + k]
+                           + (1.4453057213202769f * XX - 1.4453057213202769f * YY) * c[39 + k];
+                }
+            }
+        }
+        for (int j = 0; j < nb; ++j) {
+            gsr[3 * j] = b[j] * g[0]; gsr[3 * j + 1] = b[j] * g[1]; gsr[3 * j + 2] = b[j] * g[2];
+        }
+        const float gd[3] = { gx[0] * g[0] + gx[1] * g[1] + gx[2] * g[2], gy[0] * g[0] + gy[1] * g[1] + gy[2] * g[2],
+                              gz[0] * g[0] + gz[1] * g[1] + gz[2] * g[2] };
+        const float XX = xr * xr, YY = yr * yr, ZZ = zr * zr, XY = xr * yr, XZ = xr * zr, YZ = yr * zr;
+        const float n2 = XX + YY + ZZ;
+        const float sc = 1.0f / __builtin_sqrtf(n2 * n2 * n2);
+        dpos[0] += ((YY + ZZ) * gd[0] - XY * gd[1] - XZ * gd[2]) * sc;
+        dpos[1] += (-XY * gd[0] + (XX + ZZ) * gd[1] - YZ * gd[2]) * sc;
+        dpos[2] += (-XZ * gd[0] - YZ * gd[1] + (XX + YY) * gd[2]) * sc;
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) grad_positions[3 * (size_t)i + k] = dpos[k];
+
+    if (densification_info) {                                                    // backward.cuh:85-98
+        float z_scale = 1.0f;
+        if (use_distance_scaling) z_scale = (M[8] * p[0] + M[9] * p[1] + M[10] * p[2] + M[11]) * 0.5f;
+        const float v0 = dpos[0] * z_scale, v1 = dpos[1] * z_scale, v2 = dpos[2] * z_scale;
+        densification_info[i] += 1.0f;
+        densification_info[(size_t)n + i] += __builtin_sqrtf(v0 * v0 + v1 * v1 + v2 * v2);
+        if (helper) densification_info[2 * (size_t)n + i] += z_scale * helper[i];
+    }
+}
+
+template <int K>
+static void launch_tail_backward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
+{
+    hipLaunchKernelGGL((blend_tail_backward_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
+                       (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image, f->VPM,
+                       f->grad_acc, f->dens_helper, (uint32_t)f->n_primitives, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+}
+
+}  // namespace htgs
+
+using namespace htgs;
+
+extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: null frame");
+    if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
+    if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0 || f->n_primitives < 0)
+        return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: bad argument");
+    if (f->n_primitives == 0 || f->n_instances == 0) return HTGS_OK;
+    const bool needs_core = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K;
+    const bool needs_tail = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_OIT_BLEND;
+    if (!f->ranges || !f->vals[selector] || !f->prim || !f->grad_image || !f->grad_acc || !f->VPM ||
+        (needs_core && (!f->core_idx || !f->core_info)) || (needs_tail && !f->tail_info) ||
+        (f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING && !f->image))
+        return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: null pointer");
+    const int tile = tile_size(f->mode);
+    const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
+    const uint32_t n_tiles = grid_w * grid_h;
+    hipStream_t s = (hipStream_t)f->stream;
+    const int K = htgs_effective_k(f->K);
+    switch (f->mode) {
+        case HTGS_MODE_HYBRID_BLEND:
+            switch (K) {
+                case 32: launch_tail_backward<32>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_tail_backward<16>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_tail_backward<8>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_tail_backward<4>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_tail_backward<2>(f, selector, grid_w, n_tiles); break;
+                default: launch_tail_backward<1>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_OIT_BLEND:
+            launch_tail_backward<0>(f, selector, grid_w, n_tiles);
+            break;
+        case HTGS_MODE_ALPHA_BLEND_FIRST_K: {
+            const size_t np = (size_t)f->width * f->height, n_frag = np * (size_t)K;
+            hipLaunchKernelGGL(blend_first_k_backward_kernel, dim3((unsigned)((n_frag + 255) / 256)), dim3(256), 0, s,
+                               (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->grad_image, f->VPM, f->grad_acc,
+                               f->dens_helper, (uint32_t)f->n_primitives, (uint32_t)f->width, np, n_frag);
+            break;
+        }
+        default:
+            hipLaunchKernelGGL(blend_global_backward_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
+                               (const float4 *)f->prim, f->image, f->grad_image, f->VPM, f->grad_acc, f->dens_helper,
+                               (uint32_t)f->n_primitives, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+            break;
+    }
+    return check_launch("blend_backward");
+}
+
+extern "C" int htgs_preprocess_backward(const htgs_frame *f)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: null frame");
+    if (f->n_primitives < 0 || f->total_sh_bases < 0) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: bad sizes");
+    if (f->n_primitives == 0) return HTGS_OK;
+    if (!f->positions || !f->scales || !f->rotations || !f->n_touched || !f->clamp_info || !f->grad_acc || !f->M || !f->VPM ||
+        !f->cam_position || !f->grad_positions || !f->grad_scales || !f->grad_rotations || !f->grad_opacities || !f->grad_sh_0 ||
+        (f->total_sh_bases > 0 && (!f->sh_rest || !f->grad_sh_rest)))
+        return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: null pointer");
+    if (f->densification_info && f->densification_rows != 2 && f->densification_rows != 3)
+        return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: densification_info must have 2 or 3 rows");
+    const float *helper = (f->densification_info && f->densification_rows == 3) ? f->dens_helper : nullptr;
+    if (f->densification_info && f->densification_rows == 3 && !helper)
+        return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: 3-row densification_info needs dens_helper");
+    hipLaunchKernelGGL(preprocess_backward_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), 0, (hipStream_t)f->stream,
+                       f->positions, f->scales, f->rotations, f->sh_rest, f->n_touched, f->clamp_info, f->grad_acc, helper, f->M, f->VPM,
+                       f->cam_position, f->grad_positions, f->grad_scales, f->grad_rotations, f->grad_opacities, f->grad_sh_0,
+                       f->grad_sh_rest, f->densification_info, f->n_primitives, f->active_sh_bases, f->total_sh_bases,
+                       f->use_distance_scaling);
+    return check_launch("preprocess_backward");
+}
+
+extern "C" int htgs_backward(const htgs_frame *f, int selector)
+{
+    const int rc = htgs_blend_backward(f, selector);
+    if (rc != HTGS_OK) return rc;
+    return htgs_preprocess_backward(f);
+}

@@ -7,35 +7,9 @@
 // An 8x8 tile is exactly one wave64: one workgroup = one wave, Gaussian records are staged 64 at a
 // time in LDS (every lane then reads the same address, a broadcast), the K-buffer lives in VGPRs.
 // The 16x16 tiles of the global-ordering mode use four waves and a workgroup barrier.
-#include "common.h"
+#include "blend_common.h"
 
 namespace htgs {
-
-template <int N>
-struct Stage {
-    float4 v1[N], v2[N], v4[N], mt3[N], col[N];
-};
-
-// Stages one Gaussian record per lane.
-template <int N>
-__device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
-                                           uint32_t fetch, uint32_t last, int slot, uint32_t *idx_out)
-{
-    if (fetch < last) {
-        const uint32_t g = inst[fetch];
-        const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
-        st.v1[slot] = rec[0];
-        st.v2[slot] = rec[1];
-        st.v4[slot] = rec[2];
-        st.mt3[slot] = rec[3];
-        st.col[slot] = rec[4];
-        if (idx_out) idx_out[slot] = g;
-    }
-}
-
-// exchange two VGPRs in the active lanes (one instruction instead of a select pair)
-__device__ __forceinline__ void vswap(float &a, float &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
-__device__ __forceinline__ void vswap(uint32_t &a, uint32_t &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
 
 __device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__restrict__ depths, uint32_t w, uint32_t h,
                                             uint32_t x, uint32_t y, bool chw, float r, float g, float b, float depth)

@@ -1,0 +1,363 @@
+// Training forward blend of the four modes: unclamped [3,H,W] image plus the per-pixel records that the
+// backward pass needs.  Restates blend_cu of R/include/hybrid_blend/kernels/forward.cuh:78-235,
+// R/include/alpha_blend_first_k/kernels/forward.cuh:78-215,
+// R/include/alpha_blend_global_ordering/kernels/forward.cuh:78-156 and
+// R/include/oit_blend/kernels/forward.cuh:76-165.
+//
+// Records are pixel-minor ([slot][pixel]) so that a wave writes 64 consecutive words.  Where the reference
+// leaves a record unwritten (tail with an alpha sum below 1/255, skipped core slots) zeros are stored, so that
+// backward never reads indeterminate memory.
+#include "blend_common.h"
+
+namespace htgs {
+
+__device__ __forceinline__ float one_minus_alpha_rcp(float one_minus_alpha)
+{
+    return 1.0f / (one_minus_alpha > kOneMinusAlphaEps ? one_minus_alpha : kOneMinusAlphaEps);
+}
+
+template <int K>
+__global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, uint32_t *__restrict__ core_idx, float4 *__restrict__ core_info, float *__restrict__ tail_info,
+    uint32_t width, uint32_t height, uint32_t grid_w)
+{
+    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    __shared__ Stage<64> st;
+    __shared__ uint32_t st_idx[64];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+
+    float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f;
+    float c0[K], c1[K], c2[K], c3[K], cd[K];
+    uint32_t ci[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) { c0[i] = c1[i] = c2[i] = c3[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        __syncthreads();
+        const int nb = last - base < 64u ? (int)(last - base) : 64;
+        for (int j = 0; j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            const float4 col = st.col[j];
+            if (!frag_alpha<MODE>(col.w, f)) continue;
+            float depth = frag_depth(st.mt3[j], f);
+            float p0 = col.x, p1 = col.y, p2 = col.z, p3 = f.alpha;
+            if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
+                uint32_t idx = st_idx[j];
+#pragma unroll
+                for (int i = 0; i < K; ++i) {
+                    if (depth < cd[i]) {
+                        vswap(depth, cd[i]);
+                        vswap(p0, c0[i]);
+                        vswap(p1, c1[i]);
+                        vswap(p2, c2[i]);
+                        vswap(p3, c3[i]);
+                        vswap(idx, ci[i]);
+                    }
+                }
+            }
+            tail0 += p0 * p3; tail1 += p1 * p3; tail2 += p2 * p3; tail3 += p3;
+            T_tail *= 1.0f - p3;
+        }
+    }
+    if (!inside) return;
+
+    const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    float r = 0.0f, g = 0.0f, b = 0.0f, T_core = 1.0f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        if (T_core >= kTransmittanceThreshold) {
+            const float bw = T_core * c3[i];
+            r = __builtin_fmaf(bw, c0[i], r);
+            g = __builtin_fmaf(bw, c1[i], g);
+            b = __builtin_fmaf(bw, c2[i], b);
+            T_core *= 1.0f - c3[i];
+            if (T_core < kTransmittanceThreshold) T_core = 0.0f;
+        }
+    }
+    float w0 = 0.0f, w1 = 0.0f, w2 = 0.0f;
+    float t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, t4 = 0.0f, t5 = 0.0f;
+    if (tail3 >= ModeCfg<MODE>::min_alpha) {
+        const float asr = 1.0f / tail3;
+        const float s = (T_core * (1.0f - T_tail)) * asr;
+        w0 = s * tail0; w1 = s * tail1; w2 = s * tail2;
+        t0 = tail0; t1 = tail1; t2 = tail2; t3 = asr; t4 = T_tail; t5 = T_core;
+    }
+    tail_info[pix] = t0; tail_info[np + pix] = t1; tail_info[2 * np + pix] = t2;
+    tail_info[3 * np + pix] = t3; tail_info[4 * np + pix] = t4; tail_info[5 * np + pix] = t5;
+
+    float n0 = 0.0f, n1 = 0.0f, n2 = 0.0f;
+    T_core = 1.0f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const bool skip = ci[i] == 0xffffffffu || T_core < kTransmittanceThreshold;
+        core_idx[(size_t)i * np + pix] = skip ? 0xffffffffu : ci[i];
+        float4 info = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (!skip) {
+            const float bw = T_core * c3[i];
+            n0 = __builtin_fmaf(bw, c0[i], n0);
+            n1 = __builtin_fmaf(bw, c1[i], n1);
+            n2 = __builtin_fmaf(bw, c2[i], n2);
+            const float oma = 1.0f - c3[i];
+            const float omar = one_minus_alpha_rcp(oma);
+            info.x = __builtin_fmaf(c0[i], T_core, -(((r - n0) + w0) * omar));
+            info.y = __builtin_fmaf(c1[i], T_core, -(((g - n1) + w1) * omar));
+            info.z = __builtin_fmaf(c2[i], T_core, -(((b - n2) + w2) * omar));
+            info.w = bw;
+            T_core *= oma;
+        }
+        core_info[(size_t)i * np + pix] = info;
+    }
+    image[pix] = r + w0; image[np + pix] = g + w1; image[2 * np + pix] = b + w2;
+}
+
+template <int K>
+__global__ void __launch_bounds__(64) blend_first_k_forward_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, uint32_t *__restrict__ core_idx, float4 *__restrict__ core_info,
+    uint32_t width, uint32_t height, uint32_t grid_w)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
+    __shared__ Stage<64> st;
+    __shared__ uint32_t st_idx[64];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+
+    float ca[K], cd[K];
+    uint32_t ci[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) { ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        __syncthreads();
+        const int nb = last - base < 64u ? (int)(last - base) : 64;
+        for (int j = 0; j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            float depth = frag_depth(st.mt3[j], f);
+            if (depth >= cd[K - 1]) continue;
+            if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+            float alpha = f.alpha;
+            uint32_t idx = st_idx[j];
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                if (depth < cd[i]) {
+                    vswap(depth, cd[i]);
+                    vswap(alpha, ca[i]);
+                    vswap(idx, ci[i]);
+                }
+            }
+        }
+    }
+    if (!inside) return;
+
+    const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    float r = 0.0f, g = 0.0f, b = 0.0f, T = 1.0f;
+    float k0[K], k1[K], k2[K];
+    bool open = true;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        open = open && T >= kTransmittanceThreshold && ci[i] != 0xffffffffu;
+        k0[i] = k1[i] = k2[i] = 0.0f;
+        if (open) {
+            const float bw = T * ca[i];
+            const float4 col = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS / 4) + 4];
+            k0[i] = col.x; k1[i] = col.y; k2[i] = col.z;
+            r = __builtin_fmaf(bw, col.x, r);
+            g = __builtin_fmaf(bw, col.y, g);
+            b = __builtin_fmaf(bw, col.z, b);
+            T *= 1.0f - ca[i];
+        }
+    }
+    float n0 = 0.0f, n1 = 0.0f, n2 = 0.0f;
+    T = 1.0f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const bool skip = ci[i] == 0xffffffffu || T < kTransmittanceThreshold;
+        core_idx[(size_t)i * np + pix] = skip ? 0xffffffffu : ci[i];
+        float4 info = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (!skip) {
+            const float bw = T * ca[i];
+            n0 = __builtin_fmaf(bw, k0[i], n0);
+            n1 = __builtin_fmaf(bw, k1[i], n1);
+            n2 = __builtin_fmaf(bw, k2[i], n2);
+            const float oma = 1.0f - ca[i];
+            const float omar = one_minus_alpha_rcp(oma);
+            info.x = __builtin_fmaf(k0[i], T, -((r - n0) * omar));
+            info.y = __builtin_fmaf(k1[i], T, -((g - n1) * omar));
+            info.z = __builtin_fmaf(k2[i], T, -((b - n2) * omar));
+            info.w = bw;
+            T *= oma;
+        }
+        core_info[(size_t)i * np + pix] = info;
+    }
+    image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
+}
+
+__global__ void __launch_bounds__(64) blend_oit_forward_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ tail_info, uint32_t width, uint32_t height, uint32_t grid_w)
+{
+    constexpr int MODE = HTGS_MODE_OIT_BLEND;
+    __shared__ Stage<64> st;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, nullptr);
+        __syncthreads();
+        const int nb = last - base < 64u ? (int)(last - base) : 64;
+        for (int j = 0; j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            const float4 col = st.col[j];
+            if (!frag_alpha<MODE>(col.w, f)) continue;
+            a0 = __builtin_fmaf(f.alpha, col.x, a0);
+            a1 = __builtin_fmaf(f.alpha, col.y, a1);
+            a2 = __builtin_fmaf(f.alpha, col.z, a2);
+            alpha_sum += f.alpha;
+            T *= 1.0f - f.alpha;
+        }
+    }
+    if (!inside) return;
+    const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    float r = 0.0f, g = 0.0f, b = 0.0f, t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, t4 = 0.0f, t5 = 0.0f;
+    if (alpha_sum >= ModeCfg<MODE>::min_alpha) {
+        const float asr = 1.0f / alpha_sum;
+        const float s = (1.0f - T) * asr;
+        r = s * a0; g = s * a1; b = s * a2;
+        t0 = a0; t1 = a1; t2 = a2; t3 = asr; t4 = T; t5 = 1.0f;   // row 5 plays the hybrid mode's T_core
+    }
+    tail_info[pix] = t0; tail_info[np + pix] = t1; tail_info[2 * np + pix] = t2;
+    tail_info[3 * np + pix] = t3; tail_info[4 * np + pix] = t4; tail_info[5 * np + pix] = t5;
+    image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
+}
+
+__global__ void __launch_bounds__(256) blend_global_forward_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, uint32_t width, uint32_t height, uint32_t grid_w)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
+    __shared__ Stage<256> st;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t t = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+    float r = 0.0f, g = 0.0f, b = 0.0f, T = 1.0f;
+    bool done = !inside;
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 256) {
+        if (__syncthreads_count(done) == 256) break;
+        stage_load(st, prim, inst, base + t, last, t, nullptr);
+        __syncthreads();
+        const int nb = last - base < 256u ? (int)(last - base) : 256;
+        for (int j = 0; !done && j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            const float4 col = st.col[j];
+            if (!frag_alpha<MODE>(col.w, f)) continue;
+            const float bw = T * f.alpha;
+            r = __builtin_fmaf(bw, col.x, r);
+            g = __builtin_fmaf(bw, col.y, g);
+            b = __builtin_fmaf(bw, col.z, b);
+            T *= 1.0f - f.alpha;
+            if (T < kTransmittanceThreshold) done = true;
+        }
+    }
+    if (!inside) return;
+    const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
+}
+
+template <int K>
+static void launch_hybrid_forward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
+{
+    hipLaunchKernelGGL((blend_hybrid_forward_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
+                       (const float4 *)f->prim, f->image, f->core_idx, (float4 *)f->core_info, f->tail_info,
+                       (uint32_t)f->width, (uint32_t)f->height, grid_w);
+}
+template <int K>
+static void launch_first_k_forward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
+{
+    hipLaunchKernelGGL((blend_first_k_forward_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
+                       (const float4 *)f->prim, f->image, f->core_idx, (float4 *)f->core_info,
+                       (uint32_t)f->width, (uint32_t)f->height, grid_w);
+}
+
+}  // namespace htgs
+
+using namespace htgs;
+
+extern "C" int htgs_blend_forward(const htgs_frame *f, int selector)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: null frame");
+    if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
+    if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: bad argument");
+    const bool needs_core = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K;
+    const bool needs_tail = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_OIT_BLEND;
+    if (!f->ranges || !f->image || (f->n_instances > 0 && (!f->vals[selector] || !f->prim)) ||
+        (needs_core && (!f->core_idx || !f->core_info)) || (needs_tail && !f->tail_info))
+        return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: null pointer");
+    const int tile = tile_size(f->mode);
+    const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
+    const uint32_t n_tiles = grid_w * grid_h;
+    hipStream_t s = (hipStream_t)f->stream;
+    const int K = htgs_effective_k(f->K);
+    switch (f->mode) {
+        case HTGS_MODE_HYBRID_BLEND:
+            switch (K) {
+                case 32: launch_hybrid_forward<32>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_hybrid_forward<16>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_hybrid_forward<8>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_hybrid_forward<4>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_hybrid_forward<2>(f, selector, grid_w, n_tiles); break;
+                default: launch_hybrid_forward<1>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_ALPHA_BLEND_FIRST_K:
+            switch (K) {
+                case 32: launch_first_k_forward<32>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_first_k_forward<16>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_first_k_forward<8>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_first_k_forward<4>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_first_k_forward<2>(f, selector, grid_w, n_tiles); break;
+                default: launch_first_k_forward<1>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING:
+            hipLaunchKernelGGL(blend_global_forward_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
+                               (const float4 *)f->prim, f->image, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+            break;
+        default:
+            hipLaunchKernelGGL(blend_oit_forward_kernel, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector],
+                               (const float4 *)f->prim, f->image, f->tail_info, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+            break;
+    }
+    return check_launch("blend_forward");
+}

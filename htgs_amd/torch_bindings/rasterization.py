@@ -199,6 +199,116 @@ class FrameBuffers:
         self.back()
         return self.image, self.depth
 
+    # ---- training ---------------------------------------------------------------------------
+    def alloc_pixel_records(self):
+        """PerPixelBuffers of the reference (R/include/hybrid_blend/buffer_utils.h:96-108), pixel-minor."""
+        dev, P = self.device, self.width * self.height
+        K = self.lib.htgs_effective_k(self.frame.K)
+        if self.mode in (0, 1):
+            self.core_idx = torch.empty((K, P), dtype=torch.int32, device=dev)
+            self.core_info = torch.empty((K, P, 4), dtype=torch.float32, device=dev)
+            self.frame.core_idx, self.frame.core_info = _ptr(self.core_idx), _ptr(self.core_info)
+        if self.mode in (0, 3):
+            self.tail_info = torch.empty((6, P), dtype=torch.float32, device=dev)
+            self.frame.tail_info = _ptr(self.tail_info)
+
+    def forward_front(self):
+        _native.check(self.lib.htgs_forward_front(self._ref))
+
+    def forward_back(self):
+        sel = ctypes.c_int(0)
+        _native.check(self.lib.htgs_forward_back(self._ref, ctypes.byref(sel)))
+        self.selector = sel.value
+
+    def blend_forward(self):
+        _native.check(self.lib.htgs_blend_forward(self._ref, self.selector))
+
+    def run_forward(self):
+        """``_C.forward`` of the reference: unclamped [3,H,W] image; the frame keeps what backward needs."""
+        assert self.clamp_info is not None and self.to_chw, "training frames are built with train=True, to_chw=True"
+        self.forward_front()
+        self.alloc_instances(self.read_instance_count())
+        self.alloc_pixel_records()
+        self.forward_back()
+        return self.image
+
+    def run_backward(self, grad_image: torch.Tensor, densification_info: Optional[torch.Tensor] = None,
+                     use_distance_scaling: bool = False):
+        """``_C.backward`` of the reference: the six gradients; ``densification_info`` is updated in place."""
+        dev, n = self.device, self.n
+        grad_image = _dev_f32(grad_image, "grad_image", dev)
+        if tuple(grad_image.shape) != (3, self.height, self.width):
+            raise RuntimeError("grad_image must be [3,H,W]")
+        total_sh = int(self.sh_rest.shape[1])
+        f32 = dict(dtype=torch.float32, device=dev)
+        self.grad_acc = torch.zeros((16, n), **f32)
+        grads = [torch.empty((n, 3), **f32), torch.empty((n, 3), **f32), torch.empty((n, 4), **f32), torch.empty((n, 1), **f32),
+                 torch.empty((n, 1, 3), **f32), torch.empty((n, total_sh, 3), **f32)]
+        f = self.frame
+        f.stream = torch.cuda.current_stream(dev).cuda_stream
+        f.grad_image, f.grad_acc = _ptr(grad_image), _ptr(self.grad_acc)
+        (f.grad_positions, f.grad_scales, f.grad_rotations, f.grad_opacities, f.grad_sh_0, f.grad_sh_rest) = [_ptr(g) for g in grads]
+        rows = 0
+        helper = None
+        if densification_info is not None and densification_info.numel() > 0:
+            rows = int(densification_info.shape[0])
+            if rows not in (2, 3) or densification_info.numel() != rows * n or not densification_info.is_contiguous() \
+                    or densification_info.dtype != torch.float32 or densification_info.device != dev:
+                raise RuntimeError("densification_info must be a contiguous float32 [2,N] or [3,N] tensor on the GPU")
+            f.densification_info = densification_info.data_ptr()
+            if rows == 3:
+                helper = torch.zeros(n, **f32)
+        else:
+            f.densification_info = 0
+        f.densification_rows = rows
+        f.dens_helper = _ptr(helper)
+        f.use_distance_scaling = int(bool(use_distance_scaling))
+        _native.check(self.lib.htgs_backward(self._ref, self.selector))
+        return grads
+
+
+class _Rasterize(torch.autograd.Function):
+    """Differentiable render (reference: rasterization.py:45-113).  The frame object saved on ``ctx`` owns the
+    scratch that the reference returns to Python as four byte blobs."""
+
+    @staticmethod
+    def forward(ctx, positions, scales, rotations, opacities, sh_0, sh_rest, densification_info, rasterizer_settings,
+                use_distance_scaling):
+        fb = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, rasterizer_settings, True, False, train=True)
+        image = fb.run_forward()
+        ctx.fb = fb
+        ctx.save_for_backward(positions, scales, rotations, opacities, sh_0, sh_rest)
+        ctx.densification_info = densification_info
+        ctx.mark_non_differentiable(densification_info)
+        ctx.use_distance_scaling = use_distance_scaling
+        return image
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_image):
+        _ = ctx.saved_tensors      # raises if an input was modified in place since forward
+        grads = ctx.fb.run_backward(grad_image, ctx.densification_info, ctx.use_distance_scaling)
+        ctx.fb = None
+        return (*grads, None, None, None)
+
+
+def diff_rasterize(
+    positions: torch.Tensor,
+    scales: torch.Tensor,
+    rotations: torch.Tensor,
+    opacities: torch.Tensor,
+    sh_0: torch.Tensor,
+    sh_rest: torch.Tensor,
+    densification_info: torch.Tensor,
+    settings: RasterizerSettings,
+    use_distance_scaling: bool,
+) -> torch.Tensor:
+    """Training render: unclamped image ``[3,H,W]``, differentiable w.r.t. the six Gaussian tensors;
+    ``densification_info`` ([0], [2,N] or [3,N]) is updated in place during backward (reference:
+    rasterization.py:116-137).  ``settings.scale_modifier`` is ignored, as in the reference."""
+    return _Rasterize.apply(positions, scales, rotations, opacities, sh_0, sh_rest, densification_info, settings,
+                            use_distance_scaling)
+
 
 def rasterize(
     positions: torch.Tensor,

@@ -80,6 +80,23 @@ typedef struct htgs_frame {
     float *depth;              /* [H,W] */
     int32_t to_chw;
     int32_t use_median_depth;
+    /* ---- training: per-pixel records (PerPixelBuffers, buffer_utils.h:96-108), pixel-minor ---- */
+    uint32_t *core_idx;        /* [Keff,P] primitive of each blended core slot, 0xffffffff = none (modes 0, 1) */
+    float *core_info;          /* [Keff,P,4] (dC/dalpha of the slot, blending weight)        (modes 0, 1) */
+    float *tail_info;          /* [6,P] sum alpha*rgb (3), 1/sum alpha, T_tail, T_core       (modes 0, 3) */
+    /* ---- training: backward (backward_wrapper, rasterization_api.cu:178-363) ---- */
+    const float *grad_image;   /* [3,H,W] upstream gradient */
+    float *grad_acc;           /* [16,N] zero-filled by the caller: dL/drgb (3), dL/dopacity, dL/dVPMT1, 2, 4 (4 each) */
+    float *dens_helper;        /* [N] zero-filled, sum over fragments of |dL/dposition|_1; NULL unless 3-row densification */
+    float *grad_positions;     /* [N,3] outputs; every element is written */
+    float *grad_scales;        /* [N,3] */
+    float *grad_rotations;     /* [N,4] */
+    float *grad_opacities;     /* [N] */
+    float *grad_sh_0;          /* [N,3] */
+    float *grad_sh_rest;       /* [N,total_sh_bases,3] */
+    float *densification_info; /* [densification_rows,N] updated in place, or NULL (rasterization_api.cu:219-223) */
+    int32_t densification_rows; /* 0, 2 or 3 */
+    int32_t use_distance_scaling;
     /* ---- execution ---- */
     void *stream;              /* hipStream_t */
 } htgs_frame;
@@ -118,6 +135,24 @@ int htgs_blend(const htgs_frame *f, int selector);
  * sets n_instances and calls back = create instances + sort + ranges + blend. */
 int htgs_render_front(const htgs_frame *f);
 int htgs_render_back(const htgs_frame *f);
+
+/*
+ * Training (`_C.forward` / `_C.backward`, bindings.cpp:9-10).  The forward pass ignores scale_modifier
+ * (the reference's training preprocess uses 1, R/include/hybrid_blend/kernels/forward.cuh:10-76), needs
+ * clamp_info, writes the image as [3,H,W] without clamping and fills the per-pixel records.
+ */
+/* preprocess (training variant) + scan */
+int htgs_forward_front(const htgs_frame *f);
+/* create instances + sort + ranges + forward blend; *selector as in htgs_sort_instances */
+int htgs_forward_back(const htgs_frame *f, int *selector);
+/* blend_cu (forward) of the frame's mode, R/include/<mode>/kernels/forward.cuh */
+int htgs_blend_forward(const htgs_frame *f, int selector);
+/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: accumulates into grad_acc (and dens_helper) */
+int htgs_blend_backward(const htgs_frame *f, int selector);
+/* preprocess_cu (backward), R/include/hybrid_blend/kernels/backward.cuh:10-102: grad_acc -> the six gradients */
+int htgs_preprocess_backward(const htgs_frame *f);
+/* <mode>::backward (R/src/hybrid_blend/backward.cu:26-128): blend backward, then preprocess backward */
+int htgs_backward(const htgs_frame *f, int selector);
 
 #ifdef __cplusplus
 }

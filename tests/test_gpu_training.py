@@ -1,0 +1,98 @@
+"""GPU parity of the training path (diff_rasterize): forward image and per-pixel records, then the six gradients
+and the densification side outputs, against the CPU oracle on the same seeded inputs.
+
+Tolerances: image 1e-4 max abs; gradients 1e-3 relative (atomics make the summation order of the GPU path
+non-deterministic).  "Relative" is taken per tensor against its largest reference entry, and element-wise with
+rtol 1e-3 plus a small absolute term tied to that scale, because individual entries are sums with cancellation."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from htgs_amd.synthetic import make_scene
+from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode, diff_rasterize
+from util import oracle_frame, u32
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ["positions", "scales", "rotations", "opacities", "sh_0", "sh_rest"]
+CASES = [(0, 4000, 0, 4), (0, 4000, 1, 4), (0, 4000, 2, 4), (0, 4000, 3, 4),
+         (1, 30_000, 0, 16), (1, 30_000, 1, 16), (1, 30_000, 2, 16), (1, 30_000, 3, 16),
+         (4, 40_000, 0, 16), (0, 3000, 0, 1), (0, 3000, 0, 32), (0, 3000, 1, 2)]
+
+
+def assert_grad_close(name, got, want):
+    if want.size == 0:
+        return
+    scale = float(np.abs(want).max())
+    err = float(np.abs(got - want).max())
+    assert err <= 1e-3 * max(scale, 1e-20), f"{name}: max|err| {err:.3g} vs scale {scale:.3g}"
+    np.testing.assert_allclose(got, want, rtol=1e-3, atol=2e-4 * scale + 1e-30, err_msg=name)
+
+
+@pytest.mark.parametrize("config,n,mode,K", CASES)
+def test_forward_records_and_gradients(cuda, config, n, mode, K):
+    print(f"case config={config} n={n} mode={mode} K={K}", flush=True)
+    scene = make_scene(config, n)
+    arrays = [t.numpy() for t in scene.gaussians()]
+    fwd = oracle.forward(oracle_frame(scene, mode, K), *arrays)
+    g = torch.Generator().manual_seed(7)
+    grad_image = torch.randn(3, scene.height, scene.width, generator=g)
+    want = oracle.backward(fwd, grad_image.numpy(), *arrays)
+
+    sg = scene.to(cuda)
+    fb = FrameBuffers(*sg.gaussians(), sg.settings(RasterizerMode(mode), K, scale_modifier=2.5), True, False, train=True)
+    image = fb.run_forward()
+    grads = fb.run_backward(grad_image.to(cuda))
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(u32(fb.n_touched), fwd["pre"]["n_touched"])        # scale_modifier is ignored in training
+    vis = fwd["pre"]["n_touched"] > 0                                                 # flags of culled Gaussians are never read
+    np.testing.assert_array_equal(fb.clamp_info.cpu().numpy()[:, vis], fwd["pre"]["clamp_info"][:, vis])
+    assert np.abs(image.cpu().numpy() - fwd["image"]).max() <= 1e-4
+    Keff = oracle.effective_k(K)
+    if mode in (0, 1):
+        np.testing.assert_array_equal(u32(fb.core_idx), fwd["core_idx"][:Keff])
+        np.testing.assert_allclose(fb.core_info.cpu().numpy(), fwd["core_info"][:Keff], rtol=1e-5, atol=1e-5)
+    if mode in (0, 3):
+        rows = 6 if mode == 0 else 5
+        np.testing.assert_allclose(fb.tail_info.cpu().numpy()[:rows], fwd["tail_info"][:rows], rtol=1e-5, atol=1e-6)
+    for name, got in zip(NAMES, grads):
+        assert_grad_close(name, got.cpu().numpy(), want[name])
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("rows,scaling", [(2, False), (3, True)])
+def test_autograd_function_and_densification_info(cuda, mode, rows, scaling):
+    print(f"case mode={mode} rows={rows} scaling={scaling}", flush=True)
+    scene = make_scene(0, 3000)
+    arrays = [t.numpy() for t in scene.gaussians()]
+    fwd = oracle.forward(oracle_frame(scene, mode, 4), *arrays)
+    grad_image = torch.randn(3, scene.height, scene.width, generator=torch.Generator().manual_seed(11))
+    info_ref = np.full((rows, 3000), 0.25, np.float32)
+    want = oracle.backward(fwd, grad_image.numpy(), *arrays, densification_info=info_ref, use_distance_scaling=scaling)
+
+    sg = scene.to(cuda)
+    leaves = [t.clone().requires_grad_(True) for t in sg.gaussians()]
+    info = torch.full((rows, 3000), 0.25, device=cuda)
+    image = diff_rasterize(*leaves, info, sg.settings(RasterizerMode(mode), 4), scaling)
+    assert image.shape == (3, scene.height, scene.width) and image.requires_grad and not info.requires_grad
+    (image * grad_image.to(cuda)).sum().backward()
+    torch.cuda.synchronize()
+    for name, leaf in zip(NAMES, leaves):
+        assert leaf.grad is not None and leaf.grad.shape == leaf.shape
+        assert_grad_close(name, leaf.grad.cpu().numpy(), want[name])
+    got_info = info.cpu().numpy()
+    np.testing.assert_array_equal(got_info[0], info_ref[0])
+    for r in range(1, rows):
+        np.testing.assert_allclose(got_info[r], info_ref[r], rtol=2e-3, atol=2e-4 * float(np.abs(info_ref[r]).max()))
+
+
+def test_no_densification_tensor_and_untouched_inputs(cuda):
+    scene = make_scene(0, 2000).to(cuda)
+    leaves = [t.clone().requires_grad_(True) for t in scene.gaussians()]
+    before = [t.detach().clone() for t in leaves]
+    image = diff_rasterize(*leaves, torch.empty(0, device=cuda), scene.settings(RasterizerMode.HYBRID_BLEND, 4), False)
+    image.sum().backward()
+    for a, b in zip(before, leaves):
+        assert torch.equal(a, b.detach())
+        assert torch.isfinite(b.grad).all()
