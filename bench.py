@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--mode", type=int, default=0)
     ap.add_argument("--K", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--train", action="store_true", help="time diff_rasterize forward + backward instead of rasterize")
     return ap.parse_args()
 
 
@@ -53,6 +54,53 @@ def event_ms(fn, reps):
         b.synchronize()
         out.append(a.elapsed_time(b))
     return out
+
+
+def bench_training(args, scene_cpu, scene, settings):
+    """One step = diff_rasterize forward + backward w.r.t. all six Gaussian tensors from a fixed upstream
+    gradient ~N(0,1).  Reported as milliseconds per step with the forward / backward split."""
+    import torch
+    from htgs_amd.torch_bindings import FrameBuffers
+    gauss = scene.gaussians()
+    grad_image = torch.randn(3, scene.height, scene.width, generator=torch.Generator().manual_seed(4)).to(gauss[0].device)
+
+    def step():
+        fb = FrameBuffers(*gauss, settings, True, False, train=True)
+        fb.run_forward()
+        return fb, fb.run_backward(grad_image)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    fb = FrameBuffers(*gauss, settings, True, False, train=True)
+    fb.run_forward()
+    fwd_blend = statistics.median(event_ms(fb.blend_forward, 10))
+    bwd = statistics.median(event_ms(lambda: fb.run_backward(grad_image), 10))
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        import oracle
+        fr = oracle.Frame(scene_cpu.M.numpy(), scene_cpu.VPM.numpy(), scene_cpu.cam_position.numpy(), args.mode, args.K,
+                          scene_cpu.active_sh_bases, scene_cpu.width, scene_cpu.height, scene_cpu.near_plane, scene_cpu.far_plane)
+        arrays = [t.numpy() for t in scene_cpu.gaussians()]
+        t0 = time.perf_counter()
+        fwd = oracle.forward(fr, *arrays)
+        oracle.backward(fwd, grad_image.cpu().numpy(), *arrays)
+        cpu_s = time.perf_counter() - t0
+        cpu_baseline = {"value": round(cpu_s * 1e3, 1), "unit": "ms/step", "cores": oracle.num_threads(), "kind": "port",
+                        "sample": "one whole forward + backward of the same workload; the C oracle's blend backward is single-threaded"}
+    print(json.dumps({
+        "metric": f"training step (diff_rasterize forward + backward) {MODE_NAMES[args.mode]} K={args.K}", "value": round(ms_per_step, 4),
+        "unit": "ms/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{scene.name} {MODE_NAMES[args.mode]} K={args.K} forward+backward, {fb.n} Gaussians, "
+                               f"{scene.width}x{scene.height}", "n_instances": fb.n_instances},
+        "stages": {"blend_forward_ms": round(fwd_blend, 4), "backward_ms": round(bwd, 4)},
+        "cpu_baseline": cpu_baseline}))
 
 
 def main():
@@ -75,6 +123,9 @@ def main():
     mode = RasterizerMode(args.mode)
     settings = scene.settings(mode, args.K)
     gauss = scene.gaussians()
+
+    if args.train:
+        return bench_training(args, scene_cpu, scene, settings)
 
     def step():
         return rasterize(*gauss, settings, True, False)
