@@ -76,21 +76,28 @@ __global__ void __launch_bounds__(kSortThreads) digit_scatter_kernel(
     const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
-    __shared__ uint32_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the output base
+    __shared__ uint32_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the wave's base inside the block
+    __shared__ uint32_t digit_start[kRadix];           // first slot of each digit in the block-local order
+    __shared__ uint32_t global_base[kRadix];           // where the block's run of each digit starts in the output
     __shared__ uint32_t wave_sums[kSortWaves];
+    __shared__ KeyT local_keys[kSortTile];             // the block's items, grouped by digit, stable
+    __shared__ uint32_t local_vals[kSortTile];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
 #pragma unroll
     for (int w = 0; w < kSortWaves; ++w) counts[w][threadIdx.x] = 0;
     __syncthreads();
 
-    const uint64_t wave_base = (uint64_t)blockIdx.x * kSortTile + (uint64_t)wave * (kWave * kSortItems);
+    const uint64_t block_base = (uint64_t)blockIdx.x * kSortTile;
+    const uint64_t wave_base = block_base + (uint64_t)wave * (kWave * kSortItems);
     KeyT key[kSortItems];
+    uint32_t val[kSortItems];
     uint32_t rank[kSortItems];
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const uint64_t i = wave_base + (uint64_t)r * kWave + lane;
         const bool valid = i < n;
         key[r] = valid ? keys_in[i] : (KeyT)0;
+        val[r] = valid ? vals_in[i] : 0u;
         const uint32_t d = digit_of(key[r], shift, mask);
         // lanes of this wave holding the same digit
         uint64_t peers = __ballot(valid);
@@ -110,23 +117,31 @@ __global__ void __launch_bounds__(kSortThreads) digit_scatter_kernel(
     }
     __syncthreads();
 
-    // output base of (wave, digit): global digit base + this block's offset inside the digit + earlier waves
+    // thread d owns digit d: block-local start of the digit, base of each wave inside it, global start of the run
     {
         const uint32_t d = threadIdx.x;
-        const uint32_t total = totals[d];
-        uint32_t inc = total;
+        uint32_t block_count = 0;
+#pragma unroll
+        for (int w = 0; w < kSortWaves; ++w) block_count += counts[w][d];
+        // exclusive scans over the 256 digits: of this block's counts (local order) and of the global totals
+        uint32_t inc_local = block_count, inc_global = totals[d];
+        const uint32_t total = inc_global;
 #pragma unroll
         for (int s = 1; s < kWave; s <<= 1) {
-            const uint32_t t = __shfl_up(inc, s, kWave);
-            if (lane >= s) inc += t;
+            const uint32_t tl = __shfl_up(inc_local, s, kWave), tg = __shfl_up(inc_global, s, kWave);
+            if (lane >= s) { inc_local += tl; inc_global += tg; }
         }
-        if (lane == kWave - 1) wave_sums[wave] = inc;
+        __shared__ uint32_t wave_sums_g[kSortWaves];
+        if (lane == kWave - 1) { wave_sums[wave] = inc_local; wave_sums_g[wave] = inc_global; }
         __syncthreads();
-        uint32_t before = 0;
+        uint32_t before_l = 0, before_g = 0;
 #pragma unroll
         for (int w = 0; w < kSortWaves; ++w)
-            if (w < wave) before += wave_sums[w];
-        uint32_t run = before + inc - total + hist[(size_t)d * n_blocks + blockIdx.x];
+            if (w < wave) { before_l += wave_sums[w]; before_g += wave_sums_g[w]; }
+        const uint32_t start = before_l + inc_local - block_count;
+        digit_start[d] = start;
+        global_base[d] = before_g + inc_global - total + hist[(size_t)d * n_blocks + blockIdx.x];
+        uint32_t run = start;
 #pragma unroll
         for (int w = 0; w < kSortWaves; ++w) {
             const uint32_t c = counts[w][d];
@@ -136,13 +151,28 @@ __global__ void __launch_bounds__(kSortThreads) digit_scatter_kernel(
     }
     __syncthreads();
 
+    // group the block's items by digit in LDS (stable), ...
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const uint64_t i = wave_base + (uint64_t)r * kWave + lane;
         if (i < n) {
             const uint32_t pos = counts[wave][digit_of(key[r], shift, mask)] + rank[r];
-            keys_out[pos] = key[r];
-            vals_out[pos] = vals_in[i];
+            local_keys[pos] = key[r];
+            local_vals[pos] = val[r];
+        }
+    }
+    __syncthreads();
+    // ... then stream them out: neighbouring threads write neighbouring addresses inside each digit's run
+    const uint32_t n_local = n - block_base < (uint64_t)kSortTile ? (uint32_t)(n - block_base) : (uint32_t)kSortTile;
+#pragma unroll
+    for (int r = 0; r < kSortItems; ++r) {
+        const uint32_t i = (uint32_t)r * kSortThreads + threadIdx.x;
+        if (i < n_local) {
+            const KeyT k = local_keys[i];
+            const uint32_t d = digit_of(k, shift, mask);
+            const uint32_t pos = global_base[d] + (i - digit_start[d]);
+            keys_out[pos] = k;
+            vals_out[pos] = local_vals[i];
         }
     }
 }

@@ -61,6 +61,37 @@ def _ptr(t: Optional[torch.Tensor]) -> int:
     return 0 if t is None or t.numel() == 0 else t.data_ptr()
 
 
+class ScratchPool:
+    """Grow-only device scratch that inference frames on one (device, stream) reuse, so that a steady stream of
+    ``rasterize`` calls allocates nothing but its outputs.  Work is ordered by the stream, which is what makes the
+    reuse safe; frames issued on another stream get another pool.  Training frames do not use it (their scratch
+    has to survive until backward)."""
+
+    _pools: dict = {}
+
+    def __init__(self):
+        self.buffers: dict = {}
+
+    @classmethod
+    def current(cls, device: torch.device) -> "ScratchPool":
+        key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+        pool = cls._pools.get(key)
+        if pool is None:
+            pool = cls._pools[key] = ScratchPool()
+        return pool
+
+    @classmethod
+    def clear(cls):
+        cls._pools.clear()
+
+    def get(self, name: str, numel: int, dtype: torch.dtype, device: torch.device, headroom: float = 0.0) -> torch.Tensor:
+        buf = self.buffers.get(name)
+        if buf is None or buf.dtype != dtype or buf.numel() < numel or buf.device != device:
+            buf = torch.empty(max(int(numel * (1.0 + headroom)), 1), dtype=dtype, device=device)
+            self.buffers[name] = buf
+        return buf
+
+
 class FrameBuffers:
     """One frame on the C ABI: validated inputs, caller-owned scratch, outputs.
 
@@ -71,7 +102,8 @@ class FrameBuffers:
     """
 
     def __init__(self, positions, scales, rotations, opacities, sh_0, sh_rest, settings: RasterizerSettings,
-                 to_chw: bool = True, use_median_depth: bool = False, train: bool = False):
+                 to_chw: bool = True, use_median_depth: bool = False, train: bool = False,
+                 pool: Optional[ScratchPool] = None):
         mode = _mode_value(settings.mode)
         if mode not in (0, 1, 2, 3):
             raise RuntimeError("unsupported rasterizer mode")
@@ -106,15 +138,15 @@ class FrameBuffers:
         self.end_bit = self.lib.htgs_end_bit(mode, self.width, self.height)
         self.to_chw = bool(to_chw)
 
-        u32 = dict(dtype=torch.int32, device=dev)
-        self.n_touched = torch.empty(n, **u32)
-        self.offsets = torch.empty(n, **u32)
-        self.bounds = torch.empty((n, 4), dtype=torch.int16, device=dev)
-        self.prim = torch.empty((n, _native.PRIM_FLOATS), dtype=torch.float32, device=dev)
+        self.pool = pool
+        self.n_touched = self._scratch("n_touched", n, torch.int32)[:n]
+        self.offsets = self._scratch("offsets", n, torch.int32)[:n]
+        self.bounds = self._scratch("bounds", 4 * n, torch.int16)[:4 * n].view(n, 4)
+        self.prim = self._scratch("prim", _native.PRIM_FLOATS * n, torch.float32)[:_native.PRIM_FLOATS * n].view(n, _native.PRIM_FLOATS)
         self.clamp_info = torch.empty((3, n), dtype=torch.uint8, device=dev) if train else None
-        self.scan_tmp = torch.empty(self.lib.htgs_scan_tmp_words(n), **u32)
-        self.n_instances_dev = torch.zeros(1, **u32)
-        self.ranges = torch.empty((self.n_tiles, 2), **u32)
+        self.scan_tmp = self._scratch("scan_tmp", self.lib.htgs_scan_tmp_words(n), torch.int32)
+        self.n_instances_dev = self._scratch("n_instances_dev", 1, torch.int32)    # written by the scan
+        self.ranges = self._scratch("ranges", 2 * self.n_tiles, torch.int32)[:2 * self.n_tiles].view(self.n_tiles, 2)
         self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
                                  dtype=torch.float32, device=dev)
         self.depth = torch.empty((self.height, self.width), dtype=torch.float32, device=dev)
@@ -145,6 +177,12 @@ class FrameBuffers:
         self.frame = f
         self._ref = ctypes.byref(f)
 
+    def _scratch(self, name: str, numel: int, dtype: torch.dtype, headroom: float = 0.0) -> torch.Tensor:
+        """A buffer of at least ``numel`` elements: from the pool if the frame has one, else freshly allocated."""
+        if self.pool is not None:
+            return self.pool.get(name, numel, dtype, self.device, headroom)
+        return torch.empty(max(int(numel), 1), dtype=dtype, device=self.device)
+
     # ---- stages -----------------------------------------------------------------------------
     def preprocess(self):
         _native.check(self.lib.htgs_preprocess(self._ref))
@@ -165,9 +203,10 @@ class FrameBuffers:
         self.n_instances = int(n_instances)
         key_dtype = {2: torch.int16, 4: torch.int32, 8: torch.int64}[self.key_bytes]
         m = max(self.n_instances, 1)
-        self.keys = [torch.empty(m, dtype=key_dtype, device=dev) for _ in range(2)]
-        self.vals = [torch.empty(m, dtype=torch.int32, device=dev) for _ in range(2)]
-        self.sort_tmp = torch.empty(self.lib.htgs_sort_tmp_words(self.n_instances), dtype=torch.int32, device=dev)
+        # pooled frames keep 1/8 headroom so that a slowly changing instance count does not reallocate every frame
+        self.keys = [self._scratch(f"keys{i}_{self.key_bytes}", m, key_dtype, 0.125) for i in range(2)]
+        self.vals = [self._scratch(f"vals{i}", m, torch.int32, 0.125) for i in range(2)]
+        self.sort_tmp = self._scratch("sort_tmp", self.lib.htgs_sort_tmp_words(self.n_instances), torch.int32, 0.125)
         f = self.frame
         f.n_instances = self.n_instances
         f.keys[0], f.keys[1] = _ptr(self.keys[0]), _ptr(self.keys[1])
@@ -324,7 +363,8 @@ def rasterize(
     """Inference render: ``(image, depth)`` with ``image`` ``[3,H,W]`` (``to_chw``) or ``[H,W,3]`` clamped to
     [0,1] and ``depth`` ``[1,H,W]`` / ``[H,W,1]`` (reference: rasterization.py:140-163)."""
     with torch.no_grad():
+        pool = ScratchPool.current(positions.device) if isinstance(positions, torch.Tensor) and positions.is_cuda else None
         image, depth = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, settings,
-                                    to_chw, use_median_depth).run()
+                                    to_chw, use_median_depth, pool=pool).run()
     depth = depth.unsqueeze(0) if to_chw else depth.unsqueeze(-1)
     return image, depth
