@@ -62,17 +62,20 @@ __device__ __forceinline__ void atomic_add_nonzero(float *p, float v)
 }
 
 // ---------------------------------------------------------------------------------------------
-// HYBRID_BLEND (K >= 1) and OIT_BLEND (K == 0): one lane per Gaussian of the staged batch, all lanes walk the
-// 64 pixels of the tile together (per-pixel terms are LDS broadcasts), 16 atomics per (Gaussian, tile).
+// HYBRID_BLEND (K >= 1), OIT_BLEND (K == 0) and ALPHA_BLEND_FIRST_K (core only, no tail): one lane per Gaussian
+// of the staged batch, all lanes walk the 64 pixels of the tile together (per-pixel terms are LDS broadcasts),
+// 16 atomics per (Gaussian, tile).  The reference's FIRST_K backward runs one thread per stored fragment with
+// ~20 atomics each (R/include/alpha_blend_first_k/kernels/backward.cuh:60-206); walking the tile's list and
+// looking each (Gaussian, pixel) up in the stored core visits the same fragments.
 // ---------------------------------------------------------------------------------------------
-template <int K>
+template <int K, int MODE>
 __global__ void __launch_bounds__(64) blend_tail_backward_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
     const float *__restrict__ grad_image, const float *__restrict__ VPM, float *__restrict__ grad_acc, float *__restrict__ helper,
     uint32_t n, uint32_t width, uint32_t height, uint32_t grid_w)
 {
-    constexpr int MODE = K > 0 ? HTGS_MODE_HYBRID_BLEND : HTGS_MODE_OIT_BLEND;
+    constexpr bool kHasTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = K > 0 ? K : 1;
     __shared__ uint32_t s_idx[64 * KS];      // [pixel][slot]
     __shared__ float4 s_core[64 * KS];       // (weight * g, dC/dalpha . g)
@@ -89,8 +92,8 @@ __global__ void __launch_bounds__(64) blend_tail_backward_kernel(
         const bool inside = x < width && y < height;
         const size_t pix = inside ? (size_t)width * y + x : 0;
         float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f;
-        if (inside) {
-            g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix];
+        if (inside) { g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix]; }
+        if (inside && kHasTail) {
             const float r0 = tail_info[pix], r1 = tail_info[np + pix], r2 = tail_info[2 * np + pix];
             const float asr = tail_info[3 * np + pix], T_tail = tail_info[4 * np + pix], T_core = tail_info[5 * np + pix];
             const float w_tail = T_core * asr;                                   // backward.cuh:166
@@ -146,6 +149,7 @@ __global__ void __launch_bounds__(64) blend_tail_backward_kernel(
                 for (int i = 0; i < KS; ++i)
                     if (s_idx[p * KS + i] == g) slot = i;                        // :231-235
             }
+            if (!kHasTail && slot < 0) continue;                                   // FIRST_K: only stored fragments carry gradient
             float dL_dalpha;
             if (slot >= 0) {
                 const float4 c = s_core[p * KS + slot];
@@ -172,45 +176,6 @@ __global__ void __launch_bounds__(64) blend_tail_backward_kernel(
             if (helper) atomic_add_nonzero(helper + g, help);
         }
     }
-}
-
-// ---------------------------------------------------------------------------------------------
-// ALPHA_BLEND_FIRST_K: one thread per stored core fragment (slot, pixel), backward.cuh:81-205
-// ---------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) blend_first_k_backward_kernel(
-    const float4 *__restrict__ prim, const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info,
-    const float *__restrict__ grad_image, const float *__restrict__ VPM, float *__restrict__ grad_acc, float *__restrict__ helper,
-    uint32_t n, uint32_t width, size_t np, size_t n_fragments)
-{
-    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (tid >= n_fragments) return;
-    const uint32_t g = core_idx[tid];
-    if (g == 0xffffffffu) return;
-    const size_t pix = tid % np;
-    const float fx = (float)(uint32_t)(pix % width), fy = (float)(uint32_t)(pix / width);
-    const float g0 = grad_image[pix], g1 = grad_image[np + pix], g2 = grad_image[2 * np + pix];
-    const float4 info = core_info[tid];
-    atomic_add_nonzero(grad_acc + g, info.w * g0);
-    atomic_add_nonzero(grad_acc + (size_t)n + g, info.w * g1);
-    atomic_add_nonzero(grad_acc + 2 * (size_t)n + g, info.w * g2);
-    const float dL_dalpha = info.x * g0 + info.y * g1 + info.z * g2;
-    if (dL_dalpha == 0.0f) return;
-    const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
-    Frag f;
-    frag_cutoff<HTGS_MODE_ALPHA_BLEND_FIRST_K>(rec[0], rec[1], rec[2], fx, fy, f);   // stored fragments passed it in forward
-    f.den_rcp = 1.0f / f.den;
-    const float opacity = rec[4].w;
-    f.G = d_expf((-0.5f * f.num) * f.den_rcp);
-    FragGrads fg;
-    fragment_backward(f, opacity, dL_dalpha, fx, fy, fg);
-    atomic_add_nonzero(grad_acc + 3 * (size_t)n + g, fg.opacity);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        atomic_add_nonzero(grad_acc + (size_t)(4 + k) * n + g, fg.dV1[k]);
-        atomic_add_nonzero(grad_acc + (size_t)(8 + k) * n + g, fg.dV2[k]);
-        atomic_add_nonzero(grad_acc + (size_t)(12 + k) * n + g, fg.dV4[k]);
-    }
-    if (helper) atomic_add_nonzero(helper + g, position_grad_l1(VPM, fg));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -458,10 +423,10 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
     }
 }
 
-template <int K>
+template <int K, int MODE>
 static void launch_tail_backward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
 {
-    hipLaunchKernelGGL((blend_tail_backward_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
+    hipLaunchKernelGGL((blend_tail_backward_kernel<K, MODE>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
                        (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image, f->VPM,
                        f->grad_acc, f->dens_helper, (uint32_t)f->n_primitives, (uint32_t)f->width, (uint32_t)f->height, grid_w);
 }
@@ -491,24 +456,27 @@ extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
     switch (f->mode) {
         case HTGS_MODE_HYBRID_BLEND:
             switch (K) {
-                case 32: launch_tail_backward<32>(f, selector, grid_w, n_tiles); break;
-                case 16: launch_tail_backward<16>(f, selector, grid_w, n_tiles); break;
-                case 8: launch_tail_backward<8>(f, selector, grid_w, n_tiles); break;
-                case 4: launch_tail_backward<4>(f, selector, grid_w, n_tiles); break;
-                case 2: launch_tail_backward<2>(f, selector, grid_w, n_tiles); break;
-                default: launch_tail_backward<1>(f, selector, grid_w, n_tiles); break;
+                case 32: launch_tail_backward<32, HTGS_MODE_HYBRID_BLEND>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_tail_backward<16, HTGS_MODE_HYBRID_BLEND>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_tail_backward<8, HTGS_MODE_HYBRID_BLEND>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_tail_backward<4, HTGS_MODE_HYBRID_BLEND>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_tail_backward<2, HTGS_MODE_HYBRID_BLEND>(f, selector, grid_w, n_tiles); break;
+                default: launch_tail_backward<1, HTGS_MODE_HYBRID_BLEND>(f, selector, grid_w, n_tiles); break;
             }
             break;
         case HTGS_MODE_OIT_BLEND:
-            launch_tail_backward<0>(f, selector, grid_w, n_tiles);
+            launch_tail_backward<0, HTGS_MODE_OIT_BLEND>(f, selector, grid_w, n_tiles);
             break;
-        case HTGS_MODE_ALPHA_BLEND_FIRST_K: {
-            const size_t np = (size_t)f->width * f->height, n_frag = np * (size_t)K;
-            hipLaunchKernelGGL(blend_first_k_backward_kernel, dim3((unsigned)((n_frag + 255) / 256)), dim3(256), 0, s,
-                               (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->grad_image, f->VPM, f->grad_acc,
-                               f->dens_helper, (uint32_t)f->n_primitives, (uint32_t)f->width, np, n_frag);
+        case HTGS_MODE_ALPHA_BLEND_FIRST_K:
+            switch (K) {
+                case 32: launch_tail_backward<32, HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_tail_backward<16, HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_tail_backward<8, HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_tail_backward<4, HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_tail_backward<2, HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, grid_w, n_tiles); break;
+                default: launch_tail_backward<1, HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, grid_w, n_tiles); break;
+            }
             break;
-        }
         default:
             hipLaunchKernelGGL(blend_global_backward_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
                                (const float4 *)f->prim, f->image, f->grad_image, f->VPM, f->grad_acc, f->dens_helper,
