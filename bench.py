@@ -39,6 +39,8 @@ def parse_args():
     ap.add_argument("--mode", type=int, default=0)
     ap.add_argument("--K", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="only run the plain 1 GiB copy kernel a few times (reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--train", action="store_true", help="time diff_rasterize forward + backward instead of rasterize")
     return ap.parse_args()
 
@@ -118,6 +120,16 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate:
+        from htgs_amd import _native
+        n_bytes = 1 << 30                      # larger than the 256 MB memory-side cache: both streams come from HBM
+        src = torch.empty(n_bytes // 4, dtype=torch.float32, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            _native.check(_native.lib().htgs_copy_bytes(dst.data_ptr(), src.data_ptr(), n_bytes, torch.cuda.current_stream(dev).cuda_stream))
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "copy_bytes_kernel", "bytes_read": n_bytes, "bytes_written": n_bytes, "launches": 5}))
+        return
     scene_cpu = make_scene(args.config, args.n)
     scene = scene_cpu.to(dev)
     mode = RasterizerMode(args.mode)

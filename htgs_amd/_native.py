@@ -96,6 +96,7 @@ SYMBOLS = {
     "htgs_blend_backward": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
     "htgs_preprocess_backward": (ctypes.c_int, [_FRAME_P]),
     "htgs_backward": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
+    "htgs_copy_bytes": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
 }
 
 _lib = None

@@ -34,9 +34,26 @@ static int bit_width(uint32_t n)
     return b;
 }
 
+__global__ void __launch_bounds__(256) copy_bytes_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 }  // namespace htgs
 
 using namespace htgs;
+
+extern "C" int htgs_copy_bytes(void *dst, const void *src, size_t n_bytes, void *stream)
+{
+    if (!dst || !src || (n_bytes & 15)) return fail(HTGS_ERR_ARGUMENT, "htgs_copy_bytes: null pointer or size not a multiple of 16");
+    const size_t n = n_bytes / 16;
+    if (n == 0) return HTGS_OK;
+    if ((n + 255) / 256 > 0x7fffffffull) return fail(HTGS_ERR_ARGUMENT, "htgs_copy_bytes: too large");
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4 *)src, (uint4 *)dst, n);
+    return check_launch("copy_bytes");
+}
 
 extern "C" const char *htgs_last_error(void) { return g_error; }
 

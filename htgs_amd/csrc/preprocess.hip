@@ -65,8 +65,15 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
     int n, uint32_t grid_w, uint32_t grid_h, float tile, float min_alpha_rcp,
     int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier)
 {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+    // One LDS buffer, used twice: first the block's slice of sh_rest (contiguous in memory, loaded with coalesced
+    // 16-byte reads and then read back per Gaussian at a stride of 3 * total_sh words), then the block's 80-byte
+    // records, written back as one contiguous run of 16-byte stores.
+    extern __shared__ float4 lds4[];
+    float *lds = reinterpret_cast<float *>(lds4);
+    __shared__ uint8_t s_visible[256];
+    const int first = blockIdx.x * 256;
+    const int i = first + threadIdx.x;
+    const bool in_range = i < n;
 
     // camera: uniform addresses, the compiler turns these into scalar loads
     float M3[4], VPM[16], cam[3];
@@ -78,10 +85,11 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
     for (int k = 0; k < 3; ++k) cam[k] = cam_position[k];
 
     uint32_t touched = 0;
-    const float p[3] = { positions[3 * (size_t)i], positions[3 * (size_t)i + 1], positions[3 * (size_t)i + 2] };
-    const float opacity = opacities[i];
+    const size_t ic = in_range ? (size_t)i : 0;
+    const float p[3] = { positions[3 * ic], positions[3 * ic + 1], positions[3 * ic + 2] };
+    const float opacity = opacities[ic];
     const float z = dot3(M3, p[0], p[1], p[2]) + M3[3];                                   // kernel_utils.cuh:89
-    bool visible = !(z < near_plane || z > far_plane);                                    // :90
+    bool visible = in_range && !(z < near_plane || z > far_plane);                        // :90
     float u[3], v[3], w[3];
     Row V1, V2, V4;
     uint32_t b0 = 0, b1 = 0, b2 = 0, b3 = 0;
@@ -124,17 +132,30 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
             }
         }
     }
-    n_touched[i] = touched;
-    if (!visible) return;
+    if (in_range) n_touched[i] = touched;
+    s_visible[threadIdx.x] = visible;
+    if (visible)
+        *reinterpret_cast<ushort4 *>(bounds + 4 * (size_t)i) = make_ushort4((uint16_t)b0, (uint16_t)b1, (uint16_t)b2, (uint16_t)b3);
 
-    *reinterpret_cast<ushort4 *>(bounds + 4 * (size_t)i) = make_ushort4((uint16_t)b0, (uint16_t)b1, (uint16_t)b2, (uint16_t)b3);
+    // stage the block's SH coefficients
+    const int per = 3 * total_sh;                                  // words per Gaussian
+    const int n_block = n - first < 256 ? n - first : 256;
+    if (active_sh > 1) {
+        const size_t base_word = (size_t)first * per;             // multiple of 256 words: 16-byte aligned
+        const int words = n_block * per;
+        const float4 *src4 = reinterpret_cast<const float4 *>(sh_rest + base_word);
+        for (int q = threadIdx.x; q < words / 4; q += 256) lds4[q] = src4[q];
+        for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) lds[q] = sh_rest[base_word + q];
+    }
+    __syncthreads();
 
     // view-dependent colour, kernel_utils.cuh:152-187
-    float res[3];
+    float res[3] = { 0.0f, 0.0f, 0.0f };
+    if (visible) {
 #pragma unroll
     for (int k = 0; k < 3; ++k) res[k] = 0.5f + 0.28209479177387814f * sh_0[3 * (size_t)i + k];
     if (active_sh > 1) {
-        const float *c = sh_rest + 3 * (size_t)total_sh * (size_t)i;
+        const float *c = lds + per * threadIdx.x;
         const float dx = p[0] - cam[0], dy = p[1] - cam[1], dz = p[2] - cam[2];
         const float inv = 1.0f / __builtin_sqrtf(dx * dx + dy * dy + dz * dz);
         const float x = dx * inv, y = dy * inv, zd = dz * inv;
@@ -172,13 +193,21 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
         clamp_info[(size_t)n + i] = res[1] < 0.0f;
         clamp_info[2 * (size_t)n + i] = res[2] < 0.0f;
     }
+    }
+    __syncthreads();                                               // everyone is done reading the coefficients
 
-    float4 *rec = reinterpret_cast<float4 *>(prim + (size_t)HTGS_PRIM_FLOATS * i);
-    rec[0] = make_float4(V1.x, V1.y, V1.z, V1.w);
-    rec[1] = make_float4(V2.x, V2.y, V2.z, V2.w);
-    rec[2] = make_float4(V4.x, V4.y, V4.z, V4.w);
-    rec[3] = make_float4(dot3(M3, u[0], u[1], u[2]), dot3(M3, v[0], v[1], v[2]), dot3(M3, w[0], w[1], w[2]), z);
-    rec[4] = make_float4(clamp_pos(res[0]), clamp_pos(res[1]), clamp_pos(res[2]), opacity);
+    if (visible) {
+        float4 *rec = lds4 + (HTGS_PRIM_FLOATS / 4) * threadIdx.x;
+        rec[0] = make_float4(V1.x, V1.y, V1.z, V1.w);
+        rec[1] = make_float4(V2.x, V2.y, V2.z, V2.w);
+        rec[2] = make_float4(V4.x, V4.y, V4.z, V4.w);
+        rec[3] = make_float4(dot3(M3, u[0], u[1], u[2]), dot3(M3, v[0], v[1], v[2]), dot3(M3, w[0], w[1], w[2]), z);
+        rec[4] = make_float4(clamp_pos(res[0]), clamp_pos(res[1]), clamp_pos(res[2]), opacity);
+    }
+    __syncthreads();
+    float4 *dst4 = reinterpret_cast<float4 *>(prim + (size_t)HTGS_PRIM_FLOATS * first);
+    for (int q = threadIdx.x; q < n_block * (HTGS_PRIM_FLOATS / 4); q += 256)
+        if (s_visible[q / (HTGS_PRIM_FLOATS / 4)]) dst4[q] = lds4[q];
 }
 
 }  // namespace htgs
@@ -202,7 +231,11 @@ extern "C" int htgs_preprocess(const htgs_frame *f)
     const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
     if (grid_w > 65535u || grid_h > 65535u) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: image too large for 16-bit tile bounds");
     const float min_alpha_rcp = f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K ? 20.0f : 255.0f;
-    hipLaunchKernelGGL(preprocess_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), 0, (hipStream_t)f->stream,
+    // dynamic LDS: the larger of the block's SH coefficients (256 x 3 x total_sh words) and its records (256 x 80 bytes)
+    const size_t sh_bytes = f->active_sh_bases > 1 ? (size_t)256 * 3 * f->total_sh_bases * sizeof(float) : 0;
+    const size_t lds_bytes = sh_bytes > 256 * HTGS_PRIM_FLOATS * sizeof(float) ? sh_bytes : 256 * HTGS_PRIM_FLOATS * sizeof(float);
+    if (lds_bytes > 64 * 1024) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: sh_rest has more than 21 coefficients per Gaussian");
+    hipLaunchKernelGGL(preprocess_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), lds_bytes, (hipStream_t)f->stream,
                        f->positions, f->scales, f->rotations, f->opacities, f->sh_0, f->sh_rest, f->M, f->VPM, f->cam_position,
                        f->n_touched, f->bounds, f->prim, f->clamp_info, f->n_primitives, grid_w, grid_h, (float)tile,
                        min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier);

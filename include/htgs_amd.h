@@ -154,6 +154,11 @@ int htgs_preprocess_backward(const htgs_frame *f);
 /* <mode>::backward (R/src/hybrid_blend/backward.cu:26-128): blend backward, then preprocess backward */
 int htgs_backward(const htgs_frame *f, int selector);
 
+/* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes (multiple of 16)
+ * with one 16-byte load and store per thread.  Hardware counters read on it calibrate the same counters read on
+ * the rasterizer's kernels (bench.py --calibrate). */
+int htgs_copy_bytes(void *dst, const void *src, size_t n_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
