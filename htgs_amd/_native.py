@@ -57,6 +57,7 @@ class Frame(ctypes.Structure):
         ("core_info", ctypes.c_void_p),
         ("tail_info", ctypes.c_void_p),
         ("grad_image", ctypes.c_void_p),
+        ("grad_rows", ctypes.c_void_p),
         ("grad_acc", ctypes.c_void_p),
         ("dens_helper", ctypes.c_void_p),
         ("grad_positions", ctypes.c_void_p),

@@ -86,8 +86,11 @@ typedef struct htgs_frame {
     float *tail_info;          /* [6,P] sum alpha*rgb (3), 1/sum alpha, T_tail, T_core       (modes 0, 3) */
     /* ---- training: backward (backward_wrapper, rasterization_api.cu:178-363) ---- */
     const float *grad_image;   /* [3,H,W] upstream gradient */
-    float *grad_acc;           /* [16,N] zero-filled by the caller: dL/drgb (3), dL/dopacity, dL/dVPMT1, 2, 4 (4 each) */
-    float *dens_helper;        /* [N] zero-filled, sum over fragments of |dL/dposition|_1; NULL unless 3-row densification */
+    float *grad_rows;          /* modes 0, 1, 3: [I,16] one row per instance, in creation order: dL/drgb (3), dL/dopacity,
+                                  dL/dVPMT1, 2, 4 (4 each); every row is written, no initialisation needed */
+    float *grad_acc;           /* mode 2: [16,N] the same 16 sums per Gaussian, zero-filled by the caller (atomics) */
+    float *dens_helper;        /* sum over fragments of |dL/dposition|_1: [I] per instance (modes 0, 1, 3) or [N] zero-filled
+                                  (mode 2); NULL unless densification_rows == 3 */
     float *grad_positions;     /* [N,3] outputs; every element is written */
     float *grad_scales;        /* [N,3] */
     float *grad_rotations;     /* [N,4] */
