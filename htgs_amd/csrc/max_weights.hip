@@ -1,0 +1,211 @@
+// Per-Gaussian maximum blending weight of a view (used by the reference's importance-based pruning).
+// Restates update_max_weights_cu of R/include/hybrid_blend/kernels/update_max_weights.cuh:59-212,
+// R/include/alpha_blend_first_k/kernels/update_max_weights.cuh:59-161,
+// R/include/alpha_blend_global_ordering/kernels/update_max_weights.cuh:59-131 and
+// R/include/oit_blend/kernels/update_max_weights.cuh:58-165.  The maximum is taken on the bit patterns of the
+// (non-negative) weights with integer atomicMax, which makes the result independent of the order of arrival.
+#include "blend_common.h"
+
+namespace htgs {
+
+__device__ __forceinline__ void raise_max(uint32_t *__restrict__ max_weights, uint32_t g, float w)
+{
+    if (g == 0xffffffffu) return;
+    const uint32_t bits = float_to_bits(w);
+    if (max_weights[g] < bits) atomicMax(max_weights + g, bits);
+}
+
+// HYBRID_BLEND (TAIL = true, CORE = true), ALPHA_BLEND_FIRST_K (CORE only), OIT_BLEND (TAIL only, K unused)
+template <int K, int MODE>
+__global__ void __launch_bounds__(64) max_weights_tile_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold)
+{
+    constexpr bool kCore = MODE != HTGS_MODE_OIT_BLEND;
+    constexpr bool kTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
+    constexpr int KS = kCore ? K : 1;
+    __shared__ Stage<64> st;
+    __shared__ uint32_t st_idx[64];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+
+    float alpha_sum = 0.0f, T_tail = 1.0f;
+    float ca[KS], cd[KS];
+    uint32_t ci[KS];
+#pragma unroll
+    for (int i = 0; i < KS; ++i) { ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        __syncthreads();
+        const int nb = last - base < 64u ? (int)(last - base) : 64;
+        for (int j = 0; j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            float depth = 0.0f;
+            if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
+                depth = frag_depth(st.mt3[j], f);
+                if (depth >= cd[KS - 1]) continue;
+            }
+            if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+            float alpha = f.alpha;
+            if (MODE == HTGS_MODE_HYBRID_BLEND) depth = frag_depth(st.mt3[j], f);
+            if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
+                uint32_t idx = st_idx[j];
+#pragma unroll
+                for (int i = 0; i < KS; ++i) {
+                    if (depth < cd[i]) {
+                        vswap(depth, cd[i]);
+                        vswap(alpha, ca[i]);
+                        vswap(idx, ci[i]);
+                    }
+                }
+            }
+            if (kTail) { alpha_sum += alpha; T_tail *= 1.0f - alpha; }
+        }
+    }
+    float T_core = 1.0f;
+    if (kCore && inside) {
+#pragma unroll
+        for (int i = 0; i < KS; ++i) {
+            const float w = T_core * ca[i];
+            T_core *= 1.0f - ca[i];
+            if (T_core < kTransmittanceThreshold) T_core = 0.0f;
+            if (!(w < weight_threshold)) raise_max(max_weights, ci[i], w);
+        }
+    }
+    if (!kTail) return;
+    float tail_weight = 0.0f;
+    if (inside && alpha_sum >= weight_threshold) tail_weight = (T_core * (1.0f - T_tail)) * (1.0f / alpha_sum);
+    const bool active = inside && tail_weight >= weight_threshold;
+    if (!__any(active)) return;
+    // second walk over the tile's list: alpha * tail weight for every fragment that passes the cut-off
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        __syncthreads();
+        const int nb = last - base < 64u ? (int)(last - base) : 64;
+        for (int j = 0; j < nb; ++j) {
+            Frag f;
+            if (!active || !frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            const float G = d_expf((-0.5f * f.num) * f.den_rcp);
+            const float a = st.col[j].w * G;
+            const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
+            if (!(w < weight_threshold)) raise_max(max_weights, st_idx[j], w);
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) max_weights_global_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
+    __shared__ Stage<256> st;
+    __shared__ uint32_t st_idx[256];
+    const uint32_t tile = blockIdx.x;
+    const uint32_t t = threadIdx.x;
+    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
+    const bool inside = x < width && y < height;
+    const float fx = (float)x, fy = (float)y;
+    float T = 1.0f;
+    bool done = !inside;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 256) {
+        if (__syncthreads_count(done) == 256) break;
+        stage_load(st, prim, inst, base + t, last, t, st_idx);
+        __syncthreads();
+        const int nb = last - base < 256u ? (int)(last - base) : 256;
+        for (int j = 0; !done && j < nb; ++j) {
+            Frag f;
+            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
+            f.den_rcp = 1.0f / f.den;
+            if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+            const float w = T * f.alpha;
+            T *= 1.0f - f.alpha;
+            if (T < kTransmittanceThreshold) done = true;
+            if (!(w < weight_threshold)) raise_max(max_weights, st_idx[j], w);
+        }
+    }
+}
+
+template <int K, int MODE>
+static void launch_tile(const htgs_frame *f, int sel, uint32_t *max_weights, float thr, uint32_t grid_w, uint32_t n_tiles)
+{
+    hipLaunchKernelGGL((max_weights_tile_kernel<K, MODE>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
+                       (const float4 *)f->prim, max_weights, (uint32_t)f->width, (uint32_t)f->height, grid_w, thr);
+}
+
+template <int MODE>
+static void dispatch_tile(const htgs_frame *f, int sel, uint32_t *mw, float thr, uint32_t grid_w, uint32_t n_tiles)
+{
+    switch (htgs_effective_k(f->K)) {
+        case 32: launch_tile<32, MODE>(f, sel, mw, thr, grid_w, n_tiles); break;
+        case 16: launch_tile<16, MODE>(f, sel, mw, thr, grid_w, n_tiles); break;
+        case 8: launch_tile<8, MODE>(f, sel, mw, thr, grid_w, n_tiles); break;
+        case 4: launch_tile<4, MODE>(f, sel, mw, thr, grid_w, n_tiles); break;
+        case 2: launch_tile<2, MODE>(f, sel, mw, thr, grid_w, n_tiles); break;
+        default: launch_tile<1, MODE>(f, sel, mw, thr, grid_w, n_tiles); break;
+    }
+}
+
+}  // namespace htgs
+
+using namespace htgs;
+
+extern "C" int htgs_max_weights_front(const htgs_frame *f)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_front: null frame");
+    htgs_frame t = *f;
+    t.scale_modifier = 1.0f;      // update_max_weights.cuh:46: the scale modifier is not applied
+    t.sh_0 = nullptr;             // no colours
+    t.sh_rest = nullptr;
+    t.active_sh_bases = 1;
+    t.total_sh_bases = 0;
+    t.clamp_info = nullptr;
+    int rc = htgs_preprocess(&t);
+    if (rc != HTGS_OK) return rc;
+    return htgs_scan_offsets(&t);
+}
+
+extern "C" int htgs_max_weights_blend(const htgs_frame *f, int selector, float *max_weights, float weight_threshold)
+{
+    if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: null frame");
+    if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
+    if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: bad argument");
+    if (f->n_instances == 0 || f->n_primitives == 0) return HTGS_OK;
+    if (!f->ranges || !f->vals[selector] || !f->prim || !max_weights) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: null pointer");
+    const int tile = tile_size(f->mode);
+    const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
+    const uint32_t n_tiles = grid_w * grid_h;
+    uint32_t *mw = reinterpret_cast<uint32_t *>(max_weights);
+    switch (f->mode) {
+        case HTGS_MODE_HYBRID_BLEND: dispatch_tile<HTGS_MODE_HYBRID_BLEND>(f, selector, mw, weight_threshold, grid_w, n_tiles); break;
+        case HTGS_MODE_ALPHA_BLEND_FIRST_K: dispatch_tile<HTGS_MODE_ALPHA_BLEND_FIRST_K>(f, selector, mw, weight_threshold, grid_w, n_tiles); break;
+        case HTGS_MODE_OIT_BLEND: launch_tile<1, HTGS_MODE_OIT_BLEND>(f, selector, mw, weight_threshold, grid_w, n_tiles); break;
+        default:
+            hipLaunchKernelGGL(max_weights_global_kernel, dim3(n_tiles), dim3(256), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                               (const float4 *)f->prim, mw, (uint32_t)f->width, (uint32_t)f->height, grid_w, weight_threshold);
+            break;
+    }
+    return check_launch("max_weights");
+}
+
+extern "C" int htgs_max_weights_back(const htgs_frame *f, float *max_weights, float weight_threshold)
+{
+    int selector = 0;
+    int rc = htgs_create_instances(f);
+    if (rc != HTGS_OK) return rc;
+    rc = htgs_sort_instances(f, &selector);
+    if (rc != HTGS_OK) return rc;
+    rc = htgs_extract_ranges(f, selector);
+    if (rc != HTGS_OK) return rc;
+    return htgs_max_weights_blend(f, selector, max_weights, weight_threshold);
+}

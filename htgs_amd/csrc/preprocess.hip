@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
 
     // view-dependent colour, kernel_utils.cuh:152-187
     float res[3] = { 0.0f, 0.0f, 0.0f };
-    if (visible) {
+    if (visible && sh_0) {                                         // no colour without coefficients (max-weights pass)
 #pragma unroll
     for (int k = 0; k < 3; ++k) res[k] = 0.5f + 0.28209479177387814f * sh_0[3 * (size_t)i + k];
     if (active_sh > 1) {
@@ -220,7 +220,7 @@ extern "C" int htgs_preprocess(const htgs_frame *f)
     if (f->n_primitives < 0 || f->width <= 0 || f->height <= 0 || f->total_sh_bases < 0)
         return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: bad sizes");
     if (f->n_primitives == 0) return HTGS_OK;
-    if (!f->positions || !f->scales || !f->rotations || !f->opacities || !f->sh_0 || !f->M || !f->VPM ||
+    if (!f->positions || !f->scales || !f->rotations || !f->opacities || !f->M || !f->VPM ||
         !f->cam_position || !f->n_touched || !f->bounds || !f->prim)
         return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: null pointer");
     // the SH bands read from sh_rest must exist: 3, 8 and 15 coefficients for degrees 1, 2, 3

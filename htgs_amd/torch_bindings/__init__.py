@@ -1,3 +1,3 @@
-from .rasterization import diff_rasterize, rasterize, RasterizerSettings, RasterizerMode, FrameBuffers
+from .rasterization import diff_rasterize, rasterize, update_max_weights, RasterizerSettings, RasterizerMode, FrameBuffers
 
-__all__ = ['diff_rasterize', 'rasterize', 'RasterizerSettings', 'RasterizerMode', 'FrameBuffers']
+__all__ = ['diff_rasterize', 'rasterize', 'update_max_weights', 'RasterizerSettings', 'RasterizerMode', 'FrameBuffers']

@@ -115,14 +115,15 @@ class FrameBuffers:
         self.scales = _dev_f32(scales, "scales", dev)
         self.rotations = _dev_f32(rotations, "rotations", dev)
         self.opacities = _dev_f32(opacities, "opacities", dev)
-        self.sh_0 = _dev_f32(sh_0, "sh_0", dev)
-        self.sh_rest = _dev_f32(sh_rest, "sh_rest", dev)
+        # sh_0 / sh_rest may be None for the passes that compute no colour (update_max_weights)
+        self.sh_0 = _dev_f32(sh_0, "sh_0", dev) if sh_0 is not None else None
+        self.sh_rest = _dev_f32(sh_rest, "sh_rest", dev) if sh_rest is not None else torch.empty((positions.shape[0], 0, 3), dtype=torch.float32, device=dev)
         self.M = _dev_f32(settings.M, "settings.M", dev)
         self.VPM = _dev_f32(settings.VPM, "settings.VPM", dev)
         self.cam_position = _dev_f32(settings.cam_position, "settings.cam_position", dev)
         n = positions.shape[0]
         if positions.shape != (n, 3) or self.scales.shape != (n, 3) or self.rotations.shape != (n, 4) \
-                or self.opacities.numel() != n or self.sh_0.numel() != 3 * n or self.sh_rest.dim() != 3 \
+                or self.opacities.numel() != n or (self.sh_0 is not None and self.sh_0.numel() != 3 * n) or self.sh_rest.dim() != 3 \
                 or self.sh_rest.shape[0] != n or self.sh_rest.shape[2] != 3:
             raise RuntimeError("inconsistent Gaussian tensor shapes")
         if self.M.numel() != 16 or self.VPM.numel() != 16 or self.cam_position.numel() != 3:
@@ -350,6 +351,29 @@ def diff_rasterize(
     rasterization.py:116-137).  ``settings.scale_modifier`` is ignored, as in the reference."""
     return _Rasterize.apply(positions, scales, rotations, opacities, sh_0, sh_rest, densification_info, settings,
                             use_distance_scaling)
+
+
+def update_max_weights(
+    max_weights: torch.Tensor,
+    positions: torch.Tensor,
+    scales: torch.Tensor,
+    rotations: torch.Tensor,
+    opacities: torch.Tensor,
+    settings: RasterizerSettings,
+    weight_threshold: float,
+) -> None:
+    """Raises ``max_weights`` ([N] or [N,1] float32, in place) to the largest blending weight each Gaussian reaches in
+    this view; weights below ``weight_threshold`` are ignored (reference: rasterization.py:189-206)."""
+    n = positions.shape[0]
+    if not (isinstance(max_weights, torch.Tensor) and max_weights.is_cuda and max_weights.dtype == torch.float32
+            and max_weights.is_contiguous() and max_weights.numel() == n):
+        raise RuntimeError("max_weights must be a contiguous float32 GPU tensor with one element per Gaussian")
+    with torch.no_grad():
+        fb = FrameBuffers(positions, scales, rotations, opacities, None, None, settings, True, False,
+                          pool=ScratchPool.current(positions.device))
+        _native.check(fb.lib.htgs_max_weights_front(fb._ref))
+        fb.alloc_instances(fb.read_instance_count())
+        _native.check(fb.lib.htgs_max_weights_back(fb._ref, max_weights.data_ptr(), float(weight_threshold)))
 
 
 def rasterize(

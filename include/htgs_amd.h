@@ -47,7 +47,7 @@ typedef struct htgs_frame {
     const float *scales;       /* [N,3] activated */
     const float *rotations;    /* [N,4] (w,x,y,z), normalised */
     const float *opacities;    /* [N]   activated */
-    const float *sh_0;         /* [N,3] */
+    const float *sh_0;         /* [N,3]; NULL = no colour is computed (htgs_max_weights_front) */
     const float *sh_rest;      /* [N,total_sh_bases,3] */
     /* ---- camera, device (RasterizerSettings, rasterization.py:16-42) ---- */
     const float *M;            /* [4,4] world -> camera; only row 2 is read (inference.cu:57) */
@@ -156,6 +156,17 @@ int htgs_blend_backward(const htgs_frame *f, int selector);
 int htgs_preprocess_backward(const htgs_frame *f);
 /* <mode>::backward (R/src/hybrid_blend/backward.cu:26-128): blend backward, then preprocess backward */
 int htgs_backward(const htgs_frame *f, int selector);
+
+/*
+ * `_C.update_max_weights` (bindings.cpp:11, update_max_weights_wrapper rasterization_api.cu:518-631): raises
+ * max_weights [N] (float, non-negative) to the largest blending weight each Gaussian reaches in this view.
+ * front = per-Gaussian stage without colours and with scale modifier 1 + scan; back = create instances + sort +
+ * ranges + htgs_max_weights_blend (update_max_weights_cu, R/include/<mode>/kernels/update_max_weights.cuh).
+ * sh_0 / sh_rest / image / depth of the frame are not used.
+ */
+int htgs_max_weights_front(const htgs_frame *f);
+int htgs_max_weights_back(const htgs_frame *f, float *max_weights, float weight_threshold);
+int htgs_max_weights_blend(const htgs_frame *f, int selector, float *max_weights, float weight_threshold);
 
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes (multiple of 16)
  * with one 16-byte load and store per thread.  Hardware counters read on it calibrate the same counters read on

@@ -291,3 +291,21 @@ def backward(fwd: dict, grad_image, positions, scales, rotations, opacities, sh_
         _p(densification_info), ctypes.c_int(bool(use_distance_scaling)))
     return {"positions": g_pos, "scales": g_scale, "rotations": g_rot, "opacities": g_op, "sh_0": g_sh0, "sh_rest": g_rest,
             "grad_rgb": grad_rgb, "grad_VPMT": g_vpmt}
+
+
+def update_max_weights(frame: Frame, max_weights: np.ndarray, positions, scales, rotations, opacities, weight_threshold: float) -> None:
+    """``_C.update_max_weights`` of the reference (R/src/rasterization_api.cu:518-631): ``max_weights`` [N] float32 is
+    raised in place to the largest blending weight each Gaussian reaches in this view.  The per-Gaussian stage
+    ignores the scale modifier and needs no colours."""
+    import dataclasses
+    frame = dataclasses.replace(frame, scale_modifier=1.0, active_sh_bases=1)
+    n = np.asarray(positions).shape[0]
+    pre = preprocess(frame, positions, scales, rotations, opacities, np.zeros((n, 1, 3), np.float32), np.zeros((n, 0, 3), np.float32))
+    offsets = inclusive_scan(pre["n_touched"])
+    keys, vals = create_instances(frame, pre, offsets)
+    skeys, svals = sort_pairs(keys, vals, end_bit(frame))
+    ranges = extract_ranges(frame, skeys)
+    assert max_weights.dtype == np.float32 and max_weights.flags["C_CONTIGUOUS"]
+    cam = frame.c_struct(0)
+    lib().oracle_update_max_weights(ctypes.byref(cam), _p(ranges), _p(svals), _p(pre["VPMT1"]), _p(pre["VPMT2"]), _p(pre["VPMT4"]),
+                                    _p(pre["MT3"]), _p(pre["rgba"]), _p(max_weights), ctypes.c_float(weight_threshold))

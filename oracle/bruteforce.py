@@ -75,6 +75,7 @@ class Fragments:
     visible: torch.Tensor    # [G] bool
     height: int
     width: int
+    maha2: torch.Tensor = None   # [P, G] squared Mahalanobis distance of the ray from the centre
 
 
 def evaluate(positions, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam_position, mode: int, active_sh_bases: int,
@@ -118,7 +119,7 @@ def evaluate(positions, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam
     visible = (z_centre >= near_plane) & (z_centre <= far_plane) & (z_centre - r_z >= near_plane) & (z_centre + r_z <= far_plane)
     alpha = alpha * visible[None, :].to(F64)
     rgb = sh_colour(positions, sh_0, sh_rest, cam_position, active_sh_bases)
-    return Fragments(alpha, depth, z_centre, rgb, visible, height, width)
+    return Fragments(alpha, depth, z_centre, rgb, visible, height, width, maha2)
 
 
 def _composite_sorted(alpha_s, rgb_s, depth_s, valid_s):
@@ -233,3 +234,51 @@ def render(fr: Fragments, mode: int, K: int, use_median_depth: bool = False, cla
         col = col.clamp(0.0, 1.0)
     H, W = fr.height, fr.width
     return col.T.reshape(3, H, W), dep.reshape(H, W), total_alpha.reshape(H, W), margin.reshape(H, W)
+
+
+CUTOFF_SQ = {0: 11.0825270903, 1: 5.99146454711, 2: 11.0825270903, 3: 11.0825270903}
+
+
+def max_weights(fr: Fragments, mode: int, K: int, weight_threshold: float):
+    """Largest blending weight of every Gaussian over all pixels, by the definition of each mode (the quantity the
+    reference's update_max_weights accumulates).  Returns the maxima [G] and, per Gaussian, the largest weight it
+    would have had without the threshold (to let callers skip Gaussians that sit on the threshold)."""
+    alpha, depth = fr.alpha, fr.depth
+    P, Gn = alpha.shape
+    accepted = alpha >= MIN_ALPHA[mode]
+    big = torch.finfo(F64).max
+    W = torch.zeros_like(alpha)
+    if mode == 2:
+        order = torch.argsort(fr.z_centre, stable=True)
+        a = (alpha * accepted)[:, order]
+        T_in = torch.cumprod(torch.cat([torch.ones_like(a[:, :1]), 1.0 - a[:, :-1]], dim=1), dim=1)
+        live = torch.cumprod((T_in >= T_THRESHOLD).to(F64), dim=1)
+        W[:, order] = T_in * a * live
+    else:
+        T_core = torch.ones(P, dtype=F64)
+        in_core = torch.zeros_like(alpha, dtype=torch.bool)
+        if mode in (0, 1):
+            eligible = accepted & (alpha >= MIN_ALPHA_CORE) if mode == 0 else accepted
+            key = torch.where(eligible, depth, torch.full_like(depth, big))
+            k_eff = min(K, Gn)
+            vals, idx = torch.topk(key, k_eff, dim=1, largest=False)
+            valid = (vals < big).to(F64)
+            a_s = torch.gather(alpha, 1, idx) * valid
+            T_in = torch.cumprod(torch.cat([torch.ones_like(a_s[:, :1]), 1.0 - a_s[:, :-1]], dim=1), dim=1)
+            T_in = torch.where(T_in >= T_THRESHOLD, T_in, torch.zeros_like(T_in))     # transmittance is zeroed below 1e-4
+            w_core = T_in * a_s
+            W.scatter_(1, idx, w_core)
+            T_after = T_in[:, -1] * (1.0 - a_s[:, -1])
+            T_core = torch.where(T_after >= T_THRESHOLD, T_after, torch.zeros_like(T_after))
+            in_core.scatter_(1, idx, valid > 0)
+        if mode in (0, 3):
+            tail = accepted & ~in_core
+            ta = alpha * tail
+            sum_a = ta.sum(1)
+            T_tail = torch.prod(1.0 - ta, dim=1)
+            tail_weight = torch.where(sum_a >= weight_threshold, T_core * (1.0 - T_tail) / sum_a.clamp_min(1e-300), torch.zeros_like(sum_a))
+            tail_weight = torch.where(tail_weight >= weight_threshold, tail_weight, torch.zeros_like(tail_weight))
+            inside_cutoff = (fr.maha2 <= CUTOFF_SQ[mode]) & fr.visible[None, :]
+            W = torch.maximum(W, alpha * tail_weight[:, None] * inside_cutoff)
+    raw = W.max(dim=0).values
+    return torch.where(raw >= weight_threshold, raw, torch.zeros_like(raw)), raw

@@ -1216,3 +1216,111 @@ O_EXPORT void oracle_preprocess_backward(
         }
     }
 }
+
+/* ========================================================================= */
+/* update_max_weights: per-Gaussian maximum blending weight over all pixels  */
+/* ========================================================================= */
+
+static inline void max_weight(float *max_weights, uint32_t g, float w)
+{
+    /* atomicMax on the bit patterns of non-negative floats = float max */
+    if (g != UINT32_MAX && float_to_bits(max_weights[g]) < float_to_bits(w)) max_weights[g] = w;
+}
+
+/* update_max_weights_cu of the four modes:
+ * R/include/hybrid_blend/kernels/update_max_weights.cuh:59-212,
+ * R/include/alpha_blend_first_k/kernels/update_max_weights.cuh:59-161,
+ * R/include/alpha_blend_global_ordering/kernels/update_max_weights.cuh:59-131,
+ * R/include/oit_blend/kernels/update_max_weights.cuh:58-165.
+ * The per-Gaussian stage is preprocess_cu of the same files (scale modifier 1, no colour), i.e.
+ * oracle_preprocess with scale_modifier = 1.  max_weights [N] is updated in place.
+ * pinned by: float64 brute force of the definition (weight of a fragment in the pixel's blend). */
+O_EXPORT void oracle_update_max_weights(
+    const oracle_cam *c, const uint32_t *ranges, const uint32_t *inst,
+    const float *VPMT1, const float *VPMT2, const float *VPMT4, const float *MT3, const float *rgba,
+    float *max_weights, float weight_threshold)
+{
+    const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
+    const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
+    const int K = round_k(c->K);
+    const int mode = c->mode;
+    const float cutoff = mode_cutoff_sq(mode), min_alpha = mode_min_alpha(mode);
+    for (int t = 0; t < grid_w * grid_h; ++t) {
+        const int tx = t % grid_w, ty = t / grid_w;
+        const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        for (int l = 0; l < c->tile_w * c->tile_h; ++l) {
+            const int x = tx * c->tile_w + l % c->tile_w, y = ty * c->tile_h + l / c->tile_w;
+            if (x >= c->width || y >= c->height) continue;
+            const float fx = (float)x, fy = (float)y;
+            fragment f;
+            if (mode == MODE_GLOBAL) {
+                float T = 1.0f;
+                for (uint32_t j = first; j < last; ++j) {
+                    const size_t g = inst[j];
+                    if (!eval_fragment(VPMT1 + 4 * g, VPMT2 + 4 * g, VPMT4 + 4 * g, MT3 + 4 * g, rgba[4 * g + 3], fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+                    const float w = T * f.alpha;
+                    T *= 1.0f - f.alpha;
+                    if (!(w < weight_threshold)) max_weight(max_weights, (uint32_t)g, w);
+                    if (T < TRANSMITTANCE_THRESHOLD) break;
+                }
+                continue;
+            }
+            float alpha_sum = 0.0f, T_tail = 1.0f;
+            float core_alpha[KMAX], core_depth[KMAX];
+            uint32_t core_idx[KMAX];
+            for (int i = 0; i < K; ++i) { core_alpha[i] = 0.0f; core_depth[i] = FLT_MAX; core_idx[i] = UINT32_MAX; }
+            for (uint32_t j = first; j < last; ++j) {
+                const size_t g = inst[j];
+                const float *lim = mode == MODE_FIRST_K ? &core_depth[K - 1] : NULL;
+                if (!eval_fragment(VPMT1 + 4 * g, VPMT2 + 4 * g, VPMT4 + 4 * g, MT3 + 4 * g, rgba[4 * g + 3], fx, fy, cutoff, min_alpha,
+                                   mode != MODE_OIT, lim, &f)) continue;
+                float depth = f.depth, alpha = f.alpha;
+                if (mode == MODE_FIRST_K || (mode == MODE_HYBRID && depth < core_depth[K - 1] && alpha >= MIN_ALPHA_CORE)) {
+                    uint32_t idx = (uint32_t)g;
+                    for (int i = 0; i < K; ++i) {
+                        if (depth < core_depth[i]) {
+                            float tt = depth; depth = core_depth[i]; core_depth[i] = tt;
+                            tt = alpha; alpha = core_alpha[i]; core_alpha[i] = tt;
+                            uint32_t ti = idx; idx = core_idx[i]; core_idx[i] = ti;
+                        }
+                    }
+                }
+                if (mode != MODE_FIRST_K) { alpha_sum += alpha; T_tail *= 1.0f - alpha; }
+            }
+            float T_core = 1.0f;
+            if (mode != MODE_OIT) {
+                for (int i = 0; i < K; ++i) {
+                    const float w = T_core * core_alpha[i];
+                    T_core *= 1.0f - core_alpha[i];
+                    if (T_core < TRANSMITTANCE_THRESHOLD) T_core = 0.0f;
+                    if (w < weight_threshold) continue;
+                    max_weight(max_weights, core_idx[i], w);
+                }
+            }
+            if (mode == MODE_FIRST_K) continue;
+            float tail_weight = 0.0f;
+            if (alpha_sum >= weight_threshold) tail_weight = (T_core * (1.0f - T_tail)) * (1.0f / alpha_sum);
+            if (!(tail_weight >= weight_threshold)) continue;
+            /* second pass: every fragment that passes the cut-off gets alpha * tail_weight; no alpha threshold here */
+            for (uint32_t j = first; j < last; ++j) {
+                const size_t g = inst[j];
+                for (int k = 0; k < 4; ++k) {
+                    f.px[k] = fmaf(-VPMT4[4 * g + k], fx, VPMT1[4 * g + k]);
+                    f.py[k] = fmaf(-VPMT4[4 * g + k], fy, VPMT2[4 * g + k]);
+                }
+                for (int k = 0; k < 3; ++k) f.m[k] = fmaf(f.px[3], f.py[k], -(f.px[k] * f.py[3]));
+                f.d[0] = fmaf(f.px[1], f.py[2], -(f.px[2] * f.py[1]));
+                f.d[1] = fmaf(f.px[2], f.py[0], -(f.px[0] * f.py[2]));
+                f.d[2] = fmaf(f.px[0], f.py[1], -(f.px[1] * f.py[0]));
+                f.num = fmaf(f.m[2], f.m[2], fmaf(f.m[1], f.m[1], f.m[0] * f.m[0]));
+                f.den = fmaf(f.d[2], f.d[2], fmaf(f.d[1], f.d[1], f.d[0] * f.d[0]));
+                if (f.num > cutoff * f.den) continue;
+                const float G = o_expf((-0.5f * f.num) * (1.0f / f.den));
+                const float a = rgba[4 * g + 3] * G;
+                const float w = (a < MAX_FRAGMENT_ALPHA ? a : MAX_FRAGMENT_ALPHA) * tail_weight;
+                if (w < weight_threshold) continue;
+                max_weight(max_weights, (uint32_t)g, w);
+            }
+        }
+    }
+}

@@ -380,3 +380,25 @@ def test_hybrid_with_large_k_equals_sorted_alpha_blending_of_core_plus_tail():
     w = T * a * (T >= 1e-4)
     want = (w[..., None] * fr.rgb[order]).sum(1).clamp(0, 1).T.reshape(3, sc.height, sc.width).numpy()
     assert np.abs(hyb["image"] - want)[:, clean].max() < 2e-5
+
+
+# ---------------------------------------------------------------------------------------------------------
+# update_max_weights
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("K,threshold", [(4, 0.01), (16, 0.05)])
+def test_max_weights_match_float64_definition(mode, K, threshold):
+    sc = small_scene(n=140, seed=41 + mode)
+    got = np.full(140, 0.0, np.float32)
+    got[:5] = 0.9                                   # pre-existing maxima must survive
+    oracle.update_max_weights(oracle_frame(sc, mode, K, scale_modifier=3.0), got, *[t.numpy() for t in sc.gaussians()[:4]], threshold)
+    fr = bf.evaluate(*sc.gaussians(), sc.M, sc.VPM, sc.cam_position, mode, sc.active_sh_bases, sc.width, sc.height,
+                     sc.near_plane, sc.far_plane)            # scale modifier 1: update_max_weights ignores it
+    want, raw = bf.max_weights(fr, mode, K, threshold)
+    want = want.numpy()
+    want[:5] = np.maximum(want[:5], 0.9)
+    clear = np.abs(raw.numpy() / threshold - 1.0) > 1e-3     # not sitting on the threshold
+    assert (want[clear] > 0).sum() > 30
+    close = np.isclose(got, want, rtol=2e-4, atol=1e-6)
+    # a pixel whose core membership flips between float32 and float64 can move a maximum: allow a handful
+    assert close[clear].mean() > 0.97, (close[clear].mean(), got[clear][~close[clear]], want[clear][~close[clear]])
