@@ -100,6 +100,9 @@ SYMBOLS = {
     "htgs_max_weights_front": (ctypes.c_int, [_FRAME_P]),
     "htgs_max_weights_back": (ctypes.c_int, [_FRAME_P, ctypes.c_void_p, ctypes.c_float]),
     "htgs_max_weights_blend": (ctypes.c_int, [_FRAME_P, ctypes.c_int, ctypes.c_void_p, ctypes.c_float]),
+    "htgs_update_3d_filter": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                             ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                             ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_void_p]),
     "htgs_copy_bytes": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
 }
 

@@ -168,6 +168,15 @@ int htgs_max_weights_front(const htgs_frame *f);
 int htgs_max_weights_back(const htgs_frame *f, float *max_weights, float weight_threshold);
 int htgs_max_weights_blend(const htgs_frame *f, int selector, float *max_weights, float weight_threshold);
 
+/*
+ * `_C.update_3d_filter_cuda` (bindings.cpp:15; filter3d/src/filter3d_api.cu:6-47, filter3d_kernels.cu:6-35): for every
+ * point inside the dilated frustum of the view, filter_3d[i] = min(filter_3d[i], distance2filter * depth) and
+ * visibility_mask[i] = 1.  positions [N,3], w2c [4,4], filter_3d [N], visibility_mask [N] bytes, all on the device.
+ */
+int htgs_update_3d_filter(const float *positions, const float *w2c, float *filter_3d, uint8_t *visibility_mask, int n_points,
+                          int width, int height, float focal_x, float focal_y, float center_x, float center_y,
+                          float near_plane, float clipping_tolerance, float distance2filter, void *stream);
+
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes (multiple of 16)
  * with one 16-byte load and store per thread.  Hardware counters read on it calibrate the same counters read on
  * the rasterizer's kernels (bench.py --calibrate). */

@@ -309,3 +309,28 @@ def update_max_weights(frame: Frame, max_weights: np.ndarray, positions, scales,
     cam = frame.c_struct(0)
     lib().oracle_update_max_weights(ctypes.byref(cam), _p(ranges), _p(svals), _p(pre["VPMT1"]), _p(pre["VPMT2"]), _p(pre["VPMT4"]),
                                     _p(pre["MT3"]), _p(pre["rgba"]), _p(max_weights), ctypes.c_float(weight_threshold))
+
+
+def update_3d_filter(positions, w2c, filter_3d, visibility_mask, width, height, focal_x, focal_y, center_x, center_y,
+                     near_plane, clipping_tolerance, distance2filter) -> None:
+    """numpy float32 restatement of update_3d_filter (filter3d/src/filter3d_api.cu:6-47, filter3d_kernels.cu:6-35);
+    ``filter_3d`` (float32 [N]) and ``visibility_mask`` (bool [N]) are updated in place.
+    pinned by: points placed at known angles inside / outside a frustum (tests/test_oracle_pinning.py)."""
+    f32 = np.float32
+    p = _f32(positions)
+    w = _f32(w2c).reshape(16)
+    bounds_factor = f32(clipping_tolerance) + f32(0.5)
+    wf, hf = f32(width), f32(height)
+    max_x, max_y = bounds_factor * wf, bounds_factor * hf
+    off_x, off_y = f32(center_x) - f32(0.5) * wf, f32(center_y) - f32(0.5) * hf
+    left, right = (-max_x - off_x) / f32(focal_x), (max_x - off_x) / f32(focal_x)
+    top, bottom = (-max_y - off_y) / f32(focal_y), (max_y - off_y) / f32(focal_y)
+    px, py, pz = p[:, 0], p[:, 1], p[:, 2]
+    z = (w[8] * px + w[9] * py + w[10] * pz) + w[11]
+    x_clip = (w[0] * px + w[1] * py + w[2] * pz) + w[3]
+    y_clip = (w[4] * px + w[5] * py + w[6] * pz) + w[7]
+    inside = ~(z < f32(near_plane)) & ~((x_clip < left * z) | (x_clip > right * z)) & ~((y_clip < top * z) | (y_clip > bottom * z))
+    cand = f32(distance2filter) * z
+    update = inside & ~(filter_3d < cand)
+    filter_3d[update] = cand[update]
+    visibility_mask[update] = True

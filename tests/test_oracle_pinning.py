@@ -402,3 +402,28 @@ def test_max_weights_match_float64_definition(mode, K, threshold):
     close = np.isclose(got, want, rtol=2e-4, atol=1e-6)
     # a pixel whose core membership flips between float32 and float64 can move a maximum: allow a handful
     assert close[clear].mean() > 0.97, (close[clear].mean(), got[clear][~close[clear]], want[clear][~close[clear]])
+
+
+def test_3d_filter_frustum_and_minimum():
+    """Points on rays at known pixel positions: inside the image, inside only the dilated frustum, outside it, behind
+    the near plane; filter = min over calls of distance2filter * depth."""
+    width, height, fx, fy, cx, cy = 200, 100, 150.0, 120.0, 100.0, 50.0
+    w2c = np.eye(4, dtype=np.float32)
+
+    def point(u, v, z):                          # world point that projects to pixel (u, v) at depth z
+        return [(u - cx) / fx * z, (v - cy) / fy * z, z]
+    tol = 0.15
+    pts = np.array([point(100, 50, 2.0), point(199, 99, 3.0), point(200 + 0.14 * 200, 50, 2.0), point(200 + 0.16 * 200, 50, 2.0),
+                    point(100, -0.14 * 100, 4.0), point(100, -0.16 * 100, 4.0), point(100, 50, 0.1), point(100, 50, 5.0)], np.float32)
+    filt = np.full(8, 1e9, np.float32)
+    filt[7] = 0.001                              # already smaller than anything this view can offer
+    vis = np.zeros(8, bool)
+    oracle.update_3d_filter(pts, w2c, filt, vis, width, height, fx, fy, cx, cy, 0.2, tol, 0.01)
+    assert vis.tolist() == [True, True, True, False, True, False, False, False]
+    np.testing.assert_allclose(filt[[0, 1, 2, 4]], 0.01 * np.array([2.0, 3.0, 2.0, 4.0]), rtol=1e-6)
+    assert filt[3] == filt[5] == filt[6] == np.float32(1e9) and filt[7] == np.float32(0.001)
+    # a second, closer view lowers the filter
+    w2c2 = w2c.copy()
+    w2c2[2, 3] = -1.0
+    oracle.update_3d_filter(pts, w2c2, filt, vis, width, height, fx, fy, cx, cy, 0.2, 10.0, 0.01)
+    np.testing.assert_allclose(filt[0], 0.01 * 1.0, rtol=1e-6)
