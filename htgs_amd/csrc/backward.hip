@@ -156,7 +156,9 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_kerne
             f.den_rcp = 1.0f / f.den;
             if (!frag_alpha<MODE>(col.w, f)) continue;
             int slot = -1;
-            if (K > 0 && f.alpha >= kMinAlphaCore) {
+            // only fragments with alpha >= 1/20 can sit in the core; the margin covers the forward pass having
+            // evaluated alpha in tile-relative form (the stored index decides)
+            if (K > 0 && f.alpha >= 0.98f * kMinAlphaCore) {
 #pragma unroll
                 for (int i = 0; i < KS; ++i)
                     if (s_idx[p * KS + i] == g) slot = i;                        // :231-235

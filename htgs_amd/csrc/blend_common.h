@@ -1,10 +1,13 @@
-// Pieces shared by the inference, training-forward and backward blend kernels.
+// Pieces shared by the inference, training-forward, max-weight and backward blend kernels.
 #pragma once
 
 #include "common.h"
 
 namespace htgs {
 
+// ---------------------------------------------------------------------------------------------
+// plane form: the Gaussian's record as preprocess wrote it (backward kernels)
+// ---------------------------------------------------------------------------------------------
 template <int N>
 struct Stage {
     float4 v1[N], v2[N], v4[N], mt3[N], col[N];
@@ -27,8 +30,136 @@ __device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restric
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// tile-relative form (forward direction).  With px = px0 - dx VPMT4, py = py0 - dy VPMT4, where px0 / py0 are
+// the reference's planes (R/include/hybrid_blend/kernels/inference.cuh:137-141) through the tile centre and
+// (dx, dy) is the pixel's offset from it,
+//     d = cross(px.n, py.n)     = A  + dy B  + dx C
+//     m = px.w py.n - px.n py.w = Am + dy Bm + dx Cm            (the dx dy terms cancel)
+// so |m|^2, |d|^2 and MT3.n . cross(d, m) are quadratics in (dx, dy).  The lane that stages an instance
+// computes the 18 coefficients once; every pixel then needs 5 fused multiply-adds per quadratic.
+// LDS layout per instance, coefficient order (1, dx, dy, dx^2, dx dy, dy^2):
+//     q[0] = n0 nx ny nxx   q[1] = nxy nyy d0 dx   q[2] = dy dxx dxy dyy
+//     q[3] = z0 zx zy zxx   q[4] = zxy zyy MT3.w opacity   q[5] = r g b (primitive index bits)
+// ---------------------------------------------------------------------------------------------
+template <int N>
+struct TileStage {
+    float4 q[6][N];
+};
+
+__device__ __forceinline__ void cross3(const float *a, const float *b, float *o)
+{
+    o[0] = __builtin_fmaf(a[1], b[2], -(a[2] * b[1]));
+    o[1] = __builtin_fmaf(a[2], b[0], -(a[0] * b[2]));
+    o[2] = __builtin_fmaf(a[0], b[1], -(a[1] * b[0]));
+}
+__device__ __forceinline__ float dotf(const float *a, const float *b)
+{
+    return __builtin_fmaf(a[2], b[2], __builtin_fmaf(a[1], b[1], a[0] * b[0]));
+}
+
+template <int N, bool DEPTH>
+__device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
+                                                uint32_t fetch, uint32_t last, int slot, float cx, float cy)
+{
+    if (fetch >= last) return;
+    const uint32_t g = inst[fetch];
+    const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
+    const float4 r1 = rec[0], r2 = rec[1], r4 = rec[2], r3 = rec[3], col = rec[4];
+    const float V1[4] = { r1.x, r1.y, r1.z, r1.w }, V2[4] = { r2.x, r2.y, r2.z, r2.w }, V4[4] = { r4.x, r4.y, r4.z, r4.w };
+    float px0[4], py0[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        px0[k] = __builtin_fmaf(-V4[k], cx, V1[k]);
+        py0[k] = __builtin_fmaf(-V4[k], cy, V2[k]);
+    }
+    float A[3], B[3], C[3], Am[3], Bm[3], Cm[3];
+    cross3(px0, py0, A);
+    cross3(V4, px0, B);
+    cross3(py0, V4, C);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        Am[k] = __builtin_fmaf(px0[3], py0[k], -(px0[k] * py0[3]));
+        Bm[k] = __builtin_fmaf(px0[k], V4[3], -(px0[3] * V4[k]));
+        Cm[k] = __builtin_fmaf(V4[k], py0[3], -(V4[3] * py0[k]));
+    }
+    st.q[0][slot] = make_float4(dotf(Am, Am), 2.0f * dotf(Am, Cm), 2.0f * dotf(Am, Bm), dotf(Cm, Cm));
+    st.q[1][slot] = make_float4(2.0f * dotf(Bm, Cm), dotf(Bm, Bm), dotf(A, A), 2.0f * dotf(A, C));
+    st.q[2][slot] = make_float4(2.0f * dotf(A, B), dotf(C, C), 2.0f * dotf(B, C), dotf(B, B));
+    float zxy = 0.0f, zyy = 0.0f;
+    if (DEPTH) {
+        const float MT3[3] = { r3.x, r3.y, r3.z };
+        float PA[3], PB[3], PC[3];
+        cross3(MT3, A, PA);
+        cross3(MT3, B, PB);
+        cross3(MT3, C, PC);
+        st.q[3][slot] = make_float4(dotf(PA, Am), dotf(PA, Cm) + dotf(PC, Am), dotf(PA, Bm) + dotf(PB, Am), dotf(PC, Cm));
+        zxy = dotf(PB, Cm) + dotf(PC, Bm);
+        zyy = dotf(PB, Bm);
+    }
+    st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
+    st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
+}
+
+// the pixel's offset from the tile centre (exact)
+struct PixelTerms {
+    float X, Y;
+};
+__device__ __forceinline__ PixelTerms pixel_terms(uint32_t local_x, uint32_t local_y, int tile)
+{
+    PixelTerms p;
+    p.X = (float)local_x - 0.5f * (float)(tile - 1);
+    p.Y = (float)local_y - 0.5f * (float)(tile - 1);
+    return p;
+}
+__device__ __forceinline__ float tile_centre(uint32_t first_pixel, int tile) { return (float)first_pixel + 0.5f * (float)(tile - 1); }
+
+__device__ __forceinline__ float quad_eval(float c0, float cx, float cy, float cxx, float cxy, float cyy, const PixelTerms &p)
+{
+    const float tx = __builtin_fmaf(cxy, p.Y, __builtin_fmaf(cxx, p.X, cx));
+    const float ty = __builtin_fmaf(cyy, p.Y, cy);
+    return __builtin_fmaf(p.Y, ty, __builtin_fmaf(p.X, tx, c0));
+}
+
+struct TileFrag {
+    float num, den, den_rcp, alpha;
+};
+
+// |m|^2 <= cutoff |d|^2 ?  (inference.cuh:147)
+template <int MODE, int N>
+__device__ __forceinline__ bool tile_frag_cutoff(const TileStage<N> &st, int j, const PixelTerms &p, TileFrag &o)
+{
+    const float4 q0 = st.q[0][j], q1 = st.q[1][j], q2 = st.q[2][j];
+    o.num = quad_eval(q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, p);
+    o.den = quad_eval(q1.z, q1.w, q2.x, q2.y, q2.z, q2.w, p);
+    return !(o.num > ModeCfg<MODE>::cutoff_sq * o.den);
+}
+
+// camera-space depth of the point of maximum contribution (inference.cuh:151-152); needs o.den_rcp
+template <int N>
+__device__ __forceinline__ float tile_frag_depth(const TileStage<N> &st, int j, const PixelTerms &p, const TileFrag &o)
+{
+    const float4 q3 = st.q[3][j], q4 = st.q[4][j];
+    return __builtin_fmaf(quad_eval(q3.x, q3.y, q3.z, q3.w, q4.x, q4.y, p), o.den_rcp, q4.z);
+}
+
+// alpha of the fragment, false below the mode's threshold; needs o.den_rcp
+template <int MODE>
+__device__ __forceinline__ bool tile_frag_alpha(float opacity, TileFrag &o)
+{
+    const float G = d_exp2((o.num * kNegHalfLog2e) * o.den_rcp);
+    const float a = opacity * G;
+    o.alpha = a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha;
+    return !(o.alpha < ModeCfg<MODE>::min_alpha);
+}
+
 // exchange two VGPRs in the active lanes (one instruction instead of a select pair)
 __device__ __forceinline__ void vswap(float &a, float &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
 __device__ __forceinline__ void vswap(uint32_t &a, uint32_t &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+
+// Sorted insertion into a K-slot buffer walks the slots front to back carrying the displaced entry; the kernels
+// take the slots four at a time and the whole wave skips a group that no active lane can change (the carried
+// depth is not below the group's last slot).
+constexpr int kInsertGroup = 4;
 
 }  // namespace htgs

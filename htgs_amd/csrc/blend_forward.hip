@@ -23,13 +23,14 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
     uint32_t width, uint32_t height, uint32_t grid_w)
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
-    __shared__ Stage<64> st;
-    __shared__ uint32_t st_idx[64];
+    __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
     const bool inside = x < width && y < height;
-    const float fx = (float)x, fy = (float)y;
+    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
+    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
 
     float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f;
     float c0[K], c1[K], c2[K], c3[K], cd[K];
@@ -40,28 +41,32 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         for (int j = 0; j < nb; ++j) {
-            Frag f;
-            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
-            const float4 col = st.col[j];
-            if (!frag_alpha<MODE>(col.w, f)) continue;
-            float depth = frag_depth(st.mt3[j], f);
+            TileFrag f;
+            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            f.den_rcp = rcp_exact(f.den);
+            const float4 col = st.q[5][j];
+            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
+            float depth = tile_frag_depth(st, j, pt, f);
             float p0 = col.x, p1 = col.y, p2 = col.z, p3 = f.alpha;
             if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
-                uint32_t idx = st_idx[j];
+                uint32_t idx = float_to_bits(st.q[5][j].w);
 #pragma unroll
-                for (int i = 0; i < K; ++i) {
-                    if (depth < cd[i]) {
-                        vswap(depth, cd[i]);
-                        vswap(p0, c0[i]);
-                        vswap(p1, c1[i]);
-                        vswap(p2, c2[i]);
-                        vswap(p3, c3[i]);
-                        vswap(idx, ci[i]);
+                for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
+                    if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
+#pragma unroll
+                    for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
+                        if (depth < cd[i]) {
+                            vswap(depth, cd[i]);
+                            vswap(p0, c0[i]);
+                            vswap(p1, c1[i]);
+                            vswap(p2, c2[i]);
+                            vswap(p3, c3[i]);
+                            vswap(idx, ci[i]);
+                        }
                     }
                 }
             }
@@ -127,13 +132,14 @@ __global__ void __launch_bounds__(64) blend_first_k_forward_kernel(
     uint32_t width, uint32_t height, uint32_t grid_w)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
-    __shared__ Stage<64> st;
-    __shared__ uint32_t st_idx[64];
+    __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
     const bool inside = x < width && y < height;
-    const float fx = (float)x, fy = (float)y;
+    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
+    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
 
     float ca[K], cd[K];
     uint32_t ci[K];
@@ -143,24 +149,28 @@ __global__ void __launch_bounds__(64) blend_first_k_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         for (int j = 0; j < nb; ++j) {
-            Frag f;
-            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
-            float depth = frag_depth(st.mt3[j], f);
+            TileFrag f;
+            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            f.den_rcp = rcp_exact(f.den);
+            float depth = tile_frag_depth(st, j, pt, f);
             if (depth >= cd[K - 1]) continue;
-            if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
             float alpha = f.alpha;
-            uint32_t idx = st_idx[j];
+            uint32_t idx = float_to_bits(st.q[5][j].w);
 #pragma unroll
-            for (int i = 0; i < K; ++i) {
-                if (depth < cd[i]) {
-                    vswap(depth, cd[i]);
-                    vswap(alpha, ca[i]);
-                    vswap(idx, ci[i]);
+            for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
+                if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
+#pragma unroll
+                for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
+                    if (depth < cd[i]) {
+                        vswap(depth, cd[i]);
+                        vswap(alpha, ca[i]);
+                        vswap(idx, ci[i]);
+                    }
                 }
             }
         }
@@ -215,26 +225,28 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     float *__restrict__ image, float *__restrict__ tail_info, uint32_t width, uint32_t height, uint32_t grid_w)
 {
     constexpr int MODE = HTGS_MODE_OIT_BLEND;
-    __shared__ Stage<64> st;
+    __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
     const bool inside = x < width && y < height;
-    const float fx = (float)x, fy = (float)y;
+    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
+    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        stage_load(st, prim, inst, base + lane, last, lane, nullptr);
+        tile_stage_load<64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         for (int j = 0; j < nb; ++j) {
-            Frag f;
-            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
-            const float4 col = st.col[j];
-            if (!frag_alpha<MODE>(col.w, f)) continue;
+            TileFrag f;
+            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            f.den_rcp = rcp_exact(f.den);
+            const float4 col = st.q[5][j];
+            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
             a0 = __builtin_fmaf(f.alpha, col.x, a0);
             a1 = __builtin_fmaf(f.alpha, col.y, a1);
             a2 = __builtin_fmaf(f.alpha, col.z, a2);
@@ -261,27 +273,29 @@ __global__ void __launch_bounds__(256) blend_global_forward_kernel(
     float *__restrict__ image, uint32_t width, uint32_t height, uint32_t grid_w)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
-    __shared__ Stage<256> st;
+    __shared__ TileStage<256> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t t = threadIdx.x;
-    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
+    const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
+    const uint32_t x = x0 + (t & 15), y = y0 + (t >> 4);
     const bool inside = x < width && y < height;
-    const float fx = (float)x, fy = (float)y;
+    const PixelTerms pt = pixel_terms(t & 15, t >> 4, 16);
+    const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
     float r = 0.0f, g = 0.0f, b = 0.0f, T = 1.0f;
     bool done = !inside;
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        stage_load(st, prim, inst, base + t, last, t, nullptr);
+        tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         for (int j = 0; !done && j < nb; ++j) {
-            Frag f;
-            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
-            const float4 col = st.col[j];
-            if (!frag_alpha<MODE>(col.w, f)) continue;
+            TileFrag f;
+            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            f.den_rcp = rcp_exact(f.den);
+            const float4 col = st.q[5][j];
+            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
             const float bw = T * f.alpha;
             r = __builtin_fmaf(bw, col.x, r);
             g = __builtin_fmaf(bw, col.y, g);

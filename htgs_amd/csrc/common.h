@@ -2,11 +2,15 @@
 //
 // Rounding convention.  The whole library is compiled with -ffp-contract=off, so a fused
 // multiply-add exists exactly where __builtin_fmaf is written.  The per-Gaussian stage uses none
-// (operand order of the reference source, R/include/kernel_utils.cuh); the per-pixel stage fuses
-// the contractions listed in eval_fragment().  log and exp are the polynomial routines below, sqrt
-// and division are correctly rounded (-fhip-fp32-correctly-rounded-divide-sqrt).  The CPU checker
-// used by the test-suite follows the same convention, which is what makes tile counts, sort order
-// and every per-fragment accept/reject decision reproducible bit for bit.
+// (operand order of the reference source, R/include/kernel_utils.cuh).  The per-pixel stage has two
+// forms of the reference's ray / Gaussian evaluation: the plane form (frag_cutoff / frag_depth /
+// frag_alpha), kept by the backward pass because it needs the intermediates, and the tile-relative
+// form (TileFrag, blend_common.h) used by every forward-direction kernel, in which |m|^2, |d|^2 and
+// MT3.(d x m) are quadratics of the pixel offset from the tile centre.  log, exp and 2^x are the
+// polynomial routines below, sqrt and division are correctly rounded
+// (-fhip-fp32-correctly-rounded-divide-sqrt; rcp_exact is the same quotient, cheaper).  The CPU
+// checker used by the test-suite follows the same convention, which is what makes tile counts, sort
+// order and every per-fragment accept/reject decision reproducible bit for bit.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -83,6 +87,38 @@ __device__ __forceinline__ float d_expf(float x)
     const float y = __builtin_fmaf(p, r2, r) + 1.0f;
     const int ni = (int)n;
     return bits_to_float((uint32_t)((int)float_to_bits(y) + ni * 8388608));
+}
+
+// 2^t for t in [-126, 1): n = rint(t), r = t - n, degree-5 polynomial of 2^r on [-1/2, 1/2] (relative error 2.7e-7)
+constexpr float kNegHalfLog2e = -0.72134752044448170f;     // exp(-rho^2 / 2) = 2^(rho^2 * this)
+__device__ __forceinline__ float d_exp2(float t)
+{
+    const float n = __builtin_rintf(t);
+    const float r = t - n;
+    float p = 1.3381302124e-3f;
+    p = __builtin_fmaf(p, r, 9.6663683653e-3f);
+    p = __builtin_fmaf(p, r, 5.5503811687e-2f);
+    p = __builtin_fmaf(p, r, 2.4022349715e-1f);
+    p = __builtin_fmaf(p, r, 6.9314718246e-1f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    const int ni = (int)n;
+    return bits_to_float((uint32_t)((int)float_to_bits(p) + ni * 8388608));
+}
+
+// 1 / x.  v_rcp_f32 followed by one fused Newton step is the correctly rounded quotient for every x with
+// 2^-120 <= x < 2^121 on gfx950 (htgs_check_reciprocal compares all of them with the division); a wave in
+// which any active lane is outside that range takes the division.
+__device__ __forceinline__ bool rcp_in_range(float x) { return float_to_bits(x) - 0x03800000u < 0x78800000u; }
+__device__ __forceinline__ float rcp_refined(float x)
+{
+    const float x0 = __builtin_amdgcn_rcpf(x);
+    const float e = __builtin_fmaf(-x, x0, 1.0f);
+    return __builtin_fmaf(x0, e, x0);
+}
+__device__ __forceinline__ float rcp_exact(float x)
+{
+    if (__builtin_expect(__any(!rcp_in_range(x)), 0)) return 1.0f / x;
+    return rcp_refined(x);
 }
 
 __device__ __forceinline__ float clamp_pos(float v) { return v > 0.0f ? v : 0.0f; }

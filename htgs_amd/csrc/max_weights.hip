@@ -24,13 +24,14 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
     constexpr bool kCore = MODE != HTGS_MODE_OIT_BLEND;
     constexpr bool kTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = kCore ? K : 1;
-    __shared__ Stage<64> st;
-    __shared__ uint32_t st_idx[64];
+    __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x = (tile % grid_w) * 8 + (lane & 7), y = (tile / grid_w) * 8 + (lane >> 3);
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
     const bool inside = x < width && y < height;
-    const float fx = (float)x, fy = (float)y;
+    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
+    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
 
     float alpha_sum = 0.0f, T_tail = 1.0f;
     float ca[KS], cd[KS];
@@ -41,29 +42,33 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        tile_stage_load<64, kCore>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         for (int j = 0; j < nb; ++j) {
-            Frag f;
-            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
+            TileFrag f;
+            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            f.den_rcp = rcp_exact(f.den);
             float depth = 0.0f;
             if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
-                depth = frag_depth(st.mt3[j], f);
+                depth = tile_frag_depth(st, j, pt, f);
                 if (depth >= cd[KS - 1]) continue;
             }
-            if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
             float alpha = f.alpha;
-            if (MODE == HTGS_MODE_HYBRID_BLEND) depth = frag_depth(st.mt3[j], f);
+            if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth(st, j, pt, f);
             if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
-                uint32_t idx = st_idx[j];
+                uint32_t idx = float_to_bits(st.q[5][j].w);
 #pragma unroll
-                for (int i = 0; i < KS; ++i) {
-                    if (depth < cd[i]) {
-                        vswap(depth, cd[i]);
-                        vswap(alpha, ca[i]);
-                        vswap(idx, ci[i]);
+                for (int g0 = 0; g0 < KS; g0 += kInsertGroup) {
+                    if (KS > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < KS ? g0 + kInsertGroup - 1 : KS - 1])) continue;
+#pragma unroll
+                    for (int i = g0; i < g0 + kInsertGroup && i < KS; ++i) {
+                        if (depth < cd[i]) {
+                            vswap(depth, cd[i]);
+                            vswap(alpha, ca[i]);
+                            vswap(idx, ci[i]);
+                        }
                     }
                 }
             }
@@ -88,17 +93,16 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
     // second walk over the tile's list: alpha * tail weight for every fragment that passes the cut-off
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        stage_load(st, prim, inst, base + lane, last, lane, st_idx);
+        tile_stage_load<64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         for (int j = 0; j < nb; ++j) {
-            Frag f;
-            if (!active || !frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
-            const float G = d_expf((-0.5f * f.num) * f.den_rcp);
-            const float a = st.col[j].w * G;
+            TileFrag f;
+            if (!active || !tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            const float G = d_exp2((f.num * kNegHalfLog2e) * rcp_exact(f.den));
+            const float a = st.q[4][j].w * G;
             const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
-            if (!(w < weight_threshold)) raise_max(max_weights, st_idx[j], w);
+            if (!(w < weight_threshold)) raise_max(max_weights, float_to_bits(st.q[5][j].w), w);
         }
     }
 }
@@ -108,30 +112,31 @@ __global__ void __launch_bounds__(256) max_weights_global_kernel(
     uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
-    __shared__ Stage<256> st;
-    __shared__ uint32_t st_idx[256];
+    __shared__ TileStage<256> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t t = threadIdx.x;
-    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
+    const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
+    const uint32_t x = x0 + (t & 15), y = y0 + (t >> 4);
     const bool inside = x < width && y < height;
-    const float fx = (float)x, fy = (float)y;
+    const PixelTerms pt = pixel_terms(t & 15, t >> 4, 16);
+    const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
     float T = 1.0f;
     bool done = !inside;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        stage_load(st, prim, inst, base + t, last, t, st_idx);
+        tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         for (int j = 0; !done && j < nb; ++j) {
-            Frag f;
-            if (!frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) continue;
-            f.den_rcp = 1.0f / f.den;
-            if (!frag_alpha<MODE>(st.col[j].w, f)) continue;
+            TileFrag f;
+            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            f.den_rcp = rcp_exact(f.den);
+            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
             const float w = T * f.alpha;
             T *= 1.0f - f.alpha;
             if (T < kTransmittanceThreshold) done = true;
-            if (!(w < weight_threshold)) raise_max(max_weights, st_idx[j], w);
+            if (!(w < weight_threshold)) raise_max(max_weights, float_to_bits(st.q[5][j].w), w);
         }
     }
 }

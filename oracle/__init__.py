@@ -62,6 +62,8 @@ def lib():
         _lib.o_logf.argtypes = [ctypes.c_float]
         _lib.o_expf.restype = ctypes.c_float
         _lib.o_expf.argtypes = [ctypes.c_float]
+        _lib.o_exp2.restype = ctypes.c_float
+        _lib.o_exp2.argtypes = [ctypes.c_float]
         _lib.oracle_inclusive_scan.restype = ctypes.c_uint32
         _lib.oracle_num_threads.restype = ctypes.c_int
     return _lib
@@ -133,6 +135,20 @@ def logf(x: float) -> float:
 
 def expf(x: float) -> float:
     return float(lib().o_expf(x))
+
+
+def exp2(t: float) -> float:
+    return float(lib().o_exp2(t))
+
+
+def fragment_forms(V1, V2, V4, MT3, opacity: float, tile_x0: int, tile_y0: int, tile: int, local_x: int, local_y: int) -> np.ndarray:
+    """(num, den, depth, alpha) of one fragment in the reference's plane form, then in the tile-relative form the
+    forward direction uses; no rejection tests are applied."""
+    out = np.zeros(8, np.float32)
+    lib().oracle_fragment_forms(_p(_f32(V1)), _p(_f32(V2)), _p(_f32(V4)), _p(_f32(MT3)), ctypes.c_float(opacity),
+                                ctypes.c_int(tile_x0), ctypes.c_int(tile_y0), ctypes.c_int(tile), ctypes.c_int(tile),
+                                ctypes.c_int(local_x), ctypes.c_int(local_y), _p(out))
+    return out
 
 
 def preprocess(frame: Frame, positions, scales, rotations, opacities, sh_0, sh_rest, train: bool = False) -> dict:

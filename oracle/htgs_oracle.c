@@ -14,10 +14,18 @@
  *   - the per-Gaussian stage (bounds, VPMT rows, SH colour) uses no fused
  *     operations at all, in the operand order of the reference source;
  *   - the per-pixel stage uses fused multiply-adds exactly where fmaf() is written
- *     below (each is a contraction of the reference expression, never a
- *     re-association);
- *   - logf / expf are the small polynomial routines o_logf / o_expf below
- *     (error about 1 ulp), rsqrtf(x) is 1/sqrtf(x), sqrtf and / are IEEE.
+ *     below;
+ *   - the forward direction of the per-pixel stage (inference, training forward,
+ *     update_max_weights) evaluates the reference's ray / Gaussian expressions in
+ *     tile-relative form: |m|^2, |d|^2 and MT3.(d x m) are exact quadratic
+ *     polynomials of the pixel offset from the tile centre, whose 18 coefficients
+ *     are computed once per (Gaussian, tile) from the plane equations at the tile
+ *     centre (tile_poly_setup).  It is the same rational function of the pixel as
+ *     the reference's plane form and has the same fp32 error against float64
+ *     (both are dominated by the cancellation in VPMT1 - x VPMT4); the backward
+ *     pass keeps the plane form (eval_fragment), whose intermediates it needs;
+ *   - logf / expf / 2^x are the small polynomial routines o_logf / o_expf /
+ *     o_exp2 below, rsqrtf(x) is 1/sqrtf(x), sqrtf and / are IEEE.
  *
  * Parity status of each function is listed next to it ("pinned by ...").  Nothing
  * here can be pinned by reference-held vectors: the reference ships no tests,
@@ -126,6 +134,23 @@ O_EXPORT float o_expf(float x)
     const float y = fmaf(p, r2, r) + 1.0f;
     const int32_t ni = (int32_t)n;
     return bits_to_float((uint32_t)((int32_t)float_to_bits(y) + ni * 8388608));
+}
+
+/* 2^t for t in [-126, 1): n = rint(t), r = t - n (exact), degree-5 polynomial of 2^r on [-1/2, 1/2]
+ * (interpolated at Chebyshev nodes, relative error 2.7e-7), scaled by 2^n through the exponent field.
+ * pinned by: tests compare with 2.0**t in float64 on [-20, 0.5] (<= 3e-7 relative). */
+O_EXPORT float o_exp2(float t)
+{
+    const float n = rintf(t);
+    const float r = t - n;
+    float p = 1.3381302124e-3f;
+    p = fmaf(p, r, 9.6663683653e-3f);
+    p = fmaf(p, r, 5.5503811687e-2f);
+    p = fmaf(p, r, 2.4022349715e-1f);
+    p = fmaf(p, r, 6.9314718246e-1f);
+    p = fmaf(p, r, 1.0f);
+    const int32_t ni = (int32_t)n;
+    return bits_to_float((uint32_t)((int32_t)float_to_bits(p) + ni * 8388608));
 }
 
 static inline float clamp_pos(float v) { return v > 0.0f ? v : 0.0f; }              /* fmaxf(v, 0) with NaN -> 0 */
@@ -457,11 +482,143 @@ static inline int eval_fragment(const float *V1, const float *V2, const float *V
     return 1;
 }
 
+/* ---- tile-relative form of the same evaluation (forward direction) -------------------------------
+ * With px = px0 - dx VPMT4 and py = py0 - dy VPMT4, where px0 / py0 are the planes through the tile
+ * centre and (dx, dy) the pixel's offset from it, the reference's
+ *     d = cross(px.n, py.n)            = A  + dy B  + dx C
+ *     m = px.w py.n - px.n py.w        = Am + dy Bm + dx Cm
+ * are linear in (dx, dy) (the dx dy terms cancel), so |m|^2, |d|^2 and MT3.n . cross(d, m) are quadratic
+ * polynomials.  Coefficient order: 1, dx, dy, dx^2, dx dy, dy^2. */
+typedef struct { float n[6], d[6], z[6]; } tile_poly;
+typedef struct { float X, Y; } pixel_terms;
+
+#define NEG_HALF_LOG2E (-0.72134752044448170f)   /* -0.5 log2(e): G = exp(-rho^2 / 2) = 2^(rho^2 * this) */
+
+static inline void cross3(const float *a, const float *b, float *o)
+{
+    o[0] = fmaf(a[1], b[2], -(a[2] * b[1]));
+    o[1] = fmaf(a[2], b[0], -(a[0] * b[2]));
+    o[2] = fmaf(a[0], b[1], -(a[1] * b[0]));
+}
+static inline float dotf(const float *a, const float *b) { return fmaf(a[2], b[2], fmaf(a[1], b[1], a[0] * b[0])); }
+
+/* pinned by: the images, depths and weights built from it are compared with the float64 closed form
+ * (tests/test_oracle_pinning.py), and with the plane form fragment by fragment (same file). */
+static void tile_poly_setup(const float *V1, const float *V2, const float *V4, const float *MT3,
+                            float cx, float cy, int with_depth, tile_poly *q)
+{
+    float px0[4], py0[4];
+    for (int k = 0; k < 4; ++k) {
+        px0[k] = fmaf(-V4[k], cx, V1[k]);
+        py0[k] = fmaf(-V4[k], cy, V2[k]);
+    }
+    float A[3], B[3], C[3], Am[3], Bm[3], Cm[3];
+    cross3(px0, py0, A);
+    cross3(V4, px0, B);
+    cross3(py0, V4, C);
+    for (int k = 0; k < 3; ++k) {
+        Am[k] = fmaf(px0[3], py0[k], -(px0[k] * py0[3]));
+        Bm[k] = fmaf(px0[k], V4[3], -(px0[3] * V4[k]));
+        Cm[k] = fmaf(V4[k], py0[3], -(V4[3] * py0[k]));
+    }
+    q->n[0] = dotf(Am, Am); q->n[1] = 2.0f * dotf(Am, Cm); q->n[2] = 2.0f * dotf(Am, Bm);
+    q->n[3] = dotf(Cm, Cm); q->n[4] = 2.0f * dotf(Bm, Cm); q->n[5] = dotf(Bm, Bm);
+    q->d[0] = dotf(A, A); q->d[1] = 2.0f * dotf(A, C); q->d[2] = 2.0f * dotf(A, B);
+    q->d[3] = dotf(C, C); q->d[4] = 2.0f * dotf(B, C); q->d[5] = dotf(B, B);
+    for (int k = 0; k < 6; ++k) q->z[k] = 0.0f;
+    if (with_depth) {
+        float PA[3], PB[3], PC[3];       /* MT3.n . cross(d, m) = cross(MT3.n, d) . m */
+        cross3(MT3, A, PA);
+        cross3(MT3, B, PB);
+        cross3(MT3, C, PC);
+        q->z[0] = dotf(PA, Am); q->z[1] = dotf(PA, Cm) + dotf(PC, Am); q->z[2] = dotf(PA, Bm) + dotf(PB, Am);
+        q->z[3] = dotf(PC, Cm); q->z[4] = dotf(PB, Cm) + dotf(PC, Bm); q->z[5] = dotf(PB, Bm);
+    }
+}
+
+static inline pixel_terms pixel_terms_of(int local_x, int local_y, int tile_w, int tile_h)
+{
+    pixel_terms p;
+    p.X = (float)local_x - 0.5f * (float)(tile_w - 1);       /* exact: multiples of 1/2 */
+    p.Y = (float)local_y - 0.5f * (float)(tile_h - 1);
+    return p;
+}
+
+static inline float quad_eval(const float *c, const pixel_terms *p)
+{
+    const float tx = fmaf(c[4], p->Y, fmaf(c[3], p->X, c[1]));     /* c0 + X (cx + cxx X + cxy Y) + Y (cy + cyy Y) */
+    const float ty = fmaf(c[5], p->Y, c[2]);
+    return fmaf(p->Y, ty, fmaf(p->X, tx, c[0]));
+}
+
+/* eval_fragment in tile-relative form; fills num, den, den_rcp, G, alpha and (if asked) depth. */
+static inline int eval_fragment_tile(const tile_poly *q, float depth_centre, float opacity, const pixel_terms *p,
+                                     float cutoff_sq, float min_alpha, int need_depth, const float *depth_limit, fragment *o)
+{
+    o->num = quad_eval(q->n, p);
+    o->den = quad_eval(q->d, p);
+    if (o->num > cutoff_sq * o->den) return 0;
+    o->den_rcp = 1.0f / o->den;
+    if (depth_limit) {
+        o->depth = fmaf(quad_eval(q->z, p), o->den_rcp, depth_centre);
+        if (o->depth >= *depth_limit) return 0;
+    }
+    o->G = o_exp2((o->num * NEG_HALF_LOG2E) * o->den_rcp);
+    const float a = opacity * o->G;
+    o->alpha = a < MAX_FRAGMENT_ALPHA ? a : MAX_FRAGMENT_ALPHA;
+    if (o->alpha < min_alpha) return 0;
+    if (need_depth && !depth_limit) o->depth = fmaf(quad_eval(q->z, p), o->den_rcp, depth_centre);
+    return 1;
+}
+
+/* Test hook: both forms of one fragment, without any rejection.  out = plane form (num, den, depth, alpha),
+ * then tile-relative form (num, den, depth, alpha); tile_x0 / tile_y0 is the tile's first pixel. */
+O_EXPORT void oracle_fragment_forms(const float *V1, const float *V2, const float *V4, const float *MT3, float opacity,
+                                    int tile_x0, int tile_y0, int tile_w, int tile_h, int local_x, int local_y, float out[8])
+{
+    fragment f;
+    eval_fragment(V1, V2, V4, MT3, opacity, (float)(tile_x0 + local_x), (float)(tile_y0 + local_y), INFINITY, -1.0f, 1, NULL, &f);
+    out[0] = f.num; out[1] = f.den; out[2] = f.depth; out[3] = f.alpha;
+    tile_poly q;
+    tile_poly_setup(V1, V2, V4, MT3, (float)tile_x0 + 0.5f * (float)(tile_w - 1), (float)tile_y0 + 0.5f * (float)(tile_h - 1), 1, &q);
+    const pixel_terms p = pixel_terms_of(local_x, local_y, tile_w, tile_h);
+    eval_fragment_tile(&q, MT3[3], opacity, &p, INFINITY, -1.0f, 1, NULL, &f);
+    out[4] = f.num; out[5] = f.den; out[6] = f.depth; out[7] = f.alpha;
+}
+
 typedef struct {
     const uint32_t *ranges;      /* [n_tiles][2] */
     const uint32_t *inst;        /* sorted primitive indices */
     const float *VPMT1, *VPMT2, *VPMT4, *MT3, *rgba;
+    const tile_poly *tp;         /* forward direction: tile-relative form of the current tile's instances [last - first] */
+    uint32_t tp_first;
+    int tile_w, tile_h;
 } blend_in;
+
+/* tile-relative form of every instance of tile t; caller frees */
+static tile_poly *tile_polys(const oracle_cam *c, const blend_in *in, int t, int with_depth)
+{
+    const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
+    const uint32_t first = in->ranges[2 * t], last = in->ranges[2 * t + 1];
+    const float cx = (float)((t % grid_w) * c->tile_w) + 0.5f * (float)(c->tile_w - 1);
+    const float cy = (float)((t / grid_w) * c->tile_h) + 0.5f * (float)(c->tile_h - 1);
+    tile_poly *tp = (tile_poly *)malloc(sizeof(tile_poly) * (last > first ? last - first : 1));
+    for (uint32_t j = first; j < last; ++j) {
+        const size_t g = in->inst[j];
+        tile_poly_setup(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, cx, cy, with_depth, &tp[j - first]);
+    }
+    return tp;
+}
+
+/* fragment j of the current tile at pixel (x, y) */
+static inline int eval_instance(const blend_in *in, uint32_t j, int x, int y, float cutoff_sq, float min_alpha,
+                                int need_depth, const float *depth_limit, fragment *o)
+{
+    const size_t g = in->inst[j];
+    const pixel_terms p = pixel_terms_of(x % in->tile_w, y % in->tile_h, in->tile_w, in->tile_h);
+    return eval_fragment_tile(&in->tp[j - in->tp_first], in->MT3[4 * g + 3], in->rgba[4 * g + 3], &p,
+                              cutoff_sq, min_alpha, need_depth, depth_limit, o);
+}
 
 #define KMAX 32
 static int round_k(int K) { return K >= 32 ? 32 : K >= 16 ? 16 : K >= 8 ? 8 : K >= 4 ? 4 : K >= 2 ? 2 : 1; }  /* inference.cu:22-27 */
@@ -481,7 +638,6 @@ static inline void store_pixel(float *image, float *depths, int w, int h, int x,
 static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                          int x, int y, int K, int median, float out[5])
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
     float T_tail = 1.0f, tail[4] = { 0, 0, 0, 0 }, depth_tail = 0.0f;
     float core[KMAX][4], core_depth[KMAX];
@@ -490,8 +646,7 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
-                           fx, fy, cutoff, min_alpha, 1, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
         float pm[4] = { col[0] * f.alpha, col[1] * f.alpha, col[2] * f.alpha, f.alpha };       /* :158 */
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {                          /* :159 */
@@ -530,7 +685,6 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
 static void first_k_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                           int x, int y, int K, int median, float out[5])
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
     float core_alpha[KMAX], core_depth[KMAX];
     uint32_t core_idx[KMAX];
@@ -538,8 +692,7 @@ static void first_k_pixel(const oracle_cam *c, const blend_in *in, uint32_t firs
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
-                           fx, fy, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
         float depth = f.depth, alpha = f.alpha;
         uint32_t idx = (uint32_t)g;
         for (int i = 0; i < K; ++i) {
@@ -569,15 +722,13 @@ static void first_k_pixel(const oracle_cam *c, const blend_in *in, uint32_t firs
 static void global_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                          int x, int y, int median, float out[5])
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
     float rgb[3] = { 0, 0, 0 }, depth_pixel = 0.0f, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
-                           fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
         const float wgt = T * f.alpha;
         for (int k = 0; k < 3; ++k) rgb[k] = fmaf(wgt, col[k], rgb[k]);
         const float depth = in->MT3[4 * g + 3];                                                /* primitive_depths */
@@ -594,15 +745,13 @@ static void global_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
 static void oit_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                       int x, int y, float out[5])
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
     float acc[4] = { 0, 0, 0, 0 }, alpha_sum = 0.0f, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
-                           fx, fy, cutoff, min_alpha, 1, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, NULL, &f)) continue;
         for (int k = 0; k < 3; ++k) acc[k] = fmaf(f.alpha, col[k], acc[k]);                    /* :147 */
         acc[3] = fmaf(f.alpha, f.depth, acc[3]);
         alpha_sum += f.alpha;
@@ -630,12 +779,16 @@ O_EXPORT void oracle_blend(
 {
     const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
     const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
-    const blend_in in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba };
+    const blend_in frame_in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba, NULL, 0, c->tile_w, c->tile_h };
     const int K = round_k(c->K);
     #pragma omp parallel for schedule(dynamic, 4)
     for (int t = 0; t < grid_w * grid_h; ++t) {
         const int tx = t % grid_w, ty = t / grid_w;
         const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        blend_in in = frame_in;
+        tile_poly *tp = tile_polys(c, &frame_in, t, c->mode != MODE_GLOBAL);
+        in.tp = tp;
+        in.tp_first = first;
         for (int ly = 0; ly < c->tile_h; ++ly)
             for (int lx = 0; lx < c->tile_w; ++lx) {
                 const int x = tx * c->tile_w + lx, y = ty * c->tile_h + ly;
@@ -650,6 +803,7 @@ O_EXPORT void oracle_blend(
                 store_pixel(image, depths, c->width, c->height, x, y, to_chw, out[0], out[1], out[2], out[3], 1);
                 if (alpha_out) alpha_out[(size_t)c->width * y + x] = out[4];
             }
+        free(tp);
     }
 }
 
@@ -670,7 +824,6 @@ O_EXPORT void oracle_blend(
 static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, size_t pix, size_t np,
                                  float rgb_out[3], uint32_t *core_idx_out, float *core_info_out, float *tail_info_out)
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
     float T_tail = 1.0f, tail[4] = { 0, 0, 0, 0 };
     float core[KMAX][4], core_depth[KMAX];
@@ -680,8 +833,7 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
-                           fx, fy, cutoff, min_alpha, 1, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
         float c[4] = { col[0], col[1], col[2], f.alpha };                                      /* :160 */
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {
@@ -738,7 +890,6 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
 static void first_k_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, size_t pix, size_t np,
                                   float rgb_out[3], uint32_t *core_idx_out, float *core_info_out)
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
     float core_alpha[KMAX], core_depth[KMAX];
     uint32_t core_idx[KMAX];
@@ -746,8 +897,7 @@ static void first_k_pixel_forward(const blend_in *in, uint32_t first, uint32_t l
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
-                           fx, fy, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
         float depth = f.depth, alpha = f.alpha;
         uint32_t idx = (uint32_t)g;
         for (int i = 0; i < K; ++i) {
@@ -788,15 +938,13 @@ static void first_k_pixel_forward(const blend_in *in, uint32_t first, uint32_t l
 /* blend_cu (forward) of ALPHA_BLEND_GLOBAL_ORDERING, R/include/alpha_blend_global_ordering/kernels/forward.cuh:103-153 */
 static void global_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, float rgb_out[3])
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
     float rgb[3] = { 0, 0, 0 }, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
-                           fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
         const float bw = T * f.alpha;
         for (int k = 0; k < 3; ++k) rgb[k] = fmaf(bw, col[k], rgb[k]);
         T *= 1.0f - f.alpha;
@@ -809,15 +957,13 @@ static void global_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
 static void oit_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, size_t pix, size_t np,
                               float rgb_out[3], float *tail_info_out)
 {
-    const float fx = (float)x, fy = (float)y;
     const float cutoff = mode_cutoff_sq(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
     float acc[3] = { 0, 0, 0 }, alpha_sum = 0.0f, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, col[3],
-                           fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
         for (int k = 0; k < 3; ++k) acc[k] = fmaf(f.alpha, col[k], acc[k]);
         alpha_sum += f.alpha;
         T *= 1.0f - f.alpha;
@@ -841,13 +987,17 @@ O_EXPORT void oracle_blend_forward(
 {
     const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
     const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
-    const blend_in in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba };
+    const blend_in frame_in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba, NULL, 0, c->tile_w, c->tile_h };
     const int K = round_k(c->K);
     const size_t np = (size_t)c->width * c->height;
     #pragma omp parallel for schedule(dynamic, 4)
     for (int t = 0; t < grid_w * grid_h; ++t) {
         const int tx = t % grid_w, ty = t / grid_w;
         const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        blend_in in = frame_in;
+        tile_poly *tp = tile_polys(c, &frame_in, t, c->mode == MODE_HYBRID || c->mode == MODE_FIRST_K);
+        in.tp = tp;
+        in.tp_first = first;
         for (int ly = 0; ly < c->tile_h; ++ly)
             for (int lx = 0; lx < c->tile_w; ++lx) {
                 const int x = tx * c->tile_w + lx, y = ty * c->tile_h + ly;
@@ -862,6 +1012,7 @@ O_EXPORT void oracle_blend_forward(
                 }
                 image[pix] = rgb[0]; image[np + pix] = rgb[1]; image[2 * np + pix] = rgb[2];
             }
+        free(tp);
     }
 }
 
@@ -1245,19 +1396,24 @@ O_EXPORT void oracle_update_max_weights(
     const int K = round_k(c->K);
     const int mode = c->mode;
     const float cutoff = mode_cutoff_sq(mode), min_alpha = mode_min_alpha(mode);
+    const blend_in frame_in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba, NULL, 0, c->tile_w, c->tile_h };
     for (int t = 0; t < grid_w * grid_h; ++t) {
         const int tx = t % grid_w, ty = t / grid_w;
         const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        blend_in tile_in = frame_in;
+        tile_poly *tp = tile_polys(c, &frame_in, t, mode == MODE_HYBRID || mode == MODE_FIRST_K);
+        tile_in.tp = tp;
+        tile_in.tp_first = first;
+        const blend_in *in = &tile_in;
         for (int l = 0; l < c->tile_w * c->tile_h; ++l) {
             const int x = tx * c->tile_w + l % c->tile_w, y = ty * c->tile_h + l / c->tile_w;
             if (x >= c->width || y >= c->height) continue;
-            const float fx = (float)x, fy = (float)y;
             fragment f;
             if (mode == MODE_GLOBAL) {
                 float T = 1.0f;
                 for (uint32_t j = first; j < last; ++j) {
                     const size_t g = inst[j];
-                    if (!eval_fragment(VPMT1 + 4 * g, VPMT2 + 4 * g, VPMT4 + 4 * g, MT3 + 4 * g, rgba[4 * g + 3], fx, fy, cutoff, min_alpha, 0, NULL, &f)) continue;
+                    if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
                     const float w = T * f.alpha;
                     T *= 1.0f - f.alpha;
                     if (!(w < weight_threshold)) max_weight(max_weights, (uint32_t)g, w);
@@ -1272,8 +1428,7 @@ O_EXPORT void oracle_update_max_weights(
             for (uint32_t j = first; j < last; ++j) {
                 const size_t g = inst[j];
                 const float *lim = mode == MODE_FIRST_K ? &core_depth[K - 1] : NULL;
-                if (!eval_fragment(VPMT1 + 4 * g, VPMT2 + 4 * g, VPMT4 + 4 * g, MT3 + 4 * g, rgba[4 * g + 3], fx, fy, cutoff, min_alpha,
-                                   mode != MODE_OIT, lim, &f)) continue;
+                if (!eval_instance(in, j, x, y, cutoff, min_alpha, mode != MODE_OIT, lim, &f)) continue;
                 float depth = f.depth, alpha = f.alpha;
                 if (mode == MODE_FIRST_K || (mode == MODE_HYBRID && depth < core_depth[K - 1] && alpha >= MIN_ALPHA_CORE)) {
                     uint32_t idx = (uint32_t)g;
@@ -1304,23 +1459,17 @@ O_EXPORT void oracle_update_max_weights(
             /* second pass: every fragment that passes the cut-off gets alpha * tail_weight; no alpha threshold here */
             for (uint32_t j = first; j < last; ++j) {
                 const size_t g = inst[j];
-                for (int k = 0; k < 4; ++k) {
-                    f.px[k] = fmaf(-VPMT4[4 * g + k], fx, VPMT1[4 * g + k]);
-                    f.py[k] = fmaf(-VPMT4[4 * g + k], fy, VPMT2[4 * g + k]);
-                }
-                for (int k = 0; k < 3; ++k) f.m[k] = fmaf(f.px[3], f.py[k], -(f.px[k] * f.py[3]));
-                f.d[0] = fmaf(f.px[1], f.py[2], -(f.px[2] * f.py[1]));
-                f.d[1] = fmaf(f.px[2], f.py[0], -(f.px[0] * f.py[2]));
-                f.d[2] = fmaf(f.px[0], f.py[1], -(f.px[1] * f.py[0]));
-                f.num = fmaf(f.m[2], f.m[2], fmaf(f.m[1], f.m[1], f.m[0] * f.m[0]));
-                f.den = fmaf(f.d[2], f.d[2], fmaf(f.d[1], f.d[1], f.d[0] * f.d[0]));
+                const pixel_terms pt = pixel_terms_of(x % c->tile_w, y % c->tile_h, c->tile_w, c->tile_h);
+                f.num = quad_eval(tp[j - first].n, &pt);
+                f.den = quad_eval(tp[j - first].d, &pt);
                 if (f.num > cutoff * f.den) continue;
-                const float G = o_expf((-0.5f * f.num) * (1.0f / f.den));
+                const float G = o_exp2((f.num * NEG_HALF_LOG2E) * (1.0f / f.den));
                 const float a = rgba[4 * g + 3] * G;
                 const float w = (a < MAX_FRAGMENT_ALPHA ? a : MAX_FRAGMENT_ALPHA) * tail_weight;
                 if (w < weight_threshold) continue;
                 max_weight(max_weights, (uint32_t)g, w);
             }
         }
+        free(tp);
     }
 }

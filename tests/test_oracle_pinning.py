@@ -44,6 +44,53 @@ def test_expf_matches_libm():
     assert oracle.expf(0.0) == 1.0
 
 
+def test_exp2_matches_float64():
+    ts = np.linspace(-20.0, 0.5, 20501).astype(np.float32)
+    worst = max(abs(oracle.exp2(float(t)) / 2.0 ** float(t) - 1.0) for t in ts)
+    assert worst <= 3e-7, worst
+    assert oracle.exp2(0.0) == 1.0 and oracle.exp2(-3.0) == 0.125
+
+
+def test_tile_relative_form_matches_plane_form_and_float64():
+    """The forward direction evaluates |m|^2, |d|^2 and the depth numerator as quadratics of the pixel offset from
+    the tile centre.  Fragment by fragment this must be the reference's plane form: both are compared with a
+    float64 evaluation of the plane form (from the same float32 VPMT rows); the tile-relative form has to stay at
+    the error level of the plane form (a few float32 roundings of rho^2)."""
+    sc = make_scene(1, 4000)
+    out = oracle.render(oracle_frame(sc, 0, 16), *[t.numpy() for t in sc.gaussians()])
+    pre, keys, vals = out["pre"], out["sorted_keys"], out["sorted_vals"]
+    rng = np.random.default_rng(1)
+    gw = (sc.width + 7) // 8
+    err_plane, err_tile = [], []
+    for tile_edge in (8, 16):
+        for j in rng.choice(len(vals), 1500, replace=False):
+            g, t = int(vals[j]), int(keys[j])
+            x0, y0 = (t % gw) * 8, (t // gw) * 8
+            V1, V2, V4, MT3 = (pre[k][g] for k in ("VPMT1", "VPMT2", "VPMT4", "MT3"))
+            lx, ly = (int(v) for v in rng.integers(0, tile_edge, 2))
+            got = oracle.fragment_forms(V1, V2, V4, MT3, float(pre["rgba"][g, 3]), x0, y0, tile_edge, lx, ly).astype(np.float64)
+            v1, v2, v4, mt = (a.astype(np.float64) for a in (V1, V2, V4, MT3))
+            px, py = v1 - v4 * (x0 + lx), v2 - v4 * (y0 + ly)
+            m = px[3] * py[:3] - px[:3] * py[3]
+            d = np.cross(px[:3], py[:3])
+            rho2 = m @ m / (d @ d)
+            if rho2 > 11.08:
+                continue
+            depth = mt[:3] @ np.cross(d, m) / (d @ d) + mt[3]
+            alpha = min(float(pre["rgba"][g, 3]) * math.exp(-0.5 * rho2), 1.0)
+            want = np.array([rho2, depth, alpha])
+            err_plane.append(np.abs(np.array([got[0] / got[1], got[2], got[3]]) - want))
+            err_tile.append(np.abs(np.array([got[4] / got[5], got[6], got[7]]) - want))
+    err_plane, err_tile = np.array(err_plane), np.array(err_tile)
+    assert len(err_tile) > 500
+    # absolute errors of rho^2, depth, alpha against float64
+    assert (err_tile.max(0) < np.array([5e-3, 1e-4, 2e-4])).all(), err_tile.max(0)
+    assert (err_plane.max(0) < np.array([5e-3, 1e-4, 2e-4])).all(), err_plane.max(0)
+    assert (err_tile.mean(0) < np.array([1e-5, 2e-6, 2e-7])).all(), err_tile.mean(0)
+    # rho^2 and depth stay within a small factor of the plane form's own error (alpha also carries the 2^x polynomial)
+    assert (err_tile.mean(0)[:2] < 5.0 * err_plane.mean(0)[:2] + 1e-9).all(), (err_tile.mean(0), err_plane.mean(0))
+
+
 # ---------------------------------------------------------------------------------------------------------
 # per-Gaussian stage
 # ---------------------------------------------------------------------------------------------------------
@@ -352,14 +399,17 @@ def test_single_fragment_closed_forms():
 
 @pytest.mark.parametrize("mode", [0, 1, 3])
 def test_image_does_not_depend_on_tile_size(mode):
-    """Per-pixel fragment order is primitive-index order whatever the tiling, so 8x8 and 16x16 tiles must give the
-    very same image, bit for bit; per-tile counts of course differ."""
+    """Per-pixel fragment order is primitive-index order whatever the tiling, so 8x8 and 16x16 tiles give the same
+    image.  The forward evaluation is relative to the tile centre, so the two differ by rounding (and, at the odd
+    pixel, by a fragment that sits on the 1/255 alpha threshold); per-tile counts of course differ."""
     sc = make_scene(0, 3000)
     arrays = [t.numpy() for t in sc.gaussians()]
     a = oracle.render(oracle_frame(sc, mode, 4, tile=8), *arrays)
     b = oracle.render(oracle_frame(sc, mode, 4, tile=16), *arrays)
-    np.testing.assert_array_equal(a["image"], b["image"])
-    np.testing.assert_array_equal(a["depth"], b["depth"])
+    for key, tol in (("image", 1e-5), ("depth", 1e-4)):
+        diff = np.abs(a[key] - b[key])
+        assert np.mean(diff > tol) < 1e-3, (key, np.mean(diff > tol))
+        assert diff.max() < 2e-2, (key, diff.max())
     assert len(a["keys"]) != len(b["keys"])
 
 
