@@ -125,11 +125,31 @@ struct TileFrag {
     float num, den, den_rcp, alpha;
 };
 
+// The per-pixel loops address the staged instance through one VGPR that holds the LDS byte address of q[0][j] and
+// is advanced by an opaque add (the compiler would otherwise rebuild the address from the scalar loop counter
+// before every read).
+struct __attribute__((aligned(16))) Float4Pod { float x, y, z, w; };
+typedef __attribute__((address_space(3))) const Float4Pod lds_float4;
+typedef __attribute__((address_space(3))) const float lds_float;
+template <int N>
+__device__ __forceinline__ uint32_t stage_address(const TileStage<N> &st) { return (uint32_t)(uintptr_t)(lds_float4 *)&st.q[0][0]; }
+__device__ __forceinline__ void stage_advance(uint32_t &addr) { asm volatile("v_add_u32 %0, 16, %0" : "+v"(addr)); }
+template <int N, int ROW>
+__device__ __forceinline__ float4 stage_row(uint32_t addr)
+{
+    lds_float4 *p = (lds_float4 *)(uintptr_t)(addr + ROW * N * 16);
+    return make_float4(p->x, p->y, p->z, p->w);
+}
+template <int N>
+__device__ __forceinline__ float stage_opacity(uint32_t addr) { return *(lds_float *)(uintptr_t)(addr + 4 * N * 16 + 12); }
+template <int N>
+__device__ __forceinline__ uint32_t stage_index(uint32_t addr) { return float_to_bits(*(lds_float *)(uintptr_t)(addr + 5 * N * 16 + 12)); }
+
 // |m|^2 <= cutoff |d|^2 ?  (inference.cuh:147)
 template <int MODE, int N>
-__device__ __forceinline__ bool tile_frag_cutoff(const TileStage<N> &st, int j, const PixelTerms &p, TileFrag &o)
+__device__ __forceinline__ bool tile_frag_cutoff(uint32_t addr, const PixelTerms &p, TileFrag &o)
 {
-    const float4 q0 = st.q[0][j], q1 = st.q[1][j], q2 = st.q[2][j];
+    const float4 q0 = stage_row<N, 0>(addr), q1 = stage_row<N, 1>(addr), q2 = stage_row<N, 2>(addr);
     o.num = quad_eval(q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, p);
     o.den = quad_eval(q1.z, q1.w, q2.x, q2.y, q2.z, q2.w, p);
     return !(o.num > ModeCfg<MODE>::cutoff_sq * o.den);
@@ -137,9 +157,9 @@ __device__ __forceinline__ bool tile_frag_cutoff(const TileStage<N> &st, int j, 
 
 // camera-space depth of the point of maximum contribution (inference.cuh:151-152); needs o.den_rcp
 template <int N>
-__device__ __forceinline__ float tile_frag_depth(const TileStage<N> &st, int j, const PixelTerms &p, const TileFrag &o)
+__device__ __forceinline__ float tile_frag_depth(uint32_t addr, const PixelTerms &p, const TileFrag &o)
 {
-    const float4 q3 = st.q[3][j], q4 = st.q[4][j];
+    const float4 q3 = stage_row<N, 3>(addr), q4 = stage_row<N, 4>(addr);
     return __builtin_fmaf(quad_eval(q3.x, q3.y, q3.z, q3.w, q4.x, q4.y, p), o.den_rcp, q4.z);
 }
 

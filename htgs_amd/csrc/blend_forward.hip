@@ -43,17 +43,18 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
         __syncthreads();
         tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
-        const int nb = last - base < 64u ? (int)(last - base) : 64;
-        for (int j = 0; j < nb; ++j) {
+        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
-            const float4 col = st.q[5][j];
-            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
-            float depth = tile_frag_depth(st, j, pt, f);
+            const float4 col = stage_row<64, 5>(addr);
+            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+            float depth = tile_frag_depth<64>(addr, pt, f);
             float p0 = col.x, p1 = col.y, p2 = col.z, p3 = f.alpha;
             if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
-                uint32_t idx = float_to_bits(st.q[5][j].w);
+                uint32_t idx = stage_index<64>(addr);
 #pragma unroll
                 for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
                     if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
@@ -151,16 +152,17 @@ __global__ void __launch_bounds__(64) blend_first_k_forward_kernel(
         __syncthreads();
         tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
-        const int nb = last - base < 64u ? (int)(last - base) : 64;
-        for (int j = 0; j < nb; ++j) {
+        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
-            float depth = tile_frag_depth(st, j, pt, f);
+            float depth = tile_frag_depth<64>(addr, pt, f);
             if (depth >= cd[K - 1]) continue;
-            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
+            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
             float alpha = f.alpha;
-            uint32_t idx = float_to_bits(st.q[5][j].w);
+            uint32_t idx = stage_index<64>(addr);
 #pragma unroll
             for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
                 if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
@@ -240,13 +242,14 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
         __syncthreads();
         tile_stage_load<64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
-        const int nb = last - base < 64u ? (int)(last - base) : 64;
-        for (int j = 0; j < nb; ++j) {
+        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
-            const float4 col = st.q[5][j];
-            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
+            const float4 col = stage_row<64, 5>(addr);
+            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
             a0 = __builtin_fmaf(f.alpha, col.x, a0);
             a1 = __builtin_fmaf(f.alpha, col.y, a1);
             a2 = __builtin_fmaf(f.alpha, col.z, a2);
@@ -290,12 +293,13 @@ __global__ void __launch_bounds__(256) blend_global_forward_kernel(
         tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
-        for (int j = 0; !done && j < nb; ++j) {
+        uint32_t addr = stage_address(st);
+        for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!tile_frag_cutoff<MODE, 256>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
-            const float4 col = st.q[5][j];
-            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
+            const float4 col = stage_row<256, 5>(addr);
+            if (!tile_frag_alpha<MODE>(stage_opacity<256>(addr), f)) continue;
             const float bw = T * f.alpha;
             r = __builtin_fmaf(bw, col.x, r);
             g = __builtin_fmaf(bw, col.y, g);

@@ -44,21 +44,22 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
         __syncthreads();
         tile_stage_load<64, kCore>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
-        const int nb = last - base < 64u ? (int)(last - base) : 64;
-        for (int j = 0; j < nb; ++j) {
+        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             float depth = 0.0f;
             if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
-                depth = tile_frag_depth(st, j, pt, f);
+                depth = tile_frag_depth<64>(addr, pt, f);
                 if (depth >= cd[KS - 1]) continue;
             }
-            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
+            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
             float alpha = f.alpha;
-            if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth(st, j, pt, f);
+            if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth<64>(addr, pt, f);
             if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
-                uint32_t idx = float_to_bits(st.q[5][j].w);
+                uint32_t idx = stage_index<64>(addr);
 #pragma unroll
                 for (int g0 = 0; g0 < KS; g0 += kInsertGroup) {
                     if (KS > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < KS ? g0 + kInsertGroup - 1 : KS - 1])) continue;
@@ -95,14 +96,15 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
         __syncthreads();
         tile_stage_load<64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
-        const int nb = last - base < 64u ? (int)(last - base) : 64;
-        for (int j = 0; j < nb; ++j) {
+        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!active || !tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!active || !tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
             const float G = d_exp2((f.num * kNegHalfLog2e) * rcp_exact(f.den));
-            const float a = st.q[4][j].w * G;
+            const float a = stage_opacity<64>(addr) * G;
             const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
-            if (!(w < weight_threshold)) raise_max(max_weights, float_to_bits(st.q[5][j].w), w);
+            if (!(w < weight_threshold)) raise_max(max_weights, stage_index<64>(addr), w);
         }
     }
 }
@@ -128,15 +130,16 @@ __global__ void __launch_bounds__(256) max_weights_global_kernel(
         tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
-        for (int j = 0; !done && j < nb; ++j) {
+        uint32_t addr = stage_address(st);
+        for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE>(st, j, pt, f)) continue;
+            if (!tile_frag_cutoff<MODE, 256>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
-            if (!tile_frag_alpha<MODE>(st.q[4][j].w, f)) continue;
+            if (!tile_frag_alpha<MODE>(stage_opacity<256>(addr), f)) continue;
             const float w = T * f.alpha;
             T *= 1.0f - f.alpha;
             if (T < kTransmittanceThreshold) done = true;
-            if (!(w < weight_threshold)) raise_max(max_weights, float_to_bits(st.q[5][j].w), w);
+            if (!(w < weight_threshold)) raise_max(max_weights, stage_index<256>(addr), w);
         }
     }
 }
