@@ -40,9 +40,31 @@ __global__ void __launch_bounds__(256) copy_bytes_kernel(const uint4 *__restrict
     if (i < n) dst[i] = src[i];
 }
 
+// every positive float whose exponent field is in [7, 247]: refined reciprocal against the division
+__global__ void __launch_bounds__(256) check_reciprocal_kernel(unsigned long long *__restrict__ counts)
+{
+    const uint32_t tid = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
+    unsigned long long tested = 0, wrong = 0;
+    for (uint64_t u = tid; u < 0x80000000ull; u += stride) {
+        const float x = bits_to_float((uint32_t)u);
+        if (!rcp_in_range(x)) continue;
+        ++tested;
+        if (float_to_bits(rcp_refined(x)) != float_to_bits(1.0f / x)) ++wrong;
+    }
+    atomicAdd(counts, tested);
+    if (wrong) atomicAdd(counts + 1, wrong);
+}
+
 }  // namespace htgs
 
 using namespace htgs;
+
+extern "C" int htgs_check_reciprocal(unsigned long long *counts, void *stream)
+{
+    if (!counts) return fail(HTGS_ERR_ARGUMENT, "htgs_check_reciprocal: null pointer");
+    hipLaunchKernelGGL(check_reciprocal_kernel, dim3(4096), dim3(256), 0, (hipStream_t)stream, counts);
+    return check_launch("check_reciprocal");
+}
 
 extern "C" int htgs_copy_bytes(void *dst, const void *src, size_t n_bytes, void *stream)
 {

@@ -48,7 +48,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         {
             // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
@@ -56,7 +56,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             uint32_t addr = stage_address(st);
             for (int j = 0; j < nb; ++j, stage_advance(addr)) {
                 TileFrag f;
-                if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+                if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
                 f.den_rcp = rcp_exact(f.den);
                 const float4 col = stage_row<64, 5>(addr);
                 if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
@@ -138,14 +138,14 @@ __global__ void __launch_bounds__(64) blend_first_k_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         {
             const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
             uint32_t addr = stage_address(st);
             for (int j = 0; j < nb; ++j, stage_advance(addr)) {
                 TileFrag f;
-                if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+                if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
                 f.den_rcp = rcp_exact(f.den);
                 float depth = tile_frag_depth<64>(addr, pt, f);
                 if (depth >= cd[K - 1]) continue;                      // depth test before the exponential (:151)
@@ -210,14 +210,14 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         {
             const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
             uint32_t addr = stage_address(st);
             for (int j = 0; j < nb; ++j, stage_advance(addr)) {
                 TileFrag f;
-                if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+                if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
                 f.den_rcp = rcp_exact(f.den);
                 const float4 col = stage_row<64, 5>(addr);
                 if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
@@ -265,13 +265,13 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
+        tile_stage_load<MODE, 256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         uint32_t addr = stage_address(st);
         for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 256>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<256>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             const float4 q4 = stage_row<256, 4>(addr);
             if (!tile_frag_alpha<MODE>(q4.w, f)) continue;

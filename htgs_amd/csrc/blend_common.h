@@ -39,7 +39,7 @@ __device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restric
 // so |m|^2, |d|^2 and MT3.n . cross(d, m) are quadratics in (dx, dy).  The lane that stages an instance
 // computes the 18 coefficients once; every pixel then needs 5 fused multiply-adds per quadratic.
 // LDS layout per instance, coefficient order (1, dx, dy, dx^2, dx dy, dy^2):
-//     q[0] = n0 nx ny nxx   q[1] = nxy nyy d0 dx   q[2] = dy dxx dxy dyy
+//     q[0] = n0 nx ny nxx   q[1] = nxy nyy d0 dx   q[2] = dy dxx dxy dyy      (n = |m|^2 / cut-off)
 //     q[3] = z0 zx zy zxx   q[4] = zxy zyy MT3.w opacity   q[5] = r g b (primitive index bits)
 // ---------------------------------------------------------------------------------------------
 template <int N>
@@ -58,7 +58,7 @@ __device__ __forceinline__ float dotf(const float *a, const float *b)
     return __builtin_fmaf(a[2], b[2], __builtin_fmaf(a[1], b[1], a[0] * b[0]));
 }
 
-template <int N, bool DEPTH>
+template <int MODE, int N, bool DEPTH>
 __device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                 uint32_t fetch, uint32_t last, int slot, float cx, float cy)
 {
@@ -83,8 +83,9 @@ __device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *
         Bm[k] = __builtin_fmaf(px0[k], V4[3], -(px0[3] * V4[k]));
         Cm[k] = __builtin_fmaf(V4[k], py0[3], -(V4[3] * py0[k]));
     }
-    st.q[0][slot] = make_float4(dotf(Am, Am), 2.0f * dotf(Am, Cm), 2.0f * dotf(Am, Bm), dotf(Cm, Cm));
-    st.q[1][slot] = make_float4(2.0f * dotf(Bm, Cm), dotf(Bm, Bm), dotf(A, A), 2.0f * dotf(A, C));
+    constexpr float kc = ModeCfg<MODE>::cutoff_rcp;
+    st.q[0][slot] = make_float4(dotf(Am, Am) * kc, (2.0f * dotf(Am, Cm)) * kc, (2.0f * dotf(Am, Bm)) * kc, dotf(Cm, Cm) * kc);
+    st.q[1][slot] = make_float4((2.0f * dotf(Bm, Cm)) * kc, dotf(Bm, Bm) * kc, dotf(A, A), 2.0f * dotf(A, C));
     st.q[2][slot] = make_float4(2.0f * dotf(A, B), dotf(C, C), 2.0f * dotf(B, C), dotf(B, B));
     float zxy = 0.0f, zyy = 0.0f;
     if (DEPTH) {
@@ -146,13 +147,13 @@ template <int N>
 __device__ __forceinline__ uint32_t stage_index(uint32_t addr) { return float_to_bits(*(lds_float *)(uintptr_t)(addr + 5 * N * 16 + 12)); }
 
 // |m|^2 <= cutoff |d|^2 ?  (inference.cuh:147)
-template <int MODE, int N>
+template <int N>
 __device__ __forceinline__ bool tile_frag_cutoff(uint32_t addr, const PixelTerms &p, TileFrag &o)
 {
     const float4 q0 = stage_row<N, 0>(addr), q1 = stage_row<N, 1>(addr), q2 = stage_row<N, 2>(addr);
     o.num = quad_eval(q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, p);
     o.den = quad_eval(q1.z, q1.w, q2.x, q2.y, q2.z, q2.w, p);
-    return !(o.num > ModeCfg<MODE>::cutoff_sq * o.den);
+    return !(o.num > o.den);
 }
 
 // camera-space depth of the point of maximum contribution (inference.cuh:151-152); needs o.den_rcp
@@ -167,7 +168,7 @@ __device__ __forceinline__ float tile_frag_depth(uint32_t addr, const PixelTerms
 template <int MODE>
 __device__ __forceinline__ bool tile_frag_alpha(float opacity, TileFrag &o)
 {
-    const float G = d_exp2((o.num * kNegHalfLog2e) * o.den_rcp);
+    const float G = d_exp2((o.num * ModeCfg<MODE>::exp2_scale) * o.den_rcp);
     const float a = opacity * G;
     o.alpha = a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha;
     return !(o.alpha < ModeCfg<MODE>::min_alpha);

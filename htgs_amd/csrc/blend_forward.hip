@@ -41,13 +41,13 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
         uint32_t addr = stage_address(st);
         for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             const float4 col = stage_row<64, 5>(addr);
             if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
@@ -150,13 +150,13 @@ __global__ void __launch_bounds__(64) blend_first_k_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
         uint32_t addr = stage_address(st);
         for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             float depth = tile_frag_depth<64>(addr, pt, f);
             if (depth >= cd[K - 1]) continue;
@@ -240,13 +240,13 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
         uint32_t addr = stage_address(st);
         for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             const float4 col = stage_row<64, 5>(addr);
             if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
@@ -290,13 +290,13 @@ __global__ void __launch_bounds__(256) blend_global_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
+        tile_stage_load<MODE, 256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         uint32_t addr = stage_address(st);
         for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 256>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<256>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             const float4 col = stage_row<256, 5>(addr);
             if (!tile_frag_alpha<MODE>(stage_opacity<256>(addr), f)) continue;

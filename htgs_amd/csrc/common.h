@@ -32,6 +32,10 @@ template <int MODE> struct ModeCfg {
     static constexpr float min_alpha_rcp = MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K ? 20.0f : 255.0f;
     static constexpr float min_alpha = 1.0f / min_alpha_rcp;
     static constexpr float cutoff_sq = MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K ? 5.99146454711f : 11.0825270903f;
+    // tile-relative form: |m|^2 is staged divided by the cut-off (2 ln 20 resp. 2 ln 255), so the cut-off test is
+    // num > den and exp(-rho^2 / 2) = 2^(-log2(20 or 255) num / den)
+    static constexpr float cutoff_rcp = 1.0f / cutoff_sq;
+    static constexpr float exp2_scale = MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K ? -4.32192809488736235f : -7.99435343685885794f;
 };
 
 inline int tile_size(int mode) { return mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING ? 16 : 8; }
@@ -90,7 +94,6 @@ __device__ __forceinline__ float d_expf(float x)
 }
 
 // 2^t for t in [-126, 1): n = rint(t), r = t - n, degree-5 polynomial of 2^r on [-1/2, 1/2] (relative error 2.7e-7)
-constexpr float kNegHalfLog2e = -0.72134752044448170f;     // exp(-rho^2 / 2) = 2^(rho^2 * this)
 __device__ __forceinline__ float d_exp2(float t)
 {
     const float n = __builtin_rintf(t);

@@ -42,13 +42,13 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, kCore>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, kCore>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
         uint32_t addr = stage_address(st);
         for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             float depth = 0.0f;
             if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
@@ -94,14 +94,14 @@ __global__ void __launch_bounds__(64) max_weights_tile_kernel(
     // second walk over the tile's list: alpha * tail weight for every fragment that passes the cut-off
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
+        tile_stage_load<MODE, 64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
         __syncthreads();
         const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
         uint32_t addr = stage_address(st);
         for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!active || !tile_frag_cutoff<MODE, 64>(addr, pt, f)) continue;
-            const float G = d_exp2((f.num * kNegHalfLog2e) * rcp_exact(f.den));
+            if (!active || !tile_frag_cutoff<64>(addr, pt, f)) continue;
+            const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * rcp_exact(f.den));
             const float a = stage_opacity<64>(addr) * G;
             const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
             if (!(w < weight_threshold)) raise_max(max_weights, stage_index<64>(addr), w);
@@ -127,13 +127,13 @@ __global__ void __launch_bounds__(256) max_weights_global_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        tile_stage_load<256, false>(st, prim, inst, base + t, last, t, cx, cy);
+        tile_stage_load<MODE, 256, false>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         uint32_t addr = stage_address(st);
         for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
-            if (!tile_frag_cutoff<MODE, 256>(addr, pt, f)) continue;
+            if (!tile_frag_cutoff<256>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
             if (!tile_frag_alpha<MODE>(stage_opacity<256>(addr), f)) continue;
             const float w = T * f.alpha;

@@ -177,6 +177,12 @@ int htgs_update_3d_filter(const float *positions, const float *w2c, float *filte
                           int width, int height, float focal_x, float focal_y, float center_x, float center_y,
                           float near_plane, float clipping_tolerance, float distance2filter, void *stream);
 
+/* Self-check, no counterpart in the reference.  The forward blend kernels take 1/|d|^2 as v_rcp_f32 plus one fused
+ * Newton step wherever 2^-120 <= |d|^2 < 2^121 and as the IEEE division elsewhere; this call compares the two on
+ * every float of that range.  counts (device, two 64-bit words, zeroed by the caller) receives the number of inputs
+ * compared (241 * 2^23) and the number that differ (0 on gfx950). */
+int htgs_check_reciprocal(unsigned long long *counts, void *stream);
+
 /* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes (multiple of 16)
  * with one 16-byte load and store per thread.  Hardware counters read on it calibrate the same counters read on
  * the rasterizer's kernels (bench.py --calibrate). */

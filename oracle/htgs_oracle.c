@@ -68,6 +68,10 @@ static float mode_min_alpha_rcp(int mode) { return mode == MODE_FIRST_K ? 20.0f 
 /* 1/255 and 1/20 as the compile-time quotients of the reference's constexpr floats */
 static float mode_min_alpha(int mode) { return mode == MODE_FIRST_K ? (1.0f / 20.0f) : (1.0f / 255.0f); }
 static float mode_cutoff_sq(int mode) { return mode == MODE_FIRST_K ? 5.99146454711f : 11.0825270903f; }
+/* tile-relative form: |m|^2 is carried divided by the cut-off (2 ln 20 resp. 2 ln 255), so that the cut-off test is
+ * num > den and exp(-rho^2 / 2) = 2^(-log2(20 or 255) num / den) */
+static float mode_cutoff_rcp(int mode) { return mode == MODE_FIRST_K ? (1.0f / 5.99146454711f) : (1.0f / 11.0825270903f); }
+static float mode_exp2_scale(int mode) { return mode == MODE_FIRST_K ? -4.32192809488736235f : -7.99435343685885794f; }
 
 O_EXPORT int oracle_num_threads(void)
 {
@@ -492,8 +496,6 @@ static inline int eval_fragment(const float *V1, const float *V2, const float *V
 typedef struct { float n[6], d[6], z[6]; } tile_poly;
 typedef struct { float X, Y; } pixel_terms;
 
-#define NEG_HALF_LOG2E (-0.72134752044448170f)   /* -0.5 log2(e): G = exp(-rho^2 / 2) = 2^(rho^2 * this) */
-
 static inline void cross3(const float *a, const float *b, float *o)
 {
     o[0] = fmaf(a[1], b[2], -(a[2] * b[1]));
@@ -505,7 +507,7 @@ static inline float dotf(const float *a, const float *b) { return fmaf(a[2], b[2
 /* pinned by: the images, depths and weights built from it are compared with the float64 closed form
  * (tests/test_oracle_pinning.py), and with the plane form fragment by fragment (same file). */
 static void tile_poly_setup(const float *V1, const float *V2, const float *V4, const float *MT3,
-                            float cx, float cy, int with_depth, tile_poly *q)
+                            float cx, float cy, float cutoff_rcp, int with_depth, tile_poly *q)
 {
     float px0[4], py0[4];
     for (int k = 0; k < 4; ++k) {
@@ -523,6 +525,7 @@ static void tile_poly_setup(const float *V1, const float *V2, const float *V4, c
     }
     q->n[0] = dotf(Am, Am); q->n[1] = 2.0f * dotf(Am, Cm); q->n[2] = 2.0f * dotf(Am, Bm);
     q->n[3] = dotf(Cm, Cm); q->n[4] = 2.0f * dotf(Bm, Cm); q->n[5] = dotf(Bm, Bm);
+    for (int k = 0; k < 6; ++k) q->n[k] *= cutoff_rcp;
     q->d[0] = dotf(A, A); q->d[1] = 2.0f * dotf(A, C); q->d[2] = 2.0f * dotf(A, B);
     q->d[3] = dotf(C, C); q->d[4] = 2.0f * dotf(B, C); q->d[5] = dotf(B, B);
     for (int k = 0; k < 6; ++k) q->z[k] = 0.0f;
@@ -551,19 +554,20 @@ static inline float quad_eval(const float *c, const pixel_terms *p)
     return fmaf(p->Y, ty, fmaf(p->X, tx, c[0]));
 }
 
-/* eval_fragment in tile-relative form; fills num, den, den_rcp, G, alpha and (if asked) depth. */
+/* eval_fragment in tile-relative form; fills num (= |m|^2 / cut-off), den, den_rcp, G, alpha and (if asked) depth.
+ * apply_cutoff = 0 skips the rejection (test hook). */
 static inline int eval_fragment_tile(const tile_poly *q, float depth_centre, float opacity, const pixel_terms *p,
-                                     float cutoff_sq, float min_alpha, int need_depth, const float *depth_limit, fragment *o)
+                                     float exp2_scale, int apply_cutoff, float min_alpha, int need_depth, const float *depth_limit, fragment *o)
 {
     o->num = quad_eval(q->n, p);
     o->den = quad_eval(q->d, p);
-    if (o->num > cutoff_sq * o->den) return 0;
+    if (apply_cutoff && o->num > o->den) return 0;
     o->den_rcp = 1.0f / o->den;
     if (depth_limit) {
         o->depth = fmaf(quad_eval(q->z, p), o->den_rcp, depth_centre);
         if (o->depth >= *depth_limit) return 0;
     }
-    o->G = o_exp2((o->num * NEG_HALF_LOG2E) * o->den_rcp);
+    o->G = o_exp2((o->num * exp2_scale) * o->den_rcp);
     const float a = opacity * o->G;
     o->alpha = a < MAX_FRAGMENT_ALPHA ? a : MAX_FRAGMENT_ALPHA;
     if (o->alpha < min_alpha) return 0;
@@ -580,10 +584,11 @@ O_EXPORT void oracle_fragment_forms(const float *V1, const float *V2, const floa
     eval_fragment(V1, V2, V4, MT3, opacity, (float)(tile_x0 + local_x), (float)(tile_y0 + local_y), INFINITY, -1.0f, 1, NULL, &f);
     out[0] = f.num; out[1] = f.den; out[2] = f.depth; out[3] = f.alpha;
     tile_poly q;
-    tile_poly_setup(V1, V2, V4, MT3, (float)tile_x0 + 0.5f * (float)(tile_w - 1), (float)tile_y0 + 0.5f * (float)(tile_h - 1), 1, &q);
+    tile_poly_setup(V1, V2, V4, MT3, (float)tile_x0 + 0.5f * (float)(tile_w - 1), (float)tile_y0 + 0.5f * (float)(tile_h - 1),
+                    mode_cutoff_rcp(MODE_HYBRID), 1, &q);
     const pixel_terms p = pixel_terms_of(local_x, local_y, tile_w, tile_h);
-    eval_fragment_tile(&q, MT3[3], opacity, &p, INFINITY, -1.0f, 1, NULL, &f);
-    out[4] = f.num; out[5] = f.den; out[6] = f.depth; out[7] = f.alpha;
+    eval_fragment_tile(&q, MT3[3], opacity, &p, mode_exp2_scale(MODE_HYBRID), 0, -1.0f, 1, NULL, &f);
+    out[4] = f.num * mode_cutoff_sq(MODE_HYBRID); out[5] = f.den; out[6] = f.depth; out[7] = f.alpha;
 }
 
 typedef struct {
@@ -605,19 +610,20 @@ static tile_poly *tile_polys(const oracle_cam *c, const blend_in *in, int t, int
     tile_poly *tp = (tile_poly *)malloc(sizeof(tile_poly) * (last > first ? last - first : 1));
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
-        tile_poly_setup(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, cx, cy, with_depth, &tp[j - first]);
+        tile_poly_setup(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, cx, cy, mode_cutoff_rcp(c->mode),
+                        with_depth, &tp[j - first]);
     }
     return tp;
 }
 
 /* fragment j of the current tile at pixel (x, y) */
-static inline int eval_instance(const blend_in *in, uint32_t j, int x, int y, float cutoff_sq, float min_alpha,
+static inline int eval_instance(const blend_in *in, uint32_t j, int x, int y, float exp2_scale, float min_alpha,
                                 int need_depth, const float *depth_limit, fragment *o)
 {
     const size_t g = in->inst[j];
     const pixel_terms p = pixel_terms_of(x % in->tile_w, y % in->tile_h, in->tile_w, in->tile_h);
     return eval_fragment_tile(&in->tp[j - in->tp_first], in->MT3[4 * g + 3], in->rgba[4 * g + 3], &p,
-                              cutoff_sq, min_alpha, need_depth, depth_limit, o);
+                              exp2_scale, 1, min_alpha, need_depth, depth_limit, o);
 }
 
 #define KMAX 32
@@ -638,7 +644,7 @@ static inline void store_pixel(float *image, float *depths, int w, int h, int x,
 static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                          int x, int y, int K, int median, float out[5])
 {
-    const float cutoff = mode_cutoff_sq(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
+    const float scale = mode_exp2_scale(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
     float T_tail = 1.0f, tail[4] = { 0, 0, 0, 0 }, depth_tail = 0.0f;
     float core[KMAX][4], core_depth[KMAX];
     for (int i = 0; i < K; ++i) { core[i][0] = core[i][1] = core[i][2] = core[i][3] = 0.0f; core_depth[i] = FLT_MAX; }
@@ -646,7 +652,7 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
         float pm[4] = { col[0] * f.alpha, col[1] * f.alpha, col[2] * f.alpha, f.alpha };       /* :158 */
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {                          /* :159 */
@@ -685,14 +691,14 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
 static void first_k_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                           int x, int y, int K, int median, float out[5])
 {
-    const float cutoff = mode_cutoff_sq(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
+    const float scale = mode_exp2_scale(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
     float core_alpha[KMAX], core_depth[KMAX];
     uint32_t core_idx[KMAX];
     for (int i = 0; i < K; ++i) { core_alpha[i] = 0.0f; core_depth[i] = FLT_MAX; core_idx[i] = UINT32_MAX; }
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 1, &core_depth[K - 1], &f)) continue;
         float depth = f.depth, alpha = f.alpha;
         uint32_t idx = (uint32_t)g;
         for (int i = 0; i < K; ++i) {
@@ -722,13 +728,13 @@ static void first_k_pixel(const oracle_cam *c, const blend_in *in, uint32_t firs
 static void global_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                          int x, int y, int median, float out[5])
 {
-    const float cutoff = mode_cutoff_sq(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
+    const float scale = mode_exp2_scale(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
     float rgb[3] = { 0, 0, 0 }, depth_pixel = 0.0f, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 0, NULL, &f)) continue;
         const float wgt = T * f.alpha;
         for (int k = 0; k < 3; ++k) rgb[k] = fmaf(wgt, col[k], rgb[k]);
         const float depth = in->MT3[4 * g + 3];                                                /* primitive_depths */
@@ -745,13 +751,13 @@ static void global_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
 static void oit_pixel(const oracle_cam *c, const blend_in *in, uint32_t first, uint32_t last,
                       int x, int y, float out[5])
 {
-    const float cutoff = mode_cutoff_sq(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
+    const float scale = mode_exp2_scale(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
     float acc[4] = { 0, 0, 0, 0 }, alpha_sum = 0.0f, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 1, NULL, &f)) continue;
         for (int k = 0; k < 3; ++k) acc[k] = fmaf(f.alpha, col[k], acc[k]);                    /* :147 */
         acc[3] = fmaf(f.alpha, f.depth, acc[3]);
         alpha_sum += f.alpha;
@@ -824,7 +830,7 @@ O_EXPORT void oracle_blend(
 static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, size_t pix, size_t np,
                                  float rgb_out[3], uint32_t *core_idx_out, float *core_info_out, float *tail_info_out)
 {
-    const float cutoff = mode_cutoff_sq(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
+    const float scale = mode_exp2_scale(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
     float T_tail = 1.0f, tail[4] = { 0, 0, 0, 0 };
     float core[KMAX][4], core_depth[KMAX];
     uint32_t core_idx[KMAX];
@@ -833,7 +839,7 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
         float c[4] = { col[0], col[1], col[2], f.alpha };                                      /* :160 */
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {
@@ -890,14 +896,14 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
 static void first_k_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, size_t pix, size_t np,
                                   float rgb_out[3], uint32_t *core_idx_out, float *core_info_out)
 {
-    const float cutoff = mode_cutoff_sq(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
+    const float scale = mode_exp2_scale(MODE_FIRST_K), min_alpha = mode_min_alpha(MODE_FIRST_K);
     float core_alpha[KMAX], core_depth[KMAX];
     uint32_t core_idx[KMAX];
     for (int i = 0; i < K; ++i) { core_alpha[i] = 0.0f; core_depth[i] = FLT_MAX; core_idx[i] = UINT32_MAX; }
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 1, &core_depth[K - 1], &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 1, &core_depth[K - 1], &f)) continue;
         float depth = f.depth, alpha = f.alpha;
         uint32_t idx = (uint32_t)g;
         for (int i = 0; i < K; ++i) {
@@ -938,13 +944,13 @@ static void first_k_pixel_forward(const blend_in *in, uint32_t first, uint32_t l
 /* blend_cu (forward) of ALPHA_BLEND_GLOBAL_ORDERING, R/include/alpha_blend_global_ordering/kernels/forward.cuh:103-153 */
 static void global_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, float rgb_out[3])
 {
-    const float cutoff = mode_cutoff_sq(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
+    const float scale = mode_exp2_scale(MODE_GLOBAL), min_alpha = mode_min_alpha(MODE_GLOBAL);
     float rgb[3] = { 0, 0, 0 }, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 0, NULL, &f)) continue;
         const float bw = T * f.alpha;
         for (int k = 0; k < 3; ++k) rgb[k] = fmaf(bw, col[k], rgb[k]);
         T *= 1.0f - f.alpha;
@@ -957,13 +963,13 @@ static void global_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
 static void oit_pixel_forward(const blend_in *in, uint32_t first, uint32_t last, int x, int y, size_t pix, size_t np,
                               float rgb_out[3], float *tail_info_out)
 {
-    const float cutoff = mode_cutoff_sq(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
+    const float scale = mode_exp2_scale(MODE_OIT), min_alpha = mode_min_alpha(MODE_OIT);
     float acc[3] = { 0, 0, 0 }, alpha_sum = 0.0f, T = 1.0f;
     fragment f;
     for (uint32_t j = first; j < last; ++j) {
         const size_t g = in->inst[j];
         const float *col = in->rgba + 4 * g;
-        if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
+        if (!eval_instance(in, j, x, y, scale, min_alpha, 0, NULL, &f)) continue;
         for (int k = 0; k < 3; ++k) acc[k] = fmaf(f.alpha, col[k], acc[k]);
         alpha_sum += f.alpha;
         T *= 1.0f - f.alpha;
@@ -1395,7 +1401,7 @@ O_EXPORT void oracle_update_max_weights(
     const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
     const int K = round_k(c->K);
     const int mode = c->mode;
-    const float cutoff = mode_cutoff_sq(mode), min_alpha = mode_min_alpha(mode);
+    const float scale = mode_exp2_scale(mode), min_alpha = mode_min_alpha(mode);
     const blend_in frame_in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba, NULL, 0, c->tile_w, c->tile_h };
     for (int t = 0; t < grid_w * grid_h; ++t) {
         const int tx = t % grid_w, ty = t / grid_w;
@@ -1413,7 +1419,7 @@ O_EXPORT void oracle_update_max_weights(
                 float T = 1.0f;
                 for (uint32_t j = first; j < last; ++j) {
                     const size_t g = inst[j];
-                    if (!eval_instance(in, j, x, y, cutoff, min_alpha, 0, NULL, &f)) continue;
+                    if (!eval_instance(in, j, x, y, scale, min_alpha, 0, NULL, &f)) continue;
                     const float w = T * f.alpha;
                     T *= 1.0f - f.alpha;
                     if (!(w < weight_threshold)) max_weight(max_weights, (uint32_t)g, w);
@@ -1428,7 +1434,7 @@ O_EXPORT void oracle_update_max_weights(
             for (uint32_t j = first; j < last; ++j) {
                 const size_t g = inst[j];
                 const float *lim = mode == MODE_FIRST_K ? &core_depth[K - 1] : NULL;
-                if (!eval_instance(in, j, x, y, cutoff, min_alpha, mode != MODE_OIT, lim, &f)) continue;
+                if (!eval_instance(in, j, x, y, scale, min_alpha, mode != MODE_OIT, lim, &f)) continue;
                 float depth = f.depth, alpha = f.alpha;
                 if (mode == MODE_FIRST_K || (mode == MODE_HYBRID && depth < core_depth[K - 1] && alpha >= MIN_ALPHA_CORE)) {
                     uint32_t idx = (uint32_t)g;
@@ -1462,8 +1468,8 @@ O_EXPORT void oracle_update_max_weights(
                 const pixel_terms pt = pixel_terms_of(x % c->tile_w, y % c->tile_h, c->tile_w, c->tile_h);
                 f.num = quad_eval(tp[j - first].n, &pt);
                 f.den = quad_eval(tp[j - first].d, &pt);
-                if (f.num > cutoff * f.den) continue;
-                const float G = o_exp2((f.num * NEG_HALF_LOG2E) * (1.0f / f.den));
+                if (f.num > f.den) continue;
+                const float G = o_exp2((f.num * scale) * (1.0f / f.den));
                 const float a = rgba[4 * g + 3] * G;
                 const float w = (a < MAX_FRAGMENT_ALPHA ? a : MAX_FRAGMENT_ALPHA) * tail_weight;
                 if (w < weight_threshold) continue;

@@ -78,3 +78,14 @@ def test_k_dispatch(cuda, mode, K):
     got = gpu_stages(scene.to(cuda), mode, K)
     assert np.abs(got["image"] - ref["image"]).max() <= TOL
     assert np.abs(got["depth"] - ref["depth"]).max() <= TOL
+
+
+def test_refined_reciprocal_equals_division_on_the_whole_guarded_range(cuda):
+    """The blend kernels replace 1 / |d|^2 by v_rcp_f32 plus one fused Newton step inside [2^-120, 2^121) and keep
+    the IEEE division outside; the library compares the two on every float of that range on this device."""
+    from htgs_amd import _native
+    counts = torch.zeros(2, dtype=torch.int64, device=cuda)
+    _native.check(_native.lib().htgs_check_reciprocal(counts.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    tested, wrong = counts.cpu().tolist()
+    assert tested == 241 * 2 ** 23
+    assert wrong == 0
