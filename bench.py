@@ -25,8 +25,15 @@ MODE_NAMES = {0: "HYBRID_BLEND", 1: "ALPHA_BLEND_FIRST_K", 2: "ALPHA_BLEND_GLOBA
 HBM_PEAK_GBS = 8000.0
 # fp32 vector peak as published (157.3 TFLOP/s counts packed FP32; plain FMA issue is half of it)
 FP32_PEAK_TFLOPS = 157.3
-# flops of the mandatory part of one pixel/instance evaluation (the two planes, m, d, |m|^2, |d|^2, cut-off test)
+# flops of the mandatory part of one pixel/instance evaluation as the reference states it (the two planes, m, d,
+# |m|^2, |d|^2, cut-off test: R/include/hybrid_blend/kernels/inference.cuh:137-147).  The kernels reach the same
+# decision with two quadratics (21 flops), so this prices the problem, not the instructions issued.
 FLOPS_PER_EVAL = 46
+# HBM bytes of one blend launch of the default workload: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
+# same counters on a plain 1 GiB copy (fetch x 2.000, write x 1.000); profiles/inference_cfg2_3M_1080p_hybrid_k16.md
+MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 2963344927}
+# share of the blend kernel's duration in which the vector ALU is issuing (SQ_ACTIVE_INST_VALU, same profile)
+MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 0.98}
 
 
 def parse_args():
@@ -198,7 +205,9 @@ def main():
     achieved_tflops = blend_flops / (blend_avg_ms / 1e3) / 1e12
     roofline = {
         "kernel": "blend", "bound": "valu_fp32", "achieved": round(achieved_tflops, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved_tflops / FP32_PEAK_TFLOPS, 4), "traffic": None,
+        "frac": round(achieved_tflops / FP32_PEAK_TFLOPS, 4),
+        "traffic": MEASURED_BLEND_TRAFFIC.get((args.config, args.mode, args.K, args.n)),
+        "valu_busy": MEASURED_BLEND_VALU_BUSY.get((args.config, args.mode, args.K, args.n)),
         "launch_ms": round(blend_avg_ms, 4), "evals_per_launch": tile_px * n_inst,
     }
 
