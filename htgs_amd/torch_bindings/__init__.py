@@ -1,4 +1,4 @@
-from .rasterization import diff_rasterize, rasterize, update_max_weights, RasterizerSettings, RasterizerMode, FrameBuffers
+from .rasterization import diff_rasterize, rasterize, fast_rasterize, update_max_weights, RasterizerSettings, RasterizerMode, FrameBuffers
 from .filter3d import update_3d_filter
 
-__all__ = ['diff_rasterize', 'rasterize', 'update_max_weights', 'RasterizerSettings', 'RasterizerMode', 'update_3d_filter', 'FrameBuffers']
+__all__ = ['diff_rasterize', 'rasterize', 'fast_rasterize', 'update_max_weights', 'RasterizerSettings', 'RasterizerMode', 'update_3d_filter', 'FrameBuffers']

@@ -395,3 +395,22 @@ def rasterize(
                                     to_chw, use_median_depth, pool=pool).run()
     depth = depth.unsqueeze(0) if to_chw else depth.unsqueeze(-1)
     return image, depth
+
+
+def fast_rasterize(
+    positions: torch.Tensor,
+    scales: torch.Tensor,
+    rotations: torch.Tensor,
+    opacities: torch.Tensor,
+    sh_0: torch.Tensor,
+    sh_rest: torch.Tensor,
+    settings: RasterizerSettings,
+    to_chw: bool,
+) -> torch.Tensor:
+    """The reference's benchmark entry (rasterization.py:166-186): image only.  There it is a reduced-precision
+    build of the inference kernels (half-precision core, fast-math); here the exact fp32 kernels are the fast path,
+    so this is ``rasterize`` without the depth map and the image is the one ``rasterize`` returns."""
+    with torch.no_grad():
+        pool = ScratchPool.current(positions.device) if isinstance(positions, torch.Tensor) and positions.is_cuda else None
+        image, _ = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, settings, to_chw, False, pool=pool).run()
+    return image

@@ -150,9 +150,10 @@ int htgs_forward_front(const htgs_frame *f);
 int htgs_forward_back(const htgs_frame *f, int *selector);
 /* blend_cu (forward) of the frame's mode, R/include/<mode>/kernels/forward.cuh */
 int htgs_blend_forward(const htgs_frame *f, int selector);
-/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: accumulates into grad_acc (and dens_helper) */
+/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: writes grad_rows (modes 0, 1, 3) or accumulates into
+ * grad_acc (mode 2), and dens_helper */
 int htgs_blend_backward(const htgs_frame *f, int selector);
-/* preprocess_cu (backward), R/include/hybrid_blend/kernels/backward.cuh:10-102: grad_acc -> the six gradients */
+/* preprocess_cu (backward), R/include/hybrid_blend/kernels/backward.cuh:10-102: grad_rows / grad_acc -> the six gradients */
 int htgs_preprocess_backward(const htgs_frame *f);
 /* <mode>::backward (R/src/hybrid_blend/backward.cu:26-128): blend backward, then preprocess backward */
 int htgs_backward(const htgs_frame *f, int selector);

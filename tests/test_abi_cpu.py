@@ -89,7 +89,9 @@ def test_entry_points_reject_bad_frames_without_touching_the_gpu():
 def test_python_api_surface_and_validation():
     import HTGSCudaBackend.torch_bindings as alias
     import htgs_amd
-    for name in ("rasterize", "RasterizerSettings", "RasterizerMode"):
+    # the reference's export list (HTGSCudaBackend/__init__.py, torch_bindings/__init__.py)
+    for name in ("rasterize", "diff_rasterize", "fast_rasterize", "update_max_weights", "update_3d_filter",
+                 "RasterizerSettings", "RasterizerMode"):
         assert getattr(alias, name) is getattr(htgs_amd, name)
     assert [m.value for m in RasterizerMode] == [0, 1, 2, 3]
     assert RasterizerSettings._fields == ("M", "VPM", "cam_position", "mode", "K", "active_sh_bases", "width", "height",

@@ -89,3 +89,14 @@ def test_refined_reciprocal_equals_division_on_the_whole_guarded_range(cuda):
     tested, wrong = counts.cpu().tolist()
     assert tested == 241 * 2 ** 23
     assert wrong == 0
+
+
+def test_fast_rasterize_is_the_exact_image(cuda):
+    from htgs_amd.torch_bindings import fast_rasterize, rasterize
+    sc = make_scene(0, 5000).to(cuda)
+    for mode in range(4):
+        s = sc.settings(mode, 4)
+        image, _ = rasterize(*sc.gaussians(), s, False, False)
+        fast = fast_rasterize(*sc.gaussians(), s, False)
+        assert fast.shape == (sc.height, sc.width, 3)
+        assert torch.equal(fast, image)
