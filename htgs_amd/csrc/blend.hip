@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 const float4 col = stage_row<64, 5>(addr);
                 if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
                 float depth = tile_frag_depth<64>(addr, pt, f);
-                float p0 = col.x * f.alpha, p1 = col.y * f.alpha, p2 = col.z * f.alpha, p3 = f.alpha;
+                float p0 = col.x, p1 = col.y, p2 = col.z, p3 = f.alpha;       // slots keep colour and alpha apart
                 if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
 #pragma unroll
                     for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
@@ -78,7 +78,10 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                         }
                     }
                 }
-                tail0 += p0; tail1 += p1; tail2 += p2; tail3 += p3;
+                tail0 = __builtin_fmaf(p3, p0, tail0);
+                tail1 = __builtin_fmaf(p3, p1, tail1);
+                tail2 = __builtin_fmaf(p3, p2, tail2);
+                tail3 += p3;
                 if (!median) depth_tail = __builtin_fmaf(depth, p3, depth_tail);
                 T_tail *= 1.0f - p3;
             }
@@ -90,11 +93,12 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         if (T_core >= kTransmittanceThreshold) {
-            r = __builtin_fmaf(T_core, c0[i], r);
-            g = __builtin_fmaf(T_core, c1[i], g);
-            b = __builtin_fmaf(T_core, c2[i], b);
+            const float w = T_core * c3[i];
+            r = __builtin_fmaf(w, c0[i], r);
+            g = __builtin_fmaf(w, c1[i], g);
+            b = __builtin_fmaf(w, c2[i], b);
             if (median) depth_pixel = (T_core > 0.5f && cd[i] < __FLT_MAX__) ? cd[i] : depth_pixel;
-            else depth_pixel = __builtin_fmaf(T_core * c3[i], cd[i], depth_pixel);
+            else depth_pixel = __builtin_fmaf(w, cd[i], depth_pixel);
             T_core *= 1.0f - c3[i];
         }
     }

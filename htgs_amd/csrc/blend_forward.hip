@@ -71,7 +71,10 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
                     }
                 }
             }
-            tail0 += p0 * p3; tail1 += p1 * p3; tail2 += p2 * p3; tail3 += p3;
+            tail0 = __builtin_fmaf(p3, p0, tail0);
+            tail1 = __builtin_fmaf(p3, p1, tail1);
+            tail2 = __builtin_fmaf(p3, p2, tail2);
+            tail3 += p3;
             T_tail *= 1.0f - p3;
         }
     }

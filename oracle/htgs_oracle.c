@@ -654,7 +654,9 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
         const float *col = in->rgba + 4 * g;
         if (!eval_instance(in, j, x, y, scale, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
-        float pm[4] = { col[0] * f.alpha, col[1] * f.alpha, col[2] * f.alpha, f.alpha };       /* :158 */
+        /* the reference premultiplies here (:158); the slot keeps colour and alpha apart, as its training kernel
+         * does (forward.cuh:160), so that the tail takes one fused multiply-add per channel */
+        float pm[4] = { col[0], col[1], col[2], f.alpha };
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {                          /* :159 */
             for (int i = 0; i < K; ++i) {
                 if (depth < core_depth[i]) {
@@ -663,16 +665,18 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
                 }
             }
         }
-        for (int k = 0; k < 4; ++k) tail[k] += pm[k];                                          /* :168 */
+        for (int k = 0; k < 3; ++k) tail[k] = fmaf(pm[3], pm[k], tail[k]);                     /* :168 */
+        tail[3] += pm[3];
         if (!median) depth_tail = fmaf(depth, pm[3], depth_tail);                              /* :169 */
         T_tail *= 1.0f - pm[3];                                                                /* :170 */
     }
     float rgb[3] = { 0, 0, 0 }, depth_pixel = 0.0f, T_core = 1.0f;
     for (int i = 0; i < K && T_core >= TRANSMITTANCE_THRESHOLD; ++i) {                         /* :180 */
-        for (int k = 0; k < 3; ++k) rgb[k] = fmaf(T_core, core[i][k], rgb[k]);
+        const float w = T_core * core[i][3];
+        for (int k = 0; k < 3; ++k) rgb[k] = fmaf(w, core[i][k], rgb[k]);
         const float depth = core_depth[i];
         if (median) depth_pixel = (T_core > 0.5f && depth < FLT_MAX) ? depth : depth_pixel;    /* :184 */
-        else depth_pixel = fmaf(T_core * core[i][3], depth, depth_pixel);                      /* :185 */
+        else depth_pixel = fmaf(w, depth, depth_pixel);                                        /* :185 */
         T_core *= 1.0f - core[i][3];
     }
     float total_alpha = 0.0f;
@@ -852,7 +856,8 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
                 }
             }
         }
-        tail[0] += c[0] * c[3]; tail[1] += c[1] * c[3]; tail[2] += c[2] * c[3]; tail[3] += c[3];   /* :173 */
+        for (int k = 0; k < 3; ++k) tail[k] = fmaf(c[3], c[k], tail[k]);                       /* :173 */
+        tail[3] += c[3];
         T_tail *= 1.0f - c[3];
     }
     float rgb[3] = { 0, 0, 0 }, T_core = 1.0f;
