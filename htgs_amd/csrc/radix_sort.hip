@@ -13,21 +13,25 @@
 
 namespace htgs {
 
-constexpr int kSortThreads = 256;
-constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kSortItems = 16;                              // rounds per wave
-constexpr int kSortTile = kSortThreads * kSortItems;        // 4096 items per block
 constexpr int kRadix = 256;
+constexpr int kDigitWaves = kRadix / kWave;                 // the waves whose threads own one digit each
+constexpr int kScanThreads = 256;
+// Items per block = threads x 16.  Longer blocks give longer runs per digit, i.e. fuller cache lines in the
+// scatter; 8-byte keys stay at 256 threads so that two blocks still fit a CU's LDS.
+template <typename KeyT> struct SortShape { static constexpr int threads = sizeof(KeyT) == 8 ? 256 : 512; };
+constexpr int kSortTileMin = 256 * kSortItems;              // the smallest block (sizes the histogram scratch)
 
 template <typename KeyT>
 __device__ __forceinline__ uint32_t digit_of(KeyT k, int shift, uint32_t mask) { return (uint32_t)(k >> shift) & mask; }
 
 template <typename KeyT>
-__global__ void __launch_bounds__(kSortThreads) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
-                                                                     uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
+__global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
+                                                                                 uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
+    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems;
     __shared__ uint32_t counts[kRadix];
-    counts[threadIdx.x] = 0;
+    if (threadIdx.x < kRadix) counts[threadIdx.x] = 0;
     __syncthreads();
     const uint64_t base = (uint64_t)blockIdx.x * kSortTile;
 #pragma unroll
@@ -36,12 +40,13 @@ __global__ void __launch_bounds__(kSortThreads) digit_histogram_kernel(const Key
         if (i < n) atomicAdd(&counts[digit_of(keys[i], shift, mask)], 1u);
     }
     __syncthreads();
-    hist[(size_t)threadIdx.x * n_blocks + blockIdx.x] = counts[threadIdx.x];
+    if (threadIdx.x < kRadix) hist[(size_t)threadIdx.x * n_blocks + blockIdx.x] = counts[threadIdx.x];
 }
 
 // block d scans row d of hist in place (exclusive) and writes the row total to totals[d]
-__global__ void __launch_bounds__(kSortThreads) digit_row_scan_kernel(uint32_t *__restrict__ hist, uint32_t *__restrict__ totals, uint32_t n_blocks)
+__global__ void __launch_bounds__(kScanThreads) digit_row_scan_kernel(uint32_t *__restrict__ hist, uint32_t *__restrict__ totals, uint32_t n_blocks)
 {
+    constexpr int kSortThreads = kScanThreads, kSortWaves = kScanThreads / kWave;
     __shared__ uint32_t wave_sums[kSortWaves];
     uint32_t *row = hist + (size_t)blockIdx.x * n_blocks;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -72,19 +77,19 @@ __global__ void __launch_bounds__(kSortThreads) digit_row_scan_kernel(uint32_t *
 }
 
 template <typename KeyT>
-__global__ void __launch_bounds__(kSortThreads) digit_scatter_kernel(
+__global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel(
     const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
+    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
     __shared__ uint32_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the wave's base inside the block
     __shared__ uint32_t digit_start[kRadix];           // first slot of each digit in the block-local order
     __shared__ uint32_t global_base[kRadix];           // where the block's run of each digit starts in the output
-    __shared__ uint32_t wave_sums[kSortWaves];
+    __shared__ uint32_t wave_sums[kDigitWaves], wave_sums_g[kDigitWaves];
     __shared__ KeyT local_keys[kSortTile];             // the block's items, grouped by digit, stable
     __shared__ uint32_t local_vals[kSortTile];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-#pragma unroll
-    for (int w = 0; w < kSortWaves; ++w) counts[w][threadIdx.x] = 0;
+    for (int c = threadIdx.x; c < kSortWaves * kRadix; c += kSortThreads) (&counts[0][0])[c] = 0;
     __syncthreads();
 
     const uint64_t block_base = (uint64_t)blockIdx.x * kSortTile;
@@ -117,36 +122,41 @@ __global__ void __launch_bounds__(kSortThreads) digit_scatter_kernel(
     }
     __syncthreads();
 
-    // thread d owns digit d: block-local start of the digit, base of each wave inside it, global start of the run
+    // thread d of the first four waves owns digit d: block-local start of the digit, base of each wave inside it,
+    // global start of the run
     {
-        const uint32_t d = threadIdx.x;
+        const bool owner = threadIdx.x < kRadix;
+        const uint32_t d = threadIdx.x & (kRadix - 1);
         uint32_t block_count = 0;
+        if (owner) {
 #pragma unroll
-        for (int w = 0; w < kSortWaves; ++w) block_count += counts[w][d];
+            for (int w = 0; w < kSortWaves; ++w) block_count += counts[w][d];
+        }
         // exclusive scans over the 256 digits: of this block's counts (local order) and of the global totals
-        uint32_t inc_local = block_count, inc_global = totals[d];
+        uint32_t inc_local = block_count, inc_global = owner ? totals[d] : 0u;
         const uint32_t total = inc_global;
 #pragma unroll
         for (int s = 1; s < kWave; s <<= 1) {
             const uint32_t tl = __shfl_up(inc_local, s, kWave), tg = __shfl_up(inc_global, s, kWave);
             if (lane >= s) { inc_local += tl; inc_global += tg; }
         }
-        __shared__ uint32_t wave_sums_g[kSortWaves];
-        if (lane == kWave - 1) { wave_sums[wave] = inc_local; wave_sums_g[wave] = inc_global; }
+        if (owner && lane == kWave - 1) { wave_sums[wave] = inc_local; wave_sums_g[wave] = inc_global; }
         __syncthreads();
-        uint32_t before_l = 0, before_g = 0;
+        if (owner) {
+            uint32_t before_l = 0, before_g = 0;
 #pragma unroll
-        for (int w = 0; w < kSortWaves; ++w)
-            if (w < wave) { before_l += wave_sums[w]; before_g += wave_sums_g[w]; }
-        const uint32_t start = before_l + inc_local - block_count;
-        digit_start[d] = start;
-        global_base[d] = before_g + inc_global - total + hist[(size_t)d * n_blocks + blockIdx.x];
-        uint32_t run = start;
+            for (int w = 0; w < kDigitWaves; ++w)
+                if (w < wave) { before_l += wave_sums[w]; before_g += wave_sums_g[w]; }
+            const uint32_t start = before_l + inc_local - block_count;
+            digit_start[d] = start;
+            global_base[d] = before_g + inc_global - total + hist[(size_t)d * n_blocks + blockIdx.x];
+            uint32_t run = start;
 #pragma unroll
-        for (int w = 0; w < kSortWaves; ++w) {
-            const uint32_t c = counts[w][d];
-            counts[w][d] = run;
-            run += c;
+            for (int w = 0; w < kSortWaves; ++w) {
+                const uint32_t c = counts[w][d];
+                counts[w][d] = run;
+                run += c;
+            }
         }
     }
     __syncthreads();
@@ -181,6 +191,7 @@ template <typename KeyT>
 static int sort_pairs(const htgs_frame *f, int end_bit, int *selector)
 {
     hipStream_t s = (hipStream_t)f->stream;
+    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems;
     const uint64_t n = f->n_instances;
     const uint32_t n_blocks = (uint32_t)((n + kSortTile - 1) / kSortTile);
     uint32_t *hist = f->sort_tmp;
@@ -192,7 +203,7 @@ static int sort_pairs(const htgs_frame *f, int end_bit, int *selector)
         const KeyT *kin = (const KeyT *)f->keys[cur];
         KeyT *kout = (KeyT *)f->keys[cur ^ 1];
         hipLaunchKernelGGL((digit_histogram_kernel<KeyT>), dim3(n_blocks), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
-        hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kSortThreads), 0, s, hist, totals, n_blocks);
+        hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
         hipLaunchKernelGGL((digit_scatter_kernel<KeyT>), dim3(n_blocks), dim3(kSortThreads), 0, s, kin, f->vals[cur], kout, f->vals[cur ^ 1],
                            hist, totals, n, n_blocks, shift, mask);
         cur ^= 1;
@@ -207,7 +218,7 @@ using namespace htgs;
 
 extern "C" size_t htgs_sort_tmp_words(uint64_t n_instances)
 {
-    const uint64_t n_blocks = (n_instances + kSortTile - 1) / kSortTile;
+    const uint64_t n_blocks = (n_instances + kSortTileMin - 1) / kSortTileMin;
     return (size_t)(kRadix * (n_blocks > 0 ? n_blocks : 1) + kRadix);
 }
 
