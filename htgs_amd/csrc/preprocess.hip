@@ -56,7 +56,7 @@ __device__ __forceinline__ void axis_extent(const float f[4], const Row &Vi, con
     extent = __builtin_sqrtf(clamp_pos(center * center - q));
 }
 
-__global__ void __launch_bounds__(256) preprocess_kernel(
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) preprocess_kernel(
     const float *__restrict__ positions, const float *__restrict__ scales, const float *__restrict__ rotations,
     const float *__restrict__ opacities, const float *__restrict__ sh_0, const float *__restrict__ sh_rest,
     const float *__restrict__ M, const float *__restrict__ VPM_in, const float *__restrict__ cam_position,
@@ -83,6 +83,23 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
     for (int k = 0; k < 16; ++k) VPM[k] = VPM_in[k];
 #pragma unroll
     for (int k = 0; k < 3; ++k) cam[k] = cam_position[k];
+
+    // The block's slice of sh_rest is three quarters of everything this kernel reads.  Its loads are issued first,
+    // into registers, so that they are in flight while the bounds are computed; they reach LDS further down.
+    constexpr int kShRegs = 16;                                    // 16-byte words per thread: 256 x 3 x 21 / 4 / 256
+    const int per = 3 * total_sh;                                  // words per Gaussian
+    const int n_block = n - first < 256 ? n - first : 256;
+    const size_t base_word = (size_t)first * per;                 // multiple of 256 words: 16-byte aligned
+    const int words = active_sh > 1 ? n_block * per : 0;
+    const float4 *src4 = reinterpret_cast<const float4 *>(sh_rest + base_word);
+    float sh_regs[kShRegs][4];
+#pragma unroll
+    for (int k = 0; k < kShRegs; ++k) {
+        const int q = k * 256 + threadIdx.x;
+        float4 t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (q < words / 4) t = src4[q];
+        sh_regs[k][0] = t.x; sh_regs[k][1] = t.y; sh_regs[k][2] = t.z; sh_regs[k][3] = t.w;
+    }
 
     uint32_t touched = 0;
     const size_t ic = in_range ? (size_t)i : 0;
@@ -138,15 +155,12 @@ __global__ void __launch_bounds__(256) preprocess_kernel(
         *reinterpret_cast<ushort4 *>(bounds + 4 * (size_t)i) = make_ushort4((uint16_t)b0, (uint16_t)b1, (uint16_t)b2, (uint16_t)b3);
 
     // stage the block's SH coefficients
-    const int per = 3 * total_sh;                                  // words per Gaussian
-    const int n_block = n - first < 256 ? n - first : 256;
-    if (active_sh > 1) {
-        const size_t base_word = (size_t)first * per;             // multiple of 256 words: 16-byte aligned
-        const int words = n_block * per;
-        const float4 *src4 = reinterpret_cast<const float4 *>(sh_rest + base_word);
-        for (int q = threadIdx.x; q < words / 4; q += 256) lds4[q] = src4[q];
-        for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) lds[q] = sh_rest[base_word + q];
+#pragma unroll
+    for (int k = 0; k < kShRegs; ++k) {
+        const int q = k * 256 + threadIdx.x;
+        if (q < words / 4) lds4[q] = make_float4(sh_regs[k][0], sh_regs[k][1], sh_regs[k][2], sh_regs[k][3]);
     }
+    for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) lds[q] = sh_rest[base_word + q];
     __syncthreads();
 
     // view-dependent colour, kernel_utils.cuh:152-187
