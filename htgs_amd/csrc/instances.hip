@@ -108,6 +108,7 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
 {
     __shared__ uint32_t s_end[256];     // inclusive offsets of the block's Gaussians
     __shared__ uint32_t s_x0[256], s_y0[256], s_w[256], s_depth[DEPTH ? 256 : 1];
+    __shared__ float s_rw[256];         // 1 / width of the rectangle
     const int first = blockIdx.x * 256;
     const int i = first + threadIdx.x;
     const uint32_t block_start = first == 0 ? 0u : offsets[first - 1];
@@ -124,6 +125,7 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
     }
     s_end[threadIdx.x] = end;
     s_x0[threadIdx.x] = x0; s_y0[threadIdx.x] = y0; s_w[threadIdx.x] = w;
+    s_rw[threadIdx.x] = 1.0f / (float)w;
     if (DEPTH) s_depth[threadIdx.x] = depth;
     __syncthreads();
     if ((uint64_t)block_end > capacity) return;          // the caller's n_instances was too small: never write outside
@@ -138,7 +140,17 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
         const uint32_t l = lo;
         const uint32_t t = e - (l == 0 ? block_start : s_end[l - 1]);
         const uint32_t wl = s_w[l];
-        const uint32_t row = t / wl, colm = t - row * wl;
+        // row = t / wl without the integer division: the float quotient is within one of it while t < 2^22
+        uint32_t row;
+        if (t < (1u << 22)) {
+            row = (uint32_t)((float)t * s_rw[l]);
+            const uint32_t prod = row * wl;
+            if (prod > t) --row;
+            else if (prod + wl <= t) ++row;
+        } else {
+            row = t / wl;
+        }
+        const uint32_t colm = t - row * wl;
         const uint64_t tile = (uint64_t)(s_y0[l] + row) * grid_w + s_x0[l] + colm;
         keys[e] = DEPTH ? (KeyT)((tile << 32) | (uint64_t)s_depth[l]) : (KeyT)tile;
         vals[e] = (uint32_t)(first + l);
