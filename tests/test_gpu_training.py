@@ -1,8 +1,8 @@
 """GPU parity of the training path (diff_rasterize): forward image and per-pixel records, then the six gradients
 and the densification side outputs, against the CPU oracle on the same seeded inputs.
 
-Tolerances: image 1e-4 max abs; gradients 1e-3 relative (atomics make the summation order of the GPU path
-non-deterministic).  "Relative" is taken per tensor against its largest reference entry, and element-wise with
+Tolerances: image 1e-4 max abs; gradients 1e-3 relative (the GPU path sums a Gaussian's contributions in another
+order than the oracle; the global-ordering mode also uses float atomics).  "Relative" is taken per tensor against its largest reference entry, and element-wise with
 rtol 1e-3 plus a small absolute term tied to that scale, because individual entries are sums with cancellation."""
 import numpy as np
 import pytest
