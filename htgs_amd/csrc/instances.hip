@@ -157,21 +157,37 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
     }
 }
 
+// A thread takes the keys of one 16-byte word (and the key before them) and writes a range boundary wherever two
+// neighbours differ.
 template <typename KeyT, int SHIFT>
 __global__ void __launch_bounds__(256) extract_ranges_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ ranges, uint64_t n)
 {
-    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    const uint32_t t = (uint32_t)(keys[i] >> SHIFT);
-    if (i == 0) ranges[2 * (size_t)t] = 0;
-    else {
-        const uint32_t tp = (uint32_t)(keys[i - 1] >> SHIFT);
-        if (t != tp) {
-            ranges[2 * (size_t)tp + 1] = (uint32_t)i;
-            ranges[2 * (size_t)t] = (uint32_t)i;
+    constexpr int kPer = 16 / sizeof(KeyT);
+    const uint64_t first = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * kPer;
+    if (first >= n) return;
+    KeyT k[kPer];
+    if (first + kPer <= n) {
+        const uint4 word = *reinterpret_cast<const uint4 *>(keys + first);
+        __builtin_memcpy(k, &word, 16);
+    } else {
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) k[j] = first + j < n ? keys[first + j] : (KeyT)0;
+    }
+    uint32_t tp = first == 0 ? 0u : (uint32_t)(keys[first - 1] >> SHIFT);
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const uint64_t i = first + j;
+        if (i < n) {
+            const uint32_t t = (uint32_t)(k[j] >> SHIFT);
+            if (i == 0) ranges[2 * (size_t)t] = 0;
+            else if (t != tp) {
+                ranges[2 * (size_t)tp + 1] = (uint32_t)i;
+                ranges[2 * (size_t)t] = (uint32_t)i;
+            }
+            if (i == n - 1) ranges[2 * (size_t)t + 1] = (uint32_t)n;
+            tp = t;
         }
     }
-    if (i == n - 1) ranges[2 * (size_t)t + 1] = (uint32_t)n;
 }
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
@@ -240,8 +256,10 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((2 * n_tiles + 255) / 256)), dim3(256), 0, s, f->ranges, 2 * n_tiles);
     if (f->n_instances > 0) {
         if (!f->keys[selector]) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: null pointer");
-        const dim3 grid((unsigned)((f->n_instances + 255) / 256)), block(256);
+        if ((uintptr_t)f->keys[selector] & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: keys must be 16-byte aligned");
         const int kb = htgs_key_bytes(f->mode, f->width, f->height);
+        const uint64_t per_block = 256ull * (16 / kb);
+        const dim3 grid((unsigned)((f->n_instances + per_block - 1) / per_block)), block(256);
         if (kb == 8)
             hipLaunchKernelGGL((extract_ranges_kernel<uint64_t, 32>), grid, block, 0, s, (const uint64_t *)f->keys[selector], f->ranges, f->n_instances);
         else if (kb == 4)

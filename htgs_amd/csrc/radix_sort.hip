@@ -33,11 +33,25 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_histogram_kern
     __shared__ uint32_t counts[kRadix];
     if (threadIdx.x < kRadix) counts[threadIdx.x] = 0;
     __syncthreads();
+    // the order of the keys does not matter here, so every thread reads 16-byte words: kPer keys at a time
     const uint64_t base = (uint64_t)blockIdx.x * kSortTile;
+    constexpr int kPer = 16 / sizeof(KeyT);
+    if (base + kSortTile <= n) {
+        const uint4 *words = reinterpret_cast<const uint4 *>(keys + base);      // kSortTile keys are a multiple of 16 bytes
 #pragma unroll
-    for (int r = 0; r < kSortItems; ++r) {
-        const uint64_t i = base + (uint64_t)r * kSortThreads + threadIdx.x;
-        if (i < n) atomicAdd(&counts[digit_of(keys[i], shift, mask)], 1u);
+        for (int r = 0; r < kSortItems / kPer; ++r) {
+            const uint4 word = words[r * kSortThreads + threadIdx.x];
+            KeyT k[kPer];
+            __builtin_memcpy(k, &word, 16);
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) atomicAdd(&counts[digit_of(k[j], shift, mask)], 1u);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < kSortItems; ++r) {
+            const uint64_t i = base + (uint64_t)r * kSortThreads + threadIdx.x;
+            if (i < n) atomicAdd(&counts[digit_of(keys[i], shift, mask)], 1u);
+        }
     }
     __syncthreads();
     if (threadIdx.x < kRadix) hist[(size_t)threadIdx.x * n_blocks + blockIdx.x] = counts[threadIdx.x];
@@ -231,6 +245,7 @@ extern "C" int htgs_sort_instances(const htgs_frame *f, int *selector)
     if (f->n_instances > 0xffffffffull) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: more than 2^32-1 instances");
     if (!f->keys[0] || !f->keys[1] || !f->vals[0] || !f->vals[1] || !f->sort_tmp)
         return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: null pointer");
+    if (((uintptr_t)f->keys[0] | (uintptr_t)f->keys[1]) & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: keys must be 16-byte aligned");
     const int end_bit = htgs_end_bit(f->mode, f->width, f->height);
     switch (htgs_key_bytes(f->mode, f->width, f->height)) {
         case 8: return sort_pairs<uint64_t>(f, end_bit, selector);

@@ -72,7 +72,7 @@ typedef struct htgs_frame {
     uint32_t *ranges;          /* [n_tiles,2] first,last+1 into the sorted instance list */
     /* ---- per-instance scratch (PerInstanceBuffers, buffer_utils.h:56-84) ---- */
     uint64_t n_instances;      /* host copy of *n_instances_dev, needed from htgs_create_instances on */
-    void *keys[2];             /* [n_instances] of htgs_key_bytes() each, ping-pong */
+    void *keys[2];             /* [n_instances] of htgs_key_bytes() each, ping-pong, 16-byte aligned */
     uint32_t *vals[2];         /* [n_instances] primitive index, ping-pong */
     uint32_t *sort_tmp;        /* htgs_sort_tmp_words(n_instances) words */
     /* ---- outputs (rasterization_api.cu:392-393) ---- */
