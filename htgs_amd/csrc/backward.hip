@@ -302,18 +302,52 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
     float *__restrict__ grad_opacities, float *__restrict__ grad_sh_0, float *__restrict__ grad_sh_rest,
     float *__restrict__ densification_info, int n, int active_sh, int total_sh, int use_distance_scaling, int use_rows)
 {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    float *gsr = grad_sh_rest + 3 * (size_t)total_sh * i;
-    if (n_touched[i] == 0) {                                                     // backward.cuh:31: nothing flows to culled Gaussians
+    // The block's slices of sh_rest and grad_sh_rest are contiguous in memory (256 Gaussians x 3 total_sh words).  They
+    // go through one LDS buffer so that global traffic is coalesced 16-byte words: the coefficients are loaded into
+    // registers first (in flight during the row sums), parked in LDS, read back per Gaussian, and every Gaussian
+    // then overwrites its own slice with its gradient, which the block stores as one run.
+    extern __shared__ float4 lds4[];
+    float *lds = reinterpret_cast<float *>(lds4);
+    const int first = blockIdx.x * 256;
+    const int i = first + threadIdx.x;
+    const int per = 3 * total_sh;                                  // words per Gaussian
+    const int n_block = n - first < 256 ? n - first : 256;
+    const size_t base_word = (size_t)first * per;                 // multiple of 256 words: 16-byte aligned
+    const int words = n_block * per;
+    constexpr int kShRegs = 16;
+    float sh_regs[kShRegs][4];
+    if (active_sh > 1) {
+        const float4 *src4 = reinterpret_cast<const float4 *>(sh_rest + base_word);
+#pragma unroll
+        for (int k = 0; k < kShRegs; ++k) {
+            const int q = k * 256 + threadIdx.x;
+            float4 t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (q < words / 4) t = src4[q];
+            sh_regs[k][0] = t.x; sh_regs[k][1] = t.y; sh_regs[k][2] = t.z; sh_regs[k][3] = t.w;
+        }
+    }
+    float *gsr = lds + per * threadIdx.x;                          // this Gaussian's slice: coefficients in, gradient out
+    const bool live = i < n && n_touched[i] != 0;                  // backward.cuh:31: nothing flows to culled Gaussians
+    if (i < n && !live) {
 #pragma unroll
         for (int k = 0; k < 3; ++k) { grad_positions[3 * (size_t)i + k] = 0.0f; grad_scales[3 * (size_t)i + k] = 0.0f; grad_sh_0[3 * (size_t)i + k] = 0.0f; }
 #pragma unroll
         for (int k = 0; k < 4; ++k) grad_rotations[4 * (size_t)i + k] = 0.0f;
         grad_opacities[i] = 0.0f;
-        for (int k = 0; k < 3 * total_sh; ++k) gsr[k] = 0.0f;
-        return;
     }
+    if (active_sh > 1) {
+#pragma unroll
+        for (int k = 0; k < kShRegs; ++k) {
+            const int q = k * 256 + threadIdx.x;
+            if (q < words / 4) lds4[q] = make_float4(sh_regs[k][0], sh_regs[k][1], sh_regs[k][2], sh_regs[k][3]);
+        }
+        for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) lds[q] = sh_rest[base_word + q];
+    }
+    __syncthreads();
+    float sh_b[15];                                                // basis values of the active bands
+    float g[3] = { 0.0f, 0.0f, 0.0f };
+    int nb = 0;
+    if (live) {
     float a[16];
     float helper_sum = 0.0f;
     if (use_rows) {
@@ -384,21 +418,19 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
 
     // SH, kernel_utils.cuh:190-281
     const float p[3] = { positions[3 * (size_t)i], positions[3 * (size_t)i + 1], positions[3 * (size_t)i + 2] };
-    float g[3];
     g[0] = clamp_info[i] ? 0.0f : a[0];
     g[1] = clamp_info[(size_t)n + i] ? 0.0f : a[1];
     g[2] = clamp_info[2 * (size_t)n + i] ? 0.0f : a[2];
 #pragma unroll
     for (int k = 0; k < 3; ++k) grad_sh_0[3 * (size_t)i + k] = 0.28209479177387814f * g[k];
-    for (int k = 0; k < 3 * total_sh; ++k) gsr[k] = 0.0f;
     if (active_sh > 1) {
-        const float *c = sh_rest + 3 * (size_t)total_sh * i;
+        const float *c = gsr;
         const float xr = p[0] - cam_position[0], yr = p[1] - cam_position[1], zr = p[2] - cam_position[2];
         const float inv = 1.0f / __builtin_sqrtf(xr * xr + yr * yr + zr * zr);
         const float dx_ = xr * inv, dy_ = yr * inv, dz_ = zr * inv;
-        float b[15];
+        float (&b)[15] = sh_b;
         float gx[3], gy[3], gz[3];
-        int nb = 3;
+        nb = 3;
         b[0] = -0.48860251190291987f * dy_; b[1] = 0.48860251190291987f * dz_; b[2] = -0.48860251190291987f * dx_;
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
@@ -438,9 +470,6 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
                 }
             }
         }
-        for (int j = 0; j < nb; ++j) {
-            gsr[3 * j] = b[j] * g[0]; gsr[3 * j + 1] = b[j] * g[1]; gsr[3 * j + 2] = b[j] * g[2];
-        }
         const float gd[3] = { gx[0] * g[0] + gx[1] * g[1] + gx[2] * g[2], gy[0] * g[0] + gy[1] * g[1] + gy[2] * g[2],
                               gz[0] * g[0] + gz[1] * g[1] + gz[2] * g[2] };
         const float XX = xr * xr, YY = yr * yr, ZZ = zr * zr, XY = xr * yr, XZ = xr * zr, YZ = yr * zr;
@@ -460,6 +489,23 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
         densification_info[i] += 1.0f;
         densification_info[(size_t)n + i] += __builtin_sqrtf(v0 * v0 + v1 * v1 + v2 * v2);
         if (helper || helper_rows) densification_info[2 * (size_t)n + i] += z_scale * helper_sum;
+    }
+    }   // live
+
+    // every thread overwrites its slice with dL/dsh_rest (zeros beyond the active bands and for culled Gaussians)
+    if (total_sh > 0) {
+#pragma unroll
+        for (int j = 0; j < 15; ++j) {
+            if (j < total_sh) {
+                const float bj = j < nb ? sh_b[j] : 0.0f;
+                gsr[3 * j] = bj * g[0]; gsr[3 * j + 1] = bj * g[1]; gsr[3 * j + 2] = bj * g[2];
+            }
+        }
+        for (int k = 45; k < per; ++k) gsr[k] = 0.0f;
+        __syncthreads();
+        float4 *dst4 = reinterpret_cast<float4 *>(grad_sh_rest + base_word);
+        for (int q = threadIdx.x; q < words / 4; q += 256) dst4[q] = lds4[q];
+        for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) grad_sh_rest[base_word + q] = lds[q];
     }
 }
 
@@ -545,7 +591,9 @@ extern "C" int htgs_preprocess_backward(const htgs_frame *f)
     const float *helper = (f->densification_info && f->densification_rows == 3) ? f->dens_helper : nullptr;
     if (f->densification_info && f->densification_rows == 3 && !helper && f->n_instances > 0)
         return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: 3-row densification_info needs dens_helper");
-    hipLaunchKernelGGL(preprocess_backward_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), 0, (hipStream_t)f->stream,
+    const size_t lds_bytes = (size_t)256 * 3 * f->total_sh_bases * sizeof(float);
+    if (lds_bytes > 64 * 1024) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: sh_rest has more than 21 coefficients per Gaussian");
+    hipLaunchKernelGGL(preprocess_backward_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), lds_bytes, (hipStream_t)f->stream,
                        f->positions, f->scales, f->rotations, f->sh_rest, f->n_touched, f->clamp_info,
                        rows ? nullptr : f->grad_acc, rows ? (const float4 *)f->grad_rows : nullptr, f->offsets,
                        rows ? nullptr : helper, rows ? helper : nullptr, f->M, f->VPM,
