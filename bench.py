@@ -116,7 +116,7 @@ def main():
     args = parse_args()
     if args.gpus != 1:
         print("bench.py: this build renders one frame on one GPU; --gpus must be 1 "
-              "(sharding is described in DESIGN.md, not implemented)", file=sys.stderr)
+              "(sharding over tile rows is designed, not implemented)", file=sys.stderr)
         sys.exit(2)
     import torch
     from htgs_amd.synthetic import make_scene
