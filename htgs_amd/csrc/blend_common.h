@@ -58,6 +58,46 @@ __device__ __forceinline__ float dotf(const float *a, const float *b)
     return __builtin_fmaf(a[2], b[2], __builtin_fmaf(a[1], b[1], a[0] * b[0]));
 }
 
+// the six vectors of the tile-relative form and what they are built from
+struct TileGeometry {
+    float a[3], aw, b[3], bw, v[3], vw;        // px0 = (a, aw), py0 = (b, bw), VPMT4 = (v, vw)
+    float A[3], B[3], C[3], Am[3], Bm[3], Cm[3];
+};
+__device__ __forceinline__ void tile_geometry(const float4 &r1, const float4 &r2, const float4 &r4, float cx, float cy, TileGeometry &g)
+{
+    const float V1[4] = { r1.x, r1.y, r1.z, r1.w }, V2[4] = { r2.x, r2.y, r2.z, r2.w }, V4[4] = { r4.x, r4.y, r4.z, r4.w };
+    float px0[4], py0[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        px0[k] = __builtin_fmaf(-V4[k], cx, V1[k]);
+        py0[k] = __builtin_fmaf(-V4[k], cy, V2[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) { g.a[k] = px0[k]; g.b[k] = py0[k]; g.v[k] = V4[k]; }
+    g.aw = px0[3]; g.bw = py0[3]; g.vw = V4[3];
+    cross3(px0, py0, g.A);
+    cross3(V4, px0, g.B);
+    cross3(py0, V4, g.C);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        g.Am[k] = __builtin_fmaf(px0[3], py0[k], -(px0[k] * py0[3]));
+        g.Bm[k] = __builtin_fmaf(px0[k], V4[3], -(px0[3] * V4[k]));
+        g.Cm[k] = __builtin_fmaf(V4[k], py0[3], -(V4[3] * py0[k]));
+    }
+}
+// coefficients (1, dx, dy, dx^2, dx dy, dy^2) of |m|^2 / cut-off and of |d|^2
+template <int MODE>
+__device__ __forceinline__ void tile_quadratics(const TileGeometry &g, float (&n)[6], float (&d)[6])
+{
+    constexpr float kc = ModeCfg<MODE>::cutoff_rcp;
+    n[0] = dotf(g.Am, g.Am) * kc; n[1] = (2.0f * dotf(g.Am, g.Cm)) * kc; n[2] = (2.0f * dotf(g.Am, g.Bm)) * kc;
+    n[3] = dotf(g.Cm, g.Cm) * kc; n[4] = (2.0f * dotf(g.Bm, g.Cm)) * kc; n[5] = dotf(g.Bm, g.Bm) * kc;
+    d[0] = dotf(g.A, g.A); d[1] = 2.0f * dotf(g.A, g.C); d[2] = 2.0f * dotf(g.A, g.B);
+    d[3] = dotf(g.C, g.C); d[4] = 2.0f * dotf(g.B, g.C); d[5] = dotf(g.B, g.B);
+}
+
+// (the same arithmetic as tile_geometry / tile_quadratics, written out so that every row is stored as soon as it is
+// complete: the kernels that call this hold a K-buffer in registers)
 template <int MODE, int N, bool DEPTH>
 __device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                 uint32_t fetch, uint32_t last, int slot, float cx, float cy)

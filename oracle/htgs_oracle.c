@@ -1057,11 +1057,22 @@ static void fragment_backward(const fragment *f, float opacity, float dL_dalpha,
     }
 }
 
-/* recomputes G and alpha of a fragment exactly as the forward pass did; 0 if it was rejected */
-static inline int reeval_fragment(const blend_in *in, size_t g, float fx, float fy, int mode, fragment *f)
+/* Accept / reject and alpha of a fragment exactly as the forward pass decided them (tile-relative form), then the
+ * plane-form intermediates that the reference's chain rule (fragment_backward) is written in; 0 if rejected. */
+static inline int reeval_fragment(const oracle_cam *c, const blend_in *in, size_t g, int x, int y, int mode, fragment *f)
 {
-    return eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
-                         fx, fy, mode_cutoff_sq(mode), mode_min_alpha(mode), 0, NULL, f);
+    const float cx = (float)((x / c->tile_w) * c->tile_w) + 0.5f * (float)(c->tile_w - 1);
+    const float cy = (float)((y / c->tile_h) * c->tile_h) + 0.5f * (float)(c->tile_h - 1);
+    tile_poly q;
+    tile_poly_setup(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, cx, cy, mode_cutoff_rcp(mode), 0, &q);
+    const pixel_terms p = pixel_terms_of(x % c->tile_w, y % c->tile_h, c->tile_w, c->tile_h);
+    fragment t;
+    if (!eval_fragment_tile(&q, 0.0f, in->rgba[4 * g + 3], &p, mode_exp2_scale(mode), 1, mode_min_alpha(mode), 0, NULL, &t)) return 0;
+    eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
+                  (float)x, (float)y, INFINITY, -1.0f, 0, NULL, f);
+    f->G = t.G;
+    f->alpha = t.alpha;
+    return 1;
 }
 
 /* position gradient of one fragment from the fourth column of dL/dVPMT, backward.cuh:292-305 */
@@ -1190,7 +1201,7 @@ O_EXPORT void oracle_blend_backward(
                 for (uint32_t j = first; j < last; ++j) {
                     const size_t g = inst[j];
                     fragment f;
-                    if (!reeval_fragment(&in, g, fx, fy, mode, &f)) continue;
+                    if (!reeval_fragment(c, &in, g, x, y, mode, &f)) continue;
                     const float bw = T * f.alpha;
                     const float *col = rgba + 4 * g;
                     for (int k = 0; k < 3; ++k) grad_rgb[3 * g + k] += bw * gp[k];
@@ -1231,7 +1242,7 @@ O_EXPORT void oracle_blend_backward(
                 const size_t pix = (size_t)c->width * y + x;
                 const float fx = (float)x, fy = (float)y;
                 fragment f;
-                if (!reeval_fragment(&in, g, fx, fy, mode, &f)) continue;
+                if (!reeval_fragment(c, &in, g, x, y, mode, &f)) continue;
                 const float gp[3] = { grad_image[pix], grad_image[np + pix], grad_image[2 * np + pix] };
                 int slot = -1;
                 if (mode == MODE_HYBRID)
