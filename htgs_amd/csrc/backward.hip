@@ -405,17 +405,13 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ Stage<256> st;
-    __shared__ float4 st_q[3][256];          // the forward pass's quadratics of the staged instances (accept / reject, alpha)
     __shared__ uint32_t st_idx[256];
     const uint32_t tile = blockIdx.x;
     const uint32_t t = threadIdx.x;
     const uint32_t lane = t & (kWave - 1);
-    const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
-    const uint32_t x = x0 + (t & 15), y = y0 + (t >> 4);
+    const uint32_t x = (tile % grid_w) * 16 + (t & 15), y = (tile / grid_w) * 16 + (t >> 4);
     const bool inside = x < width && y < height;
     const float fx = (float)x, fy = (float)y;
-    const PixelTerms pt = pixel_terms(t & 15, t >> 4, 16);
-    const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
     const size_t np = (size_t)width * height, pix = inside ? (size_t)width * y + x : 0;
     float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, e0 = 0.0f, e1 = 0.0f, e2 = 0.0f;
     if (inside) {
@@ -429,15 +425,6 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
         stage_load(st, prim, inst, base + t, last, t, st_idx);
-        if (base + t < last) {
-            TileGeometry tg;
-            tile_geometry(st.v1[t], st.v2[t], st.v4[t], cx, cy, tg);
-            float qn[6], qd[6];
-            tile_quadratics<MODE>(tg, qn, qd);
-            st_q[0][t] = make_float4(qn[0], qn[1], qn[2], qn[3]);
-            st_q[1][t] = make_float4(qn[4], qn[5], qd[0], qd[1]);
-            st_q[2][t] = make_float4(qd[2], qd[3], qd[4], qd[5]);
-        }
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         for (int j = 0; j < nb; ++j) {
@@ -449,18 +436,9 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
             if (!done) {
                 Frag f;
                 const float4 col = st.col[j];
-                // decided as the forward pass decided it; the plane form supplies the chain rule's intermediates
-                const float4 q0 = st_q[0][j], q1 = st_q[1][j], q2 = st_q[2][j];
-                TileFrag tf;
-                tf.num = quad_eval(q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, pt);
-                tf.den = quad_eval(q1.z, q1.w, q2.x, q2.y, q2.z, q2.w, pt);
-                if (!(tf.num > tf.den)) {
-                    tf.den_rcp = rcp_exact(tf.den);
-                    if (tile_frag_alpha<MODE>(col.w, tf)) {
-                        frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f);
-                        f.den_rcp = 1.0f / f.den;
-                        f.G = d_exp2((tf.num * ModeCfg<MODE>::exp2_scale) * tf.den_rcp);
-                        f.alpha = tf.alpha;
+                if (frag_cutoff<MODE>(st.v1[j], st.v2[j], st.v4[j], fx, fy, f)) {
+                    f.den_rcp = 1.0f / f.den;
+                    if (frag_alpha<MODE>(col.w, f)) {
                         hit = true;
                         const float bw = T * f.alpha;
                         acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                    // :171-174
