@@ -391,11 +391,23 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_momen
 // colour of the pixel (backward.cuh:97-249); each Gaussian's contributions are summed over the wave before
 // one lane issues the atomics.
 // ---------------------------------------------------------------------------------------------
+// Sum over the 64 lanes with data-parallel-primitive moves (six v_add_f32 with a DPP operand): butterflies inside
+// each quad, half row and row, then the row totals are chained into the last row.  Returns the total as a
+// wave-uniform value.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_take(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
 __device__ __forceinline__ float wave_sum(float v)
 {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
-    return v;
+    v += dpp_take<0xB1, 0xf>(v);        // quad_perm [1,0,3,2]
+    v += dpp_take<0x4E, 0xf>(v);        // quad_perm [2,3,0,1]
+    v += dpp_take<0x141, 0xf>(v);       // row_half_mirror
+    v += dpp_take<0x140, 0xf>(v);       // row_mirror: every lane of a row holds the row's sum
+    v += dpp_take<0x142, 0xa>(v);       // row_bcast:15 into rows 1 and 3
+    v += dpp_take<0x143, 0xc>(v);       // row_bcast:31 into rows 2 and 3: lane 63 holds the total
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 __global__ void __launch_bounds__(256) blend_global_backward_kernel(
