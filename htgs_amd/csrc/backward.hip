@@ -68,6 +68,30 @@ __device__ __forceinline__ void atomic_add_nonzero(float *p, float v)
     if (v != 0.0f) unsafeAtomicAdd(p, v);
 }
 
+// Core membership.  A pixel's stored core holds up to K Gaussians; the tile-walking kernels below ask, for every
+// fragment with alpha >= 1/20, whether its Gaussian is one of them and in which slot (backward.cuh:231-235).  The
+// pixel's indices are kept packed as (Gaussian << 5 | slot); xor with (g << 5) leaves the bare slot number for the
+// entry that holds g and something >= 32 for every other entry, so the minimum over the K entries answers both
+// questions with one xor per entry and one three-way minimum per two entries, no compare / select pairs.
+constexpr int kSlotBits = 5;                 // K <= 32; Gaussian indices stay below 2^27
+template <int KS>
+__device__ __forceinline__ int find_core_slot(const uint32_t *__restrict__ keys, uint32_t g)
+{
+    const uint32_t probe = g << kSlotBits;
+    uint32_t r = 0xffffffffu;
+    if (KS == 1) {
+        r = keys[0] ^ probe;
+    } else {
+#pragma unroll
+        for (int i = 0; i < KS; i += 2) {
+            const uint32_t a = keys[i] ^ probe, b = keys[i + 1] ^ probe;
+            const uint32_t m = a < b ? a : b;
+            r = r < m ? r : m;
+        }
+    }
+    return (r >> kSlotBits) == 0 ? (int)r : -1;
+}
+
 // ---------------------------------------------------------------------------------------------
 // HYBRID_BLEND (K >= 1), OIT_BLEND (K == 0) and ALPHA_BLEND_FIRST_K (core only, no tail): one lane per Gaussian
 // of the staged batch, all lanes walk the 64 pixels of the tile together (per-pixel terms are LDS broadcasts),
@@ -89,7 +113,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_kerne
 {
     constexpr bool kHasTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = K > 0 ? K : 1;
-    __shared__ uint32_t s_idx[64 * KS];      // [pixel][slot]
+    __shared__ uint32_t s_idx[64 * KS];      // [pixel][slot]: Gaussian << 5 | slot
     __shared__ float4 s_core[64 * KS];       // (weight * g, dC/dalpha . g)
     __shared__ float4 s_tail[64];            // (full weight * g, common)
     __shared__ float s_tail_a[64];
@@ -126,7 +150,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_kerne
                     const float4 info = core_info[(size_t)i * np + pix];
                     c = make_float4(info.w * g0, info.w * g1, info.w * g2, info.x * g0 + info.y * g1 + info.z * g2);   // :154-155
                 }
-                s_idx[lane * KS + i] = idx;
+                s_idx[lane * KS + i] = idx == 0xffffffffu ? idx : (idx << kSlotBits) | (uint32_t)i;
                 s_core[lane * KS + i] = c;
             }
         }
@@ -175,9 +199,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_kerne
             // only fragments with alpha >= 1/20 can sit in the core; the margin covers the forward pass having
             // evaluated alpha in tile-relative form (the stored index decides)
             if (K > 0 && f.alpha >= 0.98f * kMinAlphaCore) {
-#pragma unroll
-                for (int i = 0; i < KS; ++i)
-                    if (s_idx[p * KS + i] == g) slot = i;                        // :231-235
+                slot = find_core_slot<KS>(s_idx + p * KS, g);                   // :231-235
             }
             if (!kHasTail && slot < 0) continue;                                   // FIRST_K: only stored fragments carry gradient
             float dL_dalpha;
@@ -225,7 +247,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_kerne
 // (cut-off, alpha thresholds) are bit for bit those of the forward pass.
 // ---------------------------------------------------------------------------------------------
 template <int K, int MODE>
-__global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_moments_kernel(
+__global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_waves_per_eu(5))) blend_tail_backward_moments_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
     const float *__restrict__ grad_image, const uint32_t *__restrict__ offsets,
@@ -234,7 +256,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_momen
 {
     constexpr bool kHasTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = K > 0 ? K : 1;
-    __shared__ uint32_t s_idx[64 * KS];      // [pixel][slot]
+    __shared__ uint32_t s_idx[64 * KS];      // [pixel][slot]: Gaussian << 5 | slot
     __shared__ float4 s_core[64 * KS];       // (weight * g, dC/dalpha . g)
     __shared__ float4 s_tail[64];            // (full weight * g, common)
     __shared__ float s_tail_a[64];
@@ -271,7 +293,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_momen
                     const float4 info = core_info[(size_t)i * np + pix];
                     c = make_float4(info.w * g0, info.w * g1, info.w * g2, info.x * g0 + info.y * g1 + info.z * g2);   // :154-155
                 }
-                s_idx[lane * KS + i] = idx;
+                s_idx[lane * KS + i] = idx == 0xffffffffu ? idx : (idx << kSlotBits) | (uint32_t)i;
                 s_core[lane * KS + i] = c;
             }
         }
@@ -314,9 +336,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_momen
             if (alpha < ModeCfg<MODE>::min_alpha) continue;
             int slot = -1;
             if (K > 0 && alpha >= kMinAlphaCore) {
-#pragma unroll
-                for (int i = 0; i < KS; ++i)
-                    if (s_idx[p * KS + i] == g) slot = i;                        // :231-235
+                slot = find_core_slot<KS>(s_idx + p * KS, g);                   // :231-235
             }
             if (!kHasTail && slot < 0) continue;                                   // FIRST_K: only stored fragments carry gradient
             float dL_dalpha;
@@ -734,6 +754,7 @@ extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0 || f->n_primitives < 0)
         return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: bad argument");
     if (f->n_primitives == 0 || f->n_instances == 0) return HTGS_OK;
+    if (f->n_primitives > (1 << 27)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: more than 2^27 Gaussians");
     const bool needs_core = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K;
     const bool needs_tail = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_OIT_BLEND;
     const bool rows = f->mode != HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
