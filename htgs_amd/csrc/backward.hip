@@ -212,7 +212,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_kerne
                 acc[0] += t.x * f.alpha; acc[1] += t.y * f.alpha; acc[2] += t.z * f.alpha;   // :244
                 const float oma = 1.0f - f.alpha;
                 dL_dalpha = t.w + (col.x * t.x + col.y * t.y + col.z * t.z)
-                          + s_tail_a[p] / (oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255
+                          + s_tail_a[p] * rcp_exact(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255
             }
             if (dL_dalpha == 0.0f) continue;                                     // :258
             FragGrads fg;
@@ -349,7 +349,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
                 a0 += t.x * alpha; a1 += t.y * alpha; a2 += t.z * alpha;         // :244
                 const float oma = 1.0f - alpha;
                 dL_dalpha = t.w + (col.x * t.x + col.y * t.y + col.z * t.z)
-                          + s_tail_a[p] / (oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255
+                          + s_tail_a[p] * rcp_exact(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255
             }
             if (dL_dalpha == 0.0f) continue;                                     // :258
             a_op += dL_dalpha * G;                                               // :262

@@ -1267,7 +1267,7 @@ O_EXPORT void oracle_blend_backward(
                     const float cg[3] = { full * gp[0], full * gp[1], full * gp[2] };              /* :172 */
                     const float a_term = w_tail * T_tail * rdg;                                    /* :173 */
                     const float oma = 1.0f - f.alpha;
-                    dL_dalpha = common + dot3(col, cg) + a_term / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS);   /* :253-255 */
+                    dL_dalpha = common + dot3(col, cg) + a_term * (1.0f / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS));   /* :253-255, as a product with the reciprocal */
                 }
                 if (dL_dalpha == 0.0f) continue;                                                   /* :258 */
                 frag_grads fg;
