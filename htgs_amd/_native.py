@@ -58,7 +58,6 @@ class Frame(ctypes.Structure):
         ("tail_info", ctypes.c_void_p),
         ("grad_image", ctypes.c_void_p),
         ("grad_rows", ctypes.c_void_p),
-        ("grad_acc", ctypes.c_void_p),
         ("dens_helper", ctypes.c_void_p),
         ("grad_positions", ctypes.c_void_p),
         ("grad_scales", ctypes.c_void_p),

@@ -281,15 +281,13 @@ class FrameBuffers:
             raise RuntimeError("grad_image must be [3,H,W]")
         total_sh = int(self.sh_rest.shape[1])
         f32 = dict(dtype=torch.float32, device=dev)
-        # per-instance rows (no initialisation needed) for the tile-walking modes, per-Gaussian atomics for mode 2
-        rows_mode = self.mode != 2
-        self.grad_rows = torch.empty((max(self.n_instances, 1), 16), **f32) if rows_mode else None
-        self.grad_acc = None if rows_mode else torch.zeros((16, n), **f32)
+        # one row per instance, every one written by the blend kernels: no initialisation needed
+        self.grad_rows = torch.empty((max(self.n_instances, 1), 16), **f32)
         grads = [torch.empty((n, 3), **f32), torch.empty((n, 3), **f32), torch.empty((n, 4), **f32), torch.empty((n, 1), **f32),
                  torch.empty((n, 1, 3), **f32), torch.empty((n, total_sh, 3), **f32)]
         f = self.frame
         f.stream = torch.cuda.current_stream(dev).cuda_stream
-        f.grad_image, f.grad_acc, f.grad_rows = _ptr(grad_image), _ptr(self.grad_acc), _ptr(self.grad_rows)
+        f.grad_image, f.grad_rows = _ptr(grad_image), _ptr(self.grad_rows)
         (f.grad_positions, f.grad_scales, f.grad_rotations, f.grad_opacities, f.grad_sh_0, f.grad_sh_rest) = [_ptr(g) for g in grads]
         rows = 0
         helper = None
@@ -300,7 +298,7 @@ class FrameBuffers:
                 raise RuntimeError("densification_info must be a contiguous float32 [2,N] or [3,N] tensor on the GPU")
             f.densification_info = densification_info.data_ptr()
             if rows == 3:
-                helper = torch.empty(max(self.n_instances, 1), **f32) if rows_mode else torch.zeros(n, **f32)
+                helper = torch.empty(max(self.n_instances, 1), **f32)
         else:
             f.densification_info = 0
         f.densification_rows = rows

@@ -86,11 +86,10 @@ typedef struct htgs_frame {
     float *tail_info;          /* [6,P] sum alpha*rgb (3), 1/sum alpha, T_tail, T_core       (modes 0, 3) */
     /* ---- training: backward (backward_wrapper, rasterization_api.cu:178-363) ---- */
     const float *grad_image;   /* [3,H,W] upstream gradient */
-    float *grad_rows;          /* modes 0, 1, 3: [I,16] one row per instance, in creation order: dL/drgb (3), dL/dopacity,
+    float *grad_rows;          /* [I,16] one row per instance, in creation order: dL/drgb (3), dL/dopacity,
                                   dL/dVPMT1, 2, 4 (4 each); every row is written, no initialisation needed */
-    float *grad_acc;           /* mode 2: [16,N] the same 16 sums per Gaussian, zero-filled by the caller (atomics) */
-    float *dens_helper;        /* sum over fragments of |dL/dposition|_1: [I] per instance (modes 0, 1, 3) or [N] zero-filled
-                                  (mode 2); NULL unless densification_rows == 3 */
+    float *dens_helper;        /* [I] per instance: sum over fragments of |dL/dposition|_1; NULL unless
+                                  densification_rows == 3 */
     float *grad_positions;     /* [N,3] outputs; every element is written */
     float *grad_scales;        /* [N,3] */
     float *grad_rotations;     /* [N,4] */
@@ -150,10 +149,9 @@ int htgs_forward_front(const htgs_frame *f);
 int htgs_forward_back(const htgs_frame *f, int *selector);
 /* blend_cu (forward) of the frame's mode, R/include/<mode>/kernels/forward.cuh */
 int htgs_blend_forward(const htgs_frame *f, int selector);
-/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: writes grad_rows (modes 0, 1, 3) or accumulates into
- * grad_acc (mode 2), and dens_helper */
+/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: writes grad_rows and dens_helper */
 int htgs_blend_backward(const htgs_frame *f, int selector);
-/* preprocess_cu (backward), R/include/hybrid_blend/kernels/backward.cuh:10-102: grad_rows / grad_acc -> the six gradients */
+/* preprocess_cu (backward), R/include/hybrid_blend/kernels/backward.cuh:10-102: grad_rows -> the six gradients */
 int htgs_preprocess_backward(const htgs_frame *f);
 /* <mode>::backward (R/src/hybrid_blend/backward.cu:26-128): blend backward, then preprocess backward */
 int htgs_backward(const htgs_frame *f, int selector);

@@ -62,9 +62,9 @@ def test_ragged_image_and_full_grid_gaussian(cuda, mode):
         assert_grad_close(name, got.cpu().numpy(), want[name])
 
 
-@pytest.mark.parametrize("mode", [0, 1, 3])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_gradients_are_deterministic(cuda, mode):
-    """Modes 0, 1, 3 write one gradient row per (Gaussian, tile) instance and sum a Gaussian's rows in a fixed order:
+    """Every mode writes one gradient row per (Gaussian, tile) instance and sums a Gaussian's rows in a fixed order:
     two runs give the same bits."""
     scene = make_scene(1, 40_000)
     print(f"case mode={mode}", flush=True)
