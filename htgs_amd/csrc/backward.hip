@@ -414,11 +414,11 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
 
 // ---------------------------------------------------------------------------------------------
 // ALPHA_BLEND_GLOBAL_ORDERING: one lane per pixel walks the depth-sorted list front to back with the final
-// colour of the pixel (backward.cuh:97-249).  Per fragment a lane produces dL/drgb, dL/dopacity and the twelve
-// moments of dL/d|m|^2 and dL/d|d|^2 about the tile centre (see the moments kernel above; the evaluation itself
-// stays in the plane form); the sixteen numbers are summed over the wave and parked in LDS, and after a batch of
-// 64 Gaussians one thread per Gaussian adds the four waves' sums, applies the chain to the VPMT rows once and
-// writes the instance's row.
+// colour of the pixel (backward.cuh:97-249), evaluating every fragment with the forward pass's arithmetic.  Per
+// fragment a lane produces dL/drgb, dL/dopacity and the twelve moments of dL/dnum and dL/dden about the tile
+// centre (see the moments kernel above); the sixteen numbers are summed over the wave and parked in LDS, and
+// after a batch of 64 Gaussians one thread per Gaussian adds the four waves' sums, applies the chain to the VPMT
+// rows once and writes the instance's row.
 // ---------------------------------------------------------------------------------------------
 // Sum over the 64 lanes with data-parallel-primitive moves (six v_add_f32 with a DPP operand): butterflies inside
 // each quad, half row and row, then the row totals are chained into the last row.  Returns the total as a
@@ -473,6 +473,7 @@ __device__ __forceinline__ void wave_sum_16(float (&v)[16])
 
 constexpr int kGlobalBatch = 64;              // Gaussians per staged batch: one bit each in a wave's 64-bit hit mask
 
+template <bool HELPER>
 __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const float *__restrict__ image, const float *__restrict__ grad_image, const float *__restrict__ VPM,
@@ -480,10 +481,10 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     float *__restrict__ helper_rows, uint32_t width, uint32_t height, uint32_t grid_w)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
-    __shared__ float4 s_rec[4][kGlobalBatch];                 // VPMT1, VPMT2, VPMT4, (rgb, opacity)
-    __shared__ uint32_t s_g[kGlobalBatch];
+    __shared__ TileStage<kGlobalBatch> st;
+    __shared__ float4 s_rows[HELPER ? 3 : 1][kGlobalBatch];   // VPMT1, VPMT2, VPMT4 (third densification row only)
     __shared__ float s_part[4][kGlobalBatch][17];             // per wave: the 16 sums of one Gaussian (padded row)
-    __shared__ float s_help[4][kGlobalBatch];
+    __shared__ float s_help[HELPER ? 4 : 1][kGlobalBatch];
     __shared__ uint32_t s_hit[4][2];
     const uint32_t tile = blockIdx.x;
     const uint32_t t = threadIdx.x;
@@ -508,59 +509,66 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     for (; base < last; base += kGlobalBatch) {
         // (the barrier also separates the previous batch's reads of the staged records and sums from the writes below)
         if (__syncthreads_count(done) == 256) break;
-        {
-            const uint32_t j = t & (kGlobalBatch - 1), part = t >> 6;             // one 16-byte row per thread
-            if (base + j < last) {
-                const uint32_t g = inst[base + j];
-                s_rec[part][j] = prim[(size_t)g * (HTGS_PRIM_FLOATS / 4) + (part == 3 ? 4 : part)];
-                if (part == 0) s_g[j] = g;
-            }
-        }
+        if (wave == 0) tile_stage_load<MODE, kGlobalBatch, false>(st, prim, inst, base + lane, last, lane, cx, cy);
+        if (HELPER && wave >= 1 && base + lane < last)
+            s_rows[wave - 1][lane] = prim[(size_t)inst[base + lane] * (HTGS_PRIM_FLOATS / 4) + (wave - 1)];
         __syncthreads();
         const int nb = last - base < (uint32_t)kGlobalBatch ? (int)(last - base) : kGlobalBatch;
         uint32_t hit_lo = 0u, hit_hi = 0u;                                       // wave-uniform
-        for (int j = 0; j < nb; ++j) {
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
             float acc[16];
 #pragma unroll
             for (int k = 0; k < 16; ++k) acc[k] = 0.0f;
             float help = 0.0f;
             bool hit = false;
-            if (!done) {
-                Frag f;
-                const float4 col = s_rec[3][j];
-                if (frag_cutoff<MODE>(s_rec[0][j], s_rec[1][j], s_rec[2][j], fx, fy, f)) {
-                    f.den_rcp = 1.0f / f.den;
-                    if (frag_alpha<MODE>(col.w, f)) {
-                        hit = true;
-                        const float bw = T * f.alpha;
-                        acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                    // :171-174
-                        n0 += bw * col.x; n1 += bw * col.y; n2 += bw * col.z;                    // :178
-                        const float oma = 1.0f - f.alpha;
-                        const float omar = 1.0f / (oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);
-                        const float dL_dalpha = (T * col.x - (e0 - n0) * omar) * g0 + (T * col.y - (e1 - n1) * omar) * g1
-                                              + (T * col.z - (e2 - n2) * omar) * g2;            // :181
-                        if (dL_dalpha != 0.0f) {
-                            acc[3] = dL_dalpha * f.G;                                            // :262
-                            const float dL_drho2 = dL_dalpha * col.w * -0.5f * f.G;
-                            const float wn = dL_drho2 * f.den_rcp;                               // dL/d|m|^2
-                            const float wd = -(wn * f.num) * f.den_rcp;                          // dL/d|d|^2
-                            const float wnx = wn * pt.X, wny = wn * pt.Y, wdx = wd * pt.X, wdy = wd * pt.Y;
-                            acc[4] = wn; acc[5] = wnx; acc[6] = wny; acc[7] = wnx * pt.X; acc[8] = wnx * pt.Y; acc[9] = wny * pt.Y;
-                            acc[10] = wd; acc[11] = wdx; acc[12] = wdy; acc[13] = wdx * pt.X; acc[14] = wdx * pt.Y; acc[15] = wdy * pt.Y;
-                            if (helper_rows) {
-                                // fourth components of the fragment's dL/dVPMT rows (:260-289) -> |dL/dposition|_1 (:292-306)
-                                const float w2 = 2.0f * wn;
-                                const float dm0 = w2 * f.m[0], dm1 = w2 * f.m[1], dm2 = w2 * f.m[2];
-                                const float dpx3 = f.py[0] * dm0 + f.py[1] * dm1 + f.py[2] * dm2;
-                                const float dpy3 = -(f.px[0] * dm0 + f.px[1] * dm1 + f.px[2] * dm2);
-                                const float dv3 = -fx * dpx3 - fy * dpy3;
+            TileFrag f;
+            // the forward pass's own arithmetic (blend_global_forward_kernel): same accept / reject decisions, same alpha
+            if (!done && tile_frag_cutoff<kGlobalBatch>(addr, pt, f)) {
+                f.den_rcp = rcp_exact(f.den);
+                const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * f.den_rcp);
+                const float4 col = stage_row<kGlobalBatch, 5>(addr);
+                const float opacity = stage_opacity<kGlobalBatch>(addr);
+                const float ag = opacity * G;
+                const float alpha = ag < kMaxFragmentAlpha ? ag : kMaxFragmentAlpha;
+                if (!(alpha < ModeCfg<MODE>::min_alpha)) {
+                    hit = true;
+                    const float bw = T * alpha;
+                    acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                        // :171-174
+                    n0 = __builtin_fmaf(bw, col.x, n0); n1 = __builtin_fmaf(bw, col.y, n1); n2 = __builtin_fmaf(bw, col.z, n2);   // :178
+                    const float oma = 1.0f - alpha;
+                    const float omar = rcp_exact(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);
+                    const float dL_dalpha = (T * col.x - (e0 - n0) * omar) * g0 + (T * col.y - (e1 - n1) * omar) * g1
+                                          + (T * col.z - (e2 - n2) * omar) * g2;                // :181
+                    if (dL_dalpha != 0.0f) {
+                        acc[3] = dL_dalpha * G;                                                  // :262
+                        // rho^2 = num / (kc den) with num = kc |m|^2:  dL/dnum and dL/dden  (:263-266)
+                        const float dL_drho2 = dL_dalpha * opacity * -0.5f * G;
+                        const float wn = (dL_drho2 * ModeCfg<MODE>::cutoff_sq) * f.den_rcp;
+                        const float wd = -(wn * f.num) * f.den_rcp;
+                        const float wnx = wn * pt.X, wny = wn * pt.Y, wdx = wd * pt.X, wdy = wd * pt.Y;
+                        acc[4] = wn; acc[5] = wnx; acc[6] = wny; acc[7] = wnx * pt.X; acc[8] = wnx * pt.Y; acc[9] = wny * pt.Y;
+                        acc[10] = wd; acc[11] = wdx; acc[12] = wdy; acc[13] = wdx * pt.X; acc[14] = wdx * pt.Y; acc[15] = wdy * pt.Y;
+                        if (HELPER) {
+                            // fourth components of the fragment's dL/dVPMT rows (:260-289) -> |dL/dposition|_1 (:292-306)
+                            const float4 V1 = s_rows[0][j], V2 = s_rows[1][j], V4 = s_rows[2][j];
+                            const float px0 = __builtin_fmaf(-V4.x, fx, V1.x), px1 = __builtin_fmaf(-V4.y, fx, V1.y);
+                            const float px2 = __builtin_fmaf(-V4.z, fx, V1.z), px3 = __builtin_fmaf(-V4.w, fx, V1.w);
+                            const float py0 = __builtin_fmaf(-V4.x, fy, V2.x), py1 = __builtin_fmaf(-V4.y, fy, V2.y);
+                            const float py2 = __builtin_fmaf(-V4.z, fy, V2.z), py3 = __builtin_fmaf(-V4.w, fy, V2.w);
+                            const float w2 = 2.0f * (dL_drho2 * f.den_rcp);                       // 2 dL/d|m|^2
+                            const float dm0 = w2 * __builtin_fmaf(px3, py0, -(px0 * py3));
+                            const float dm1 = w2 * __builtin_fmaf(px3, py1, -(px1 * py3));
+                            const float dm2 = w2 * __builtin_fmaf(px3, py2, -(px2 * py3));
+                            const float dpx3 = py0 * dm0 + py1 * dm1 + py2 * dm2;
+                            const float dpy3 = -(px0 * dm0 + px1 * dm1 + px2 * dm2);
+                            const float dv3 = -fx * dpx3 - fy * dpy3;
 #pragma unroll
-                                for (int k = 0; k < 3; ++k) help += fabsf(VPM[k] * dpx3 + VPM[4 + k] * dpy3 + VPM[12 + k] * dv3);
-                            }
+                            for (int k = 0; k < 3; ++k) help += fabsf(VPM[k] * dpx3 + VPM[4 + k] * dpy3 + VPM[12 + k] * dv3);
                         }
-                        T *= oma;                                                                // :245
-                        if (T < kTransmittanceThreshold) done = true;
                     }
+                    T *= oma;                                                                    // :245
+                    if (T < kTransmittanceThreshold) done = true;
                 }
             }
             if (__any(hit)) {                                                                    // wave-uniform
@@ -569,7 +577,7 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
                     float *dst = &s_part[wave][j][4 * (lane >> 4)];
                     dst[0] = acc[0]; dst[1] = acc[1]; dst[2] = acc[2]; dst[3] = acc[3];
                 }
-                if (helper_rows) {
+                if (HELPER) {
                     const float s = wave_sum(help);
                     if (lane == 0) s_help[wave][j] = s;
                 }
@@ -591,9 +599,10 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
                     any = true;
 #pragma unroll
                     for (int k = 0; k < 16; ++k) m[k] += s_part[w][t][k];
-                    if (helper_rows) help += s_help[w][t];
+                    if (HELPER) help += s_help[w][t];
                 }
             }
+            const uint32_t g = inst[base + t];
             RowGrads rg;
 #pragma unroll
             for (int k = 0; k < 3; ++k) rg.da[k] = rg.db[k] = 0.0f;
@@ -601,10 +610,10 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
 #pragma unroll
             for (int k = 0; k < 4; ++k) rg.e4[k] = 0.0f;
             if (any) {
+                const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
                 const float S[6] = { m[4], m[5], m[6], m[7], m[8], m[9] }, Tm[6] = { m[10], m[11], m[12], m[13], m[14], m[15] };
-                moments_to_rows(s_rec[0][t], s_rec[1][t], s_rec[2][t], cx, cy, 2.0f, S, Tm, rg);
+                moments_to_rows(rec[0], rec[1], rec[2], cx, cy, 2.0f * ModeCfg<MODE>::cutoff_rcp, S, Tm, rg);
             }
-            const uint32_t g = s_g[t];
             const ushort4 bnd = *reinterpret_cast<const ushort4 *>(bounds + 4 * (size_t)g);
             const uint32_t slot = (g == 0 ? 0u : offsets[g - 1]) + (tile / grid_w - bnd.z) * ((uint32_t)bnd.y - bnd.x) + (tile % grid_w - bnd.x);
             float4 *row = grad_rows + 4 * (size_t)slot;
@@ -612,7 +621,7 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
             row[1] = make_float4(rg.da[0], rg.da[1], rg.da[2], rg.daw);
             row[2] = make_float4(rg.db[0], rg.db[1], rg.db[2], rg.dbw);
             row[3] = make_float4(rg.e4[0], rg.e4[1], rg.e4[2], rg.e4[3]);
-            if (helper_rows) helper_rows[slot] = help;
+            if (HELPER) helper_rows[slot] = help;
         }
     }
     // instances behind the point where every pixel of the tile is saturated: rows of zeros
@@ -623,7 +632,7 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
         float4 *row = grad_rows + 4 * (size_t)slot;
         const float4 z = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         row[0] = z; row[1] = z; row[2] = z; row[3] = z;
-        if (helper_rows) helper_rows[slot] = 0.0f;
+        if (HELPER) helper_rows[slot] = 0.0f;
     }
 }
 
@@ -906,9 +915,14 @@ extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
             }
             break;
         default:
-            hipLaunchKernelGGL(blend_global_backward_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
-                               (const float4 *)f->prim, f->image, f->grad_image, f->VPM, f->offsets, f->bounds, (float4 *)f->grad_rows,
-                               f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+            if (f->dens_helper)
+                hipLaunchKernelGGL(blend_global_backward_kernel<true>, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
+                                   (const float4 *)f->prim, f->image, f->grad_image, f->VPM, f->offsets, f->bounds, (float4 *)f->grad_rows,
+                                   f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+            else
+                hipLaunchKernelGGL(blend_global_backward_kernel<false>, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
+                                   (const float4 *)f->prim, f->image, f->grad_image, f->VPM, f->offsets, f->bounds, (float4 *)f->grad_rows,
+                                   f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
             break;
     }
     return check_launch("blend_backward");

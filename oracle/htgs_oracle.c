@@ -1061,9 +1061,6 @@ static void fragment_backward(const fragment *f, float opacity, float dL_dalpha,
  * plane-form intermediates that the reference's chain rule (fragment_backward) is written in; 0 if rejected. */
 static inline int reeval_fragment(const oracle_cam *c, const blend_in *in, size_t g, int x, int y, int mode, fragment *f)
 {
-    if (mode == MODE_GLOBAL)     /* the global-ordering backward stays in the plane form altogether */
-        return eval_fragment(in->VPMT1 + 4 * g, in->VPMT2 + 4 * g, in->VPMT4 + 4 * g, in->MT3 + 4 * g, in->rgba[4 * g + 3],
-                             (float)x, (float)y, mode_cutoff_sq(mode), mode_min_alpha(mode), 0, NULL, f);
     const float cx = (float)((x / c->tile_w) * c->tile_w) + 0.5f * (float)(c->tile_w - 1);
     const float cy = (float)((y / c->tile_h) * c->tile_h) + 0.5f * (float)(c->tile_h - 1);
     tile_poly q;
