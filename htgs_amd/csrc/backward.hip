@@ -692,28 +692,72 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
         for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) lds[q] = sh_rest[base_word + q];
     }
     __syncthreads();
+    // Row sums.  The Gaussian's instances are the rows [offsets[i-1], offsets[i]).  A Gaussian with few rows adds them
+    // up in its own lane, front to back; one with many would keep the other 63 lanes of its wave waiting, so the wave
+    // takes those one at a time: 16 rows x 4 quarters per step (1 KB of consecutive memory), a butterfly over the 16
+    // row groups, and the owner lane picks up the four quarters.  Either order is fixed by the offsets alone, so the
+    // sums are reproducible.
+    constexpr uint32_t kShortRows = 16;
+    float4 s0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), s1 = s0, s2 = s0, s3 = s0;
+    float helper_sum = 0.0f;
+    {
+        const uint32_t lane = threadIdx.x & (kWave - 1);
+        uint32_t r0 = 0u, r1 = 0u;
+        if (live) { r0 = i == 0 ? 0u : offsets[i - 1]; r1 = offsets[i]; }
+        const uint32_t count = r1 - r0;
+        if (count <= kShortRows) {
+            for (uint32_t r = r0; r < r1; ++r) {
+                const float4 *row = grad_rows + 4 * (size_t)r;
+                const float4 v0 = row[0], v1 = row[1], v2 = row[2], v3 = row[3];
+                s0.x += v0.x; s0.y += v0.y; s0.z += v0.z; s0.w += v0.w;
+                s1.x += v1.x; s1.y += v1.y; s1.z += v1.z; s1.w += v1.w;
+                s2.x += v2.x; s2.y += v2.y; s2.z += v2.z; s2.w += v2.w;
+                s3.x += v3.x; s3.y += v3.y; s3.z += v3.z; s3.w += v3.w;
+                if (helper_rows) helper_sum += helper_rows[r];
+            }
+        }
+        unsigned long long pending = __ballot(count > kShortRows);
+        while (pending) {                                                        // wave-uniform
+            const int owner = __ffsll(pending) - 1;
+            pending &= pending - 1;
+            const uint32_t R0 = __builtin_amdgcn_readlane(r0, owner), R1 = __builtin_amdgcn_readlane(r1, owner);
+            float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            for (uint32_t r = R0 + (lane >> 2); r < R1; r += 16) {
+                const float4 v = grad_rows[4 * (size_t)r + (lane & 3)];
+                acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+            }
+#pragma unroll
+            for (int m = 4; m < kWave; m <<= 1) {
+                acc.x += __shfl_xor(acc.x, m); acc.y += __shfl_xor(acc.y, m);
+                acc.z += __shfl_xor(acc.z, m); acc.w += __shfl_xor(acc.w, m);
+            }
+            float hs = 0.0f;
+            if (helper_rows) {
+                for (uint32_t r = R0 + lane; r < R1; r += kWave) hs += helper_rows[r];
+                hs = wave_sum(hs);
+            }
+            float q[4][4];                                                       // lane k holds quarter k of the total
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                q[k][0] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc.x), k));
+                q[k][1] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc.y), k));
+                q[k][2] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc.z), k));
+                q[k][3] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(acc.w), k));
+            }
+            if ((int)lane == owner) {
+                s0 = make_float4(q[0][0], q[0][1], q[0][2], q[0][3]); s1 = make_float4(q[1][0], q[1][1], q[1][2], q[1][3]);
+                s2 = make_float4(q[2][0], q[2][1], q[2][2], q[2][3]); s3 = make_float4(q[3][0], q[3][1], q[3][2], q[3][3]);
+                helper_sum = hs;
+            }
+        }
+    }
     float sh_b[15];                                                // basis values of the active bands
     float g[3] = { 0.0f, 0.0f, 0.0f };
     int nb = 0;
     if (live) {
     float a[16];
-    float helper_sum = 0.0f;
-    {
-        // the Gaussian's instances are the rows [offsets[i-1], offsets[i]); summed front to back
-        float4 s0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), s1 = s0, s2 = s0, s3 = s0;
-        const uint32_t r0 = i == 0 ? 0u : offsets[i - 1], r1 = offsets[i];
-        for (uint32_t r = r0; r < r1; ++r) {
-            const float4 *row = grad_rows + 4 * (size_t)r;
-            const float4 v0 = row[0], v1 = row[1], v2 = row[2], v3 = row[3];
-            s0.x += v0.x; s0.y += v0.y; s0.z += v0.z; s0.w += v0.w;
-            s1.x += v1.x; s1.y += v1.y; s1.z += v1.z; s1.w += v1.w;
-            s2.x += v2.x; s2.y += v2.y; s2.z += v2.z; s2.w += v2.w;
-            s3.x += v3.x; s3.y += v3.y; s3.z += v3.z; s3.w += v3.w;
-            if (helper_rows) helper_sum += helper_rows[r];
-        }
-        a[0] = s0.x; a[1] = s0.y; a[2] = s0.z; a[3] = s0.w; a[4] = s1.x; a[5] = s1.y; a[6] = s1.z; a[7] = s1.w;
-        a[8] = s2.x; a[9] = s2.y; a[10] = s2.z; a[11] = s2.w; a[12] = s3.x; a[13] = s3.y; a[14] = s3.z; a[15] = s3.w;
-    }
+    a[0] = s0.x; a[1] = s0.y; a[2] = s0.z; a[3] = s0.w; a[4] = s1.x; a[5] = s1.y; a[6] = s1.z; a[7] = s1.w;
+    a[8] = s2.x; a[9] = s2.y; a[10] = s2.z; a[11] = s2.w; a[12] = s3.x; a[13] = s3.y; a[14] = s3.z; a[15] = s3.w;
     float V1[4], V2[4], V4[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) { V1[k] = VPM_in[k]; V2[k] = VPM_in[4 + k]; V4[k] = VPM_in[12 + k]; }
