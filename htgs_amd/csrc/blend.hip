@@ -41,9 +41,13 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
 
     float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f, depth_tail = 0.0f;
-    float c0[K], c1[K], c2[K], c3[K], cd[K];
+    // A core slot holds depth, alpha and the Gaussian's index (an exchange moves three registers); the colours are
+    // fetched once, when the sorted core is blended.  Every fragment's alpha * colour goes into the tail sums when it
+    // is evaluated, and the share of the fragments that end up in the core is taken out again at the end, so an
+    // entry pushed out of the core needs no colour: its alpha and depth, which the tail also needs, are in the slot.
+    float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
 #pragma unroll
-    for (int i = 0; i < K; ++i) { c0[i] = c1[i] = c2[i] = c3[i] = 0.0f; cd[i] = __FLT_MAX__; }
+    for (int i = 0; i < K; ++i) { cd[i] = __FLT_MAX__; ca[i] = 0.0f; ci[i] = 0.0f; }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
@@ -61,8 +65,12 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 const float4 col = stage_row<64, 5>(addr);
                 if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
                 float depth = tile_frag_depth<64>(addr, pt, f);
-                float p0 = col.x, p1 = col.y, p2 = col.z, p3 = f.alpha;       // slots keep colour and alpha apart
+                float p3 = f.alpha;
+                tail0 = __builtin_fmaf(p3, col.x, tail0);
+                tail1 = __builtin_fmaf(p3, col.y, tail1);
+                tail2 = __builtin_fmaf(p3, col.z, tail2);
                 if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
+                    float pi = col.w;
 #pragma unroll
                     for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
                         if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
@@ -70,17 +78,13 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                         for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
                             if (depth < cd[i]) {
                                 vswap(depth, cd[i]);
-                                vswap(p0, c0[i]);
-                                vswap(p1, c1[i]);
-                                vswap(p2, c2[i]);
-                                vswap(p3, c3[i]);
+                                vswap(p3, ca[i]);
+                                vswap(pi, ci[i]);
                             }
                         }
                     }
                 }
-                tail0 = __builtin_fmaf(p3, p0, tail0);
-                tail1 = __builtin_fmaf(p3, p1, tail1);
-                tail2 = __builtin_fmaf(p3, p2, tail2);
+                // (depth, p3) is the fragment itself, the entry it pushed out of the core, or an empty slot (alpha 0)
                 tail3 += p3;
                 if (!median) depth_tail = __builtin_fmaf(depth, p3, depth_tail);
                 T_tail *= 1.0f - p3;
@@ -90,16 +94,26 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     if (!inside) return;
 
     float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T_core = 1.0f;
+    float4 cc[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+        cc[i] = ca[i] > 0.0f ? prim[(size_t)float_to_bits(ci[i]) * (HTGS_PRIM_FLOATS / 4) + 4] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+    for (int i = 0; i < K; ++i) {                      // the core's share of the colour sums
+        tail0 = __builtin_fmaf(-ca[i], cc[i].x, tail0);
+        tail1 = __builtin_fmaf(-ca[i], cc[i].y, tail1);
+        tail2 = __builtin_fmaf(-ca[i], cc[i].z, tail2);
+    }
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         if (T_core >= kTransmittanceThreshold) {
-            const float w = T_core * c3[i];
-            r = __builtin_fmaf(w, c0[i], r);
-            g = __builtin_fmaf(w, c1[i], g);
-            b = __builtin_fmaf(w, c2[i], b);
+            const float w = T_core * ca[i];
+            r = __builtin_fmaf(w, cc[i].x, r);
+            g = __builtin_fmaf(w, cc[i].y, g);
+            b = __builtin_fmaf(w, cc[i].z, b);
             if (median) depth_pixel = (T_core > 0.5f && cd[i] < __FLT_MAX__) ? cd[i] : depth_pixel;
             else depth_pixel = __builtin_fmaf(w, cd[i], depth_pixel);
-            T_core *= 1.0f - c3[i];
+            T_core *= 1.0f - ca[i];
         }
     }
     float total_alpha = 0.0f;

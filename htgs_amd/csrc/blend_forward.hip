@@ -33,10 +33,12 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
     const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
 
     float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f;
-    float c0[K], c1[K], c2[K], c3[K], cd[K];
+    // slots hold depth, alpha and index; colours are fetched at the end and the core's share of the colour sums is
+    // taken out there (see blend_hybrid_kernel)
+    float c3[K], cd[K];
     uint32_t ci[K];
 #pragma unroll
-    for (int i = 0; i < K; ++i) { c0[i] = c1[i] = c2[i] = c3[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+    for (int i = 0; i < K; ++i) { c3[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
@@ -52,7 +54,10 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
             const float4 col = stage_row<64, 5>(addr);
             if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
             float depth = tile_frag_depth<64>(addr, pt, f);
-            float p0 = col.x, p1 = col.y, p2 = col.z, p3 = f.alpha;
+            float p3 = f.alpha;
+            tail0 = __builtin_fmaf(p3, col.x, tail0);
+            tail1 = __builtin_fmaf(p3, col.y, tail1);
+            tail2 = __builtin_fmaf(p3, col.z, tail2);
             if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
                 uint32_t idx = stage_index<64>(addr);
 #pragma unroll
@@ -62,18 +67,12 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
                     for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
                         if (depth < cd[i]) {
                             vswap(depth, cd[i]);
-                            vswap(p0, c0[i]);
-                            vswap(p1, c1[i]);
-                            vswap(p2, c2[i]);
                             vswap(p3, c3[i]);
                             vswap(idx, ci[i]);
                         }
                     }
                 }
             }
-            tail0 = __builtin_fmaf(p3, p0, tail0);
-            tail1 = __builtin_fmaf(p3, p1, tail1);
-            tail2 = __builtin_fmaf(p3, p2, tail2);
             tail3 += p3;
             T_tail *= 1.0f - p3;
         }
@@ -81,6 +80,19 @@ __global__ void __launch_bounds__(64) blend_hybrid_forward_kernel(
     if (!inside) return;
 
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    float c0[K], c1[K], c2[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        float4 c = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (c3[i] > 0.0f) c = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS / 4) + 4];
+        c0[i] = c.x; c1[i] = c.y; c2[i] = c.z;
+    }
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        tail0 = __builtin_fmaf(-c3[i], c0[i], tail0);
+        tail1 = __builtin_fmaf(-c3[i], c1[i], tail1);
+        tail2 = __builtin_fmaf(-c3[i], c2[i], tail2);
+    }
     float r = 0.0f, g = 0.0f, b = 0.0f, T_core = 1.0f;
 #pragma unroll
     for (int i = 0; i < K; ++i) {

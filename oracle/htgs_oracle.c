@@ -654,9 +654,12 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
         const float *col = in->rgba + 4 * g;
         if (!eval_instance(in, j, x, y, scale, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
-        /* the reference premultiplies here (:158); the slot keeps colour and alpha apart, as its training kernel
-         * does (forward.cuh:160), so that the tail takes one fused multiply-add per channel */
+        /* The reference premultiplies here (:158) and adds whatever leaves the core to the tail (:168).  Here every
+         * fragment's alpha * colour enters the colour sums when it is evaluated and the final core's share is taken
+         * out after the walk: the same sums up to rounding, and an entry pushed out of the core is dealt with
+         * through its alpha and depth alone. */
         float pm[4] = { col[0], col[1], col[2], f.alpha };
+        for (int k = 0; k < 3; ++k) tail[k] = fmaf(pm[3], pm[k], tail[k]);
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {                          /* :159 */
             for (int i = 0; i < K; ++i) {
                 if (depth < core_depth[i]) {
@@ -665,11 +668,12 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
                 }
             }
         }
-        for (int k = 0; k < 3; ++k) tail[k] = fmaf(pm[3], pm[k], tail[k]);                     /* :168 */
         tail[3] += pm[3];
         if (!median) depth_tail = fmaf(depth, pm[3], depth_tail);                              /* :169 */
         T_tail *= 1.0f - pm[3];                                                                /* :170 */
     }
+    for (int i = 0; i < K; ++i)
+        for (int k = 0; k < 3; ++k) tail[k] = fmaf(-core[i][3], core[i][k], tail[k]);
     float rgb[3] = { 0, 0, 0 }, depth_pixel = 0.0f, T_core = 1.0f;
     for (int i = 0; i < K && T_core >= TRANSMITTANCE_THRESHOLD; ++i) {                         /* :180 */
         const float w = T_core * core[i][3];
@@ -846,6 +850,7 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
         if (!eval_instance(in, j, x, y, scale, min_alpha, 1, NULL, &f)) continue;
         float depth = f.depth;
         float c[4] = { col[0], col[1], col[2], f.alpha };                                      /* :160 */
+        for (int k = 0; k < 3; ++k) tail[k] = fmaf(c[3], c[k], tail[k]);                       /* :173, see hybrid_pixel */
         if (depth < core_depth[K - 1] && f.alpha >= MIN_ALPHA_CORE) {
             uint32_t idx = (uint32_t)g;
             for (int i = 0; i < K; ++i) {
@@ -856,10 +861,11 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
                 }
             }
         }
-        for (int k = 0; k < 3; ++k) tail[k] = fmaf(c[3], c[k], tail[k]);                       /* :173 */
         tail[3] += c[3];
         T_tail *= 1.0f - c[3];
     }
+    for (int i = 0; i < K; ++i)
+        for (int k = 0; k < 3; ++k) tail[k] = fmaf(-core[i][3], core[i][k], tail[k]);
     float rgb[3] = { 0, 0, 0 }, T_core = 1.0f;
     for (int i = 0; i < K && T_core >= TRANSMITTANCE_THRESHOLD; ++i) {                         /* :184-190 */
         const float bw = T_core * core[i][3];
