@@ -134,7 +134,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 // ALPHA_BLEND_FIRST_K: the K nearest fragments with alpha >= 1/20, alpha-blended; no tail.
 // ---------------------------------------------------------------------------------------------
 template <int K>
-__global__ void __launch_bounds__(64) blend_first_k_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
 {

@@ -17,7 +17,7 @@ __device__ __forceinline__ void raise_max(uint32_t *__restrict__ max_weights, ui
 
 // HYBRID_BLEND (TAIL = true, CORE = true), ALPHA_BLEND_FIRST_K (CORE only), OIT_BLEND (TAIL only, K unused)
 template <int K, int MODE>
-__global__ void __launch_bounds__(64) max_weights_tile_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) max_weights_tile_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold)
 {
