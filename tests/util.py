@@ -51,3 +51,15 @@ def gpu_stages(scene_gpu: Scene, mode: int, K=None, to_chw=True, median=False, s
         "sorted_keys": u32(fb.keys[sel])[:n_inst].astype(np.uint64), "sorted_vals": u32(fb.vals[sel])[:n_inst].copy(),
         "ranges": u32(fb.ranges), "image": fb.image.cpu().numpy(), "depth": fb.depth.cpu().numpy(),
     }
+
+
+def load_golden(name: str = "small_scene"):
+    """The frozen known-answer fixture tests/golden/<name>.npz (written by tests/golden/make_fixtures.py from the
+    float64 evaluator): the scene and the arrays of expected outputs."""
+    import os
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name + ".npz"))
+    t = lambda k: torch.from_numpy(z[k].copy())
+    width, height = (int(v) for v in z["size"])
+    scene = Scene(name, t("positions"), t("scales"), t("rotations"), t("opacities"), t("sh_0"), t("sh_rest"), t("M"), t("VPM"),
+                  t("cam_position"), width, height, float(z["planes"][0]), float(z["planes"][1]), int(z["active_sh_bases"]), int(z["K"]))
+    return scene, z
