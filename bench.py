@@ -49,6 +49,7 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 1 GiB copy kernel a few times (reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--train", action="store_true", help="time diff_rasterize forward + backward instead of rasterize")
+    ap.add_argument("--fast", action="store_true", help="time fast_rasterize (image only, hardware reciprocal and 2^x) instead of rasterize")
     return ap.parse_args()
 
 
@@ -120,7 +121,7 @@ def main():
         sys.exit(2)
     import torch
     from htgs_amd.synthetic import make_scene
-    from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode, rasterize
+    from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode, fast_rasterize, rasterize
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -147,6 +148,8 @@ def main():
         return bench_training(args, scene_cpu, scene, settings)
 
     def step():
+        if args.fast:
+            return fast_rasterize(*gauss, settings, True)
         return rasterize(*gauss, settings, True, False)
 
     for _ in range(args.warmup):
@@ -160,7 +163,7 @@ def main():
 
     # ---- per-stage breakdown (HIP events on the launch stream), median over reps -------------------
     reps = max(5, min(30, args.steps))
-    fb = FrameBuffers(*gauss, settings, True, False)
+    fb = FrameBuffers(*gauss, settings, True, False, fast=args.fast)
     fb.front()
     n_inst = fb.read_instance_count()
     fb.alloc_instances(n_inst)
@@ -206,8 +209,8 @@ def main():
     roofline = {
         "kernel": "blend", "bound": "valu_fp32", "achieved": round(achieved_tflops, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved_tflops / FP32_PEAK_TFLOPS, 4),
-        "traffic": MEASURED_BLEND_TRAFFIC.get((args.config, args.mode, args.K, args.n)),
-        "valu_busy": MEASURED_BLEND_VALU_BUSY.get((args.config, args.mode, args.K, args.n)),
+        "traffic": None if args.fast else MEASURED_BLEND_TRAFFIC.get((args.config, args.mode, args.K, args.n)),
+        "valu_busy": None if args.fast else MEASURED_BLEND_VALU_BUSY.get((args.config, args.mode, args.K, args.n)),
         "launch_ms": round(blend_avg_ms, 4), "evals_per_launch": tile_px * n_inst,
     }
 
@@ -225,7 +228,8 @@ def main():
                         "sample": f"one whole frame of the same workload, C oracle with OpenMP, {cpu_s:.2f} s"}
 
     line = {
-        "metric": "FPS HYBRID_BLEND K=16 fwd @1080p, 3M Gaussians" if (args.config, args.mode, args.K) == (2, 0, 16)
+        "metric": f"FPS {MODE_NAMES[args.mode]} K={args.K} fast_rasterize (image only, reduced accuracy)" if args.fast
+        else "FPS HYBRID_BLEND K=16 fwd @1080p, 3M Gaussians" if (args.config, args.mode, args.K) == (2, 0, 16)
         else f"FPS {MODE_NAMES[args.mode]} K={args.K} fwd",
         "value": round(1e3 / ms_per_step, 2), "unit": "FPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

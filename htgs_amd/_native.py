@@ -53,6 +53,7 @@ class Frame(ctypes.Structure):
         ("depth", ctypes.c_void_p),
         ("to_chw", ctypes.c_int32),
         ("use_median_depth", ctypes.c_int32),
+        ("fast_math", ctypes.c_int32),
         ("core_idx", ctypes.c_void_p),
         ("core_info", ctypes.c_void_p),
         ("tail_info", ctypes.c_void_p),

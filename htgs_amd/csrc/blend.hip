@@ -18,14 +18,14 @@ __device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__
     r = saturate(r); g = saturate(g); b = saturate(b);
     if (chw) { image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b; }
     else { image[3 * pix] = r; image[3 * pix + 1] = g; image[3 * pix + 2] = b; }
-    depths[pix] = depth;
+    if (depths) depths[pix] = depth;
 }
 
 // ---------------------------------------------------------------------------------------------
 // HYBRID_BLEND: K nearest fragments with alpha >= 1/20 are alpha-blended in depth order, everything
 // else is merged order-independently into one tail fragment behind them.
 // ---------------------------------------------------------------------------------------------
-template <int K>
+template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
@@ -61,9 +61,9 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             for (int j = 0; j < nb; ++j, stage_advance(addr)) {
                 TileFrag f;
                 if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
-                f.den_rcp = rcp_exact(f.den);
+                f.den_rcp = frag_rcp<FAST>(f.den);
                 const float4 col = stage_row<64, 5>(addr);
-                if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
                 float depth = tile_frag_depth<64>(addr, pt, f);
                 float p3 = f.alpha;
                 tail0 = __builtin_fmaf(p3, col.x, tail0);
@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 }
                 // (depth, p3) is the fragment itself, the entry it pushed out of the core, or an empty slot (alpha 0)
                 tail3 += p3;
-                if (!median) depth_tail = __builtin_fmaf(depth, p3, depth_tail);
+                if (!FAST && !median) depth_tail = __builtin_fmaf(depth, p3, depth_tail);
                 T_tail *= 1.0f - p3;
             }
         }
@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 // ---------------------------------------------------------------------------------------------
 // ALPHA_BLEND_FIRST_K: the K nearest fragments with alpha >= 1/20, alpha-blended; no tail.
 // ---------------------------------------------------------------------------------------------
-template <int K>
+template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
@@ -164,10 +164,10 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             for (int j = 0; j < nb; ++j, stage_advance(addr)) {
                 TileFrag f;
                 if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
-                f.den_rcp = rcp_exact(f.den);
+                f.den_rcp = frag_rcp<FAST>(f.den);
                 float depth = tile_frag_depth<64>(addr, pt, f);
                 if (depth >= cd[K - 1]) continue;                      // depth test before the exponential (:151)
-                if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
                 float alpha = f.alpha;
                 uint32_t idx = stage_index<64>(addr);
 #pragma unroll
@@ -210,6 +210,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 // ---------------------------------------------------------------------------------------------
 // OIT_BLEND: weighted-sum order-independent transparency over all fragments.
 // ---------------------------------------------------------------------------------------------
+template <bool FAST>
 __global__ void __launch_bounds__(64) blend_oit_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw)
@@ -236,14 +237,14 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
             for (int j = 0; j < nb; ++j, stage_advance(addr)) {
                 TileFrag f;
                 if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
-                f.den_rcp = rcp_exact(f.den);
+                f.den_rcp = frag_rcp<FAST>(f.den);
                 const float4 col = stage_row<64, 5>(addr);
-                if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
-                const float depth = tile_frag_depth<64>(addr, pt, f);
+                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
+                const float depth = FAST ? 0.0f : tile_frag_depth<64>(addr, pt, f);
                 a0 = __builtin_fmaf(f.alpha, col.x, a0);
                 a1 = __builtin_fmaf(f.alpha, col.y, a1);
                 a2 = __builtin_fmaf(f.alpha, col.z, a2);
-                a3 = __builtin_fmaf(f.alpha, depth, a3);
+                if (!FAST) a3 = __builtin_fmaf(f.alpha, depth, a3);
                 alpha_sum += f.alpha;
                 T *= 1.0f - f.alpha;
             }
@@ -264,6 +265,7 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
 // ALPHA_BLEND_GLOBAL_ORDERING: instances arrive sorted by (tile, depth of the Gaussian centre);
 // classic front-to-back blending, a pixel stops at T < 1e-4, the workgroup stops when all have.
 // ---------------------------------------------------------------------------------------------
+template <bool FAST>
 __global__ void __launch_bounds__(256) blend_global_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
@@ -290,9 +292,9 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
         for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
             TileFrag f;
             if (!tile_frag_cutoff<256>(addr, pt, f)) continue;
-            f.den_rcp = rcp_exact(f.den);
+            f.den_rcp = frag_rcp<FAST>(f.den);
             const float4 q4 = stage_row<256, 4>(addr);
-            if (!tile_frag_alpha<MODE>(q4.w, f)) continue;
+            if (!tile_frag_alpha<MODE, FAST>(q4.w, f)) continue;
             const float4 col = stage_row<256, 5>(addr);
             const float wgt = T * f.alpha;
             r = __builtin_fmaf(wgt, col.x, r);
@@ -310,17 +312,57 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
-template <int K>
+template <int K, bool FAST>
 static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
-    hipLaunchKernelGGL((blend_hybrid_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
-                       (const float4 *)f->prim, f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+    hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                       (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
+                       f->use_median_depth);
 }
-template <int K>
+template <int K, bool FAST>
 static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
-    hipLaunchKernelGGL((blend_first_k_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
-                       (const float4 *)f->prim, f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+    hipLaunchKernelGGL((blend_first_k_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                       (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
+                       f->use_median_depth);
+}
+
+template <bool FAST>
+static void launch_blend(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
+{
+    const int K = htgs_effective_k(f->K);
+    hipStream_t s = (hipStream_t)f->stream;
+    float *depth = FAST ? nullptr : f->depth;
+    switch (f->mode) {
+        case HTGS_MODE_HYBRID_BLEND:
+            switch (K) {
+                case 32: launch_hybrid<32, FAST>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_hybrid<16, FAST>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_hybrid<8, FAST>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_hybrid<4, FAST>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_hybrid<2, FAST>(f, selector, grid_w, n_tiles); break;
+                default: launch_hybrid<1, FAST>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_ALPHA_BLEND_FIRST_K:
+            switch (K) {
+                case 32: launch_first_k<32, FAST>(f, selector, grid_w, n_tiles); break;
+                case 16: launch_first_k<16, FAST>(f, selector, grid_w, n_tiles); break;
+                case 8: launch_first_k<8, FAST>(f, selector, grid_w, n_tiles); break;
+                case 4: launch_first_k<4, FAST>(f, selector, grid_w, n_tiles); break;
+                case 2: launch_first_k<2, FAST>(f, selector, grid_w, n_tiles); break;
+                default: launch_first_k<1, FAST>(f, selector, grid_w, n_tiles); break;
+            }
+            break;
+        case HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING:
+            hipLaunchKernelGGL(blend_global_kernel<FAST>, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
+                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+            break;
+        default:
+            hipLaunchKernelGGL(blend_oit_kernel<FAST>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
+                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw);
+            break;
+    }
 }
 
 }  // namespace htgs
@@ -337,42 +379,12 @@ extern "C" int htgs_blend(const htgs_frame *f, int selector)
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: null frame");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: bad argument");
-    if (!f->ranges || !f->image || !f->depth || (f->n_instances > 0 && (!f->vals[selector] || !f->prim)))
+    if (!f->ranges || !f->image || (!f->depth && !f->fast_math) || (f->n_instances > 0 && (!f->vals[selector] || !f->prim)))
         return fail(HTGS_ERR_ARGUMENT, "htgs_blend: null pointer");
     const int tile = tile_size(f->mode);
     const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
     const uint32_t n_tiles = grid_w * grid_h;
-    const int K = htgs_effective_k(f->K);
-    hipStream_t s = (hipStream_t)f->stream;
-    switch (f->mode) {
-        case HTGS_MODE_HYBRID_BLEND:
-            switch (K) {
-                case 32: launch_hybrid<32>(f, selector, grid_w, n_tiles); break;
-                case 16: launch_hybrid<16>(f, selector, grid_w, n_tiles); break;
-                case 8: launch_hybrid<8>(f, selector, grid_w, n_tiles); break;
-                case 4: launch_hybrid<4>(f, selector, grid_w, n_tiles); break;
-                case 2: launch_hybrid<2>(f, selector, grid_w, n_tiles); break;
-                default: launch_hybrid<1>(f, selector, grid_w, n_tiles); break;
-            }
-            break;
-        case HTGS_MODE_ALPHA_BLEND_FIRST_K:
-            switch (K) {
-                case 32: launch_first_k<32>(f, selector, grid_w, n_tiles); break;
-                case 16: launch_first_k<16>(f, selector, grid_w, n_tiles); break;
-                case 8: launch_first_k<8>(f, selector, grid_w, n_tiles); break;
-                case 4: launch_first_k<4>(f, selector, grid_w, n_tiles); break;
-                case 2: launch_first_k<2>(f, selector, grid_w, n_tiles); break;
-                default: launch_first_k<1>(f, selector, grid_w, n_tiles); break;
-            }
-            break;
-        case HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING:
-            hipLaunchKernelGGL(blend_global_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
-                               f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
-            break;
-        default:
-            hipLaunchKernelGGL(blend_oit_kernel, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
-                               f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw);
-            break;
-    }
+    if (f->fast_math) launch_blend<true>(f, selector, grid_w, n_tiles);
+    else launch_blend<false>(f, selector, grid_w, n_tiles);
     return check_launch("blend");
 }

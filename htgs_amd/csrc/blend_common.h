@@ -204,11 +204,17 @@ __device__ __forceinline__ float tile_frag_depth(uint32_t addr, const PixelTerms
     return __builtin_fmaf(quad_eval(q3.x, q3.y, q3.z, q3.w, q4.x, q4.y, p), o.den_rcp, q4.z);
 }
 
+// The image-only fast path (FAST) takes the hardware's reciprocal and 2^x (v_rcp_f32, v_exp_f32: one ulp, a quarter of
+// the instruction slots); every other kernel uses the exactly reproducible routines.
+template <bool FAST>
+__device__ __forceinline__ float frag_rcp(float x) { return FAST ? __builtin_amdgcn_rcpf(x) : rcp_exact(x); }
+
 // alpha of the fragment, false below the mode's threshold; needs o.den_rcp
-template <int MODE>
+template <int MODE, bool FAST = false>
 __device__ __forceinline__ bool tile_frag_alpha(float opacity, TileFrag &o)
 {
-    const float G = d_exp2((o.num * ModeCfg<MODE>::exp2_scale) * o.den_rcp);
+    const float t = (o.num * ModeCfg<MODE>::exp2_scale) * o.den_rcp;
+    const float G = FAST ? __builtin_amdgcn_exp2f(t) : d_exp2(t);
     const float a = opacity * G;
     o.alpha = a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha;
     return !(o.alpha < ModeCfg<MODE>::min_alpha);

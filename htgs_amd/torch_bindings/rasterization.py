@@ -103,7 +103,7 @@ class FrameBuffers:
 
     def __init__(self, positions, scales, rotations, opacities, sh_0, sh_rest, settings: RasterizerSettings,
                  to_chw: bool = True, use_median_depth: bool = False, train: bool = False,
-                 pool: Optional[ScratchPool] = None):
+                 pool: Optional[ScratchPool] = None, fast: bool = False):
         mode = _mode_value(settings.mode)
         if mode not in (0, 1, 2, 3):
             raise RuntimeError("unsupported rasterizer mode")
@@ -150,7 +150,8 @@ class FrameBuffers:
         self.ranges = self._scratch("ranges", 2 * self.n_tiles, torch.int32)[:2 * self.n_tiles].view(self.n_tiles, 2)
         self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
                                  dtype=torch.float32, device=dev)
-        self.depth = torch.empty((self.height, self.width), dtype=torch.float32, device=dev)
+        # the image-only fast path (``fast_rasterize``) writes no depth map
+        self.depth = None if fast else torch.empty((self.height, self.width), dtype=torch.float32, device=dev)
         self.keys = [None, None]
         self.vals = [None, None]
         self.sort_tmp = None
@@ -173,7 +174,7 @@ class FrameBuffers:
         f.scan_tmp, f.n_instances_dev = _ptr(self.scan_tmp), _ptr(self.n_instances_dev)
         f.ranges = _ptr(self.ranges)
         f.image, f.depth = _ptr(self.image), _ptr(self.depth)
-        f.to_chw, f.use_median_depth = int(bool(to_chw)), int(bool(use_median_depth))
+        f.to_chw, f.use_median_depth, f.fast_math = int(bool(to_chw)), int(bool(use_median_depth)), int(bool(fast))
         f.stream = torch.cuda.current_stream(dev).cuda_stream
         self.frame = f
         self._ref = ctypes.byref(f)
@@ -405,10 +406,12 @@ def fast_rasterize(
     settings: RasterizerSettings,
     to_chw: bool,
 ) -> torch.Tensor:
-    """The reference's benchmark entry (rasterization.py:166-186): image only.  There it is a reduced-precision
-    build of the inference kernels (half-precision core, fast-math); here the exact fp32 kernels are the fast path,
-    so this is ``rasterize`` without the depth map and the image is the one ``rasterize`` returns."""
+    """The reference's benchmark entry (rasterization.py:166-186): image only, reduced accuracy.  There it is a
+    fast-math build of the inference kernels with a half-precision core; here the same pipeline runs blend kernels that
+    take the hardware's reciprocal and 2^x (one ulp each) instead of the exactly reproducible routines and skip the
+    depth map.  The image agrees with ``rasterize`` to rounding, except at the few pixels where a fragment sits
+    within an ulp of an alpha threshold."""
     with torch.no_grad():
         pool = ScratchPool.current(positions.device) if isinstance(positions, torch.Tensor) and positions.is_cuda else None
-        image, _ = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, settings, to_chw, False, pool=pool).run()
+        image, _ = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, settings, to_chw, False, pool=pool, fast=True).run()
     return image

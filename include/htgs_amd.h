@@ -80,6 +80,9 @@ typedef struct htgs_frame {
     float *depth;              /* [H,W] */
     int32_t to_chw;
     int32_t use_median_depth;
+    int32_t fast_math;         /* htgs_blend only: image-only variant with the hardware's reciprocal and 2^x (one ulp each)
+                                  instead of the exactly reproducible routines; depth is not written and may be NULL
+                                  (the reference's fast_inference kernels, <mode>/kernels/fast_inference.cuh) */
     /* ---- training: per-pixel records (PerPixelBuffers, buffer_utils.h:96-108), pixel-minor ---- */
     uint32_t *core_idx;        /* [Keff,P] primitive of each blended core slot, 0xffffffff = none (modes 0, 1) */
     float *core_info;          /* [Keff,P,4] (dC/dalpha of the slot, blending weight)        (modes 0, 1) */

@@ -91,12 +91,22 @@ def test_refined_reciprocal_equals_division_on_the_whole_guarded_range(cuda):
     assert wrong == 0
 
 
-def test_fast_rasterize_is_the_exact_image(cuda):
+def test_fast_rasterize_agrees_with_rasterize_to_rounding(cuda):
+    """The image-only fast path uses the hardware's reciprocal and 2^x (one ulp each): the image is the exact one to
+    rounding, except where a fragment sits within an ulp of an alpha threshold (1/255: worth 4e-3 of a colour; 1/20, the
+    gate of the sorted core: worth up to 5e-2), which may happen at a handful of pixels."""
     from htgs_amd.torch_bindings import fast_rasterize, rasterize
-    sc = make_scene(0, 5000).to(cuda)
-    for mode in range(4):
-        s = sc.settings(mode, 4)
-        image, _ = rasterize(*sc.gaussians(), s, False, False)
-        fast = fast_rasterize(*sc.gaussians(), s, False)
-        assert fast.shape == (sc.height, sc.width, 3)
-        assert torch.equal(fast, image)
+    for config, n in ((0, 5000), (1, 60_000)):
+        sc = make_scene(config, n).to(cuda)
+        for mode in range(4):
+            print(f"case config={config} mode={mode}", flush=True)
+            s = sc.settings(mode, 16)
+            image, _ = rasterize(*sc.gaussians(), s, False, False)
+            fast = fast_rasterize(*sc.gaussians(), s, False)
+            assert fast.shape == (sc.height, sc.width, 3)
+            diff = (fast - image).abs()
+            assert float(image.max()) > 0.05
+            assert float((diff > 1e-5).float().mean()) < 1e-3
+            assert float(diff.max()) <= 5e-2
+            chw = fast_rasterize(*sc.gaussians(), s, True)
+            assert torch.equal(chw, fast.permute(2, 0, 1))
