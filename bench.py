@@ -49,6 +49,8 @@ def parse_args():
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 1 GiB copy kernel a few times (reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--train", action="store_true", help="time diff_rasterize forward + backward instead of rasterize")
+    ap.add_argument("--densification-rows", type=int, default=0, choices=(0, 2, 3),
+                    help="with --train: pass a densification_info tensor of this many rows to the backward pass")
     ap.add_argument("--fast", action="store_true", help="time fast_rasterize (image only, hardware reciprocal and 2^x) instead of rasterize")
     return ap.parse_args()
 
@@ -74,10 +76,12 @@ def bench_training(args, scene_cpu, scene, settings):
     gauss = scene.gaussians()
     grad_image = torch.randn(3, scene.height, scene.width, generator=torch.Generator().manual_seed(4)).to(gauss[0].device)
 
+    info = torch.zeros((args.densification_rows, scene.positions.shape[0]), device=gauss[0].device) if args.densification_rows else None
+
     def step():
         fb = FrameBuffers(*gauss, settings, True, False, train=True)
         fb.run_forward()
-        return fb, fb.run_backward(grad_image)
+        return fb, fb.run_backward(grad_image, info, info is not None)
 
     for _ in range(args.warmup):
         step()
@@ -90,7 +94,7 @@ def bench_training(args, scene_cpu, scene, settings):
     fb = FrameBuffers(*gauss, settings, True, False, train=True)
     fb.run_forward()
     fwd_blend = statistics.median(event_ms(fb.blend_forward, 10))
-    bwd = statistics.median(event_ms(lambda: fb.run_backward(grad_image), 10))
+    bwd = statistics.median(event_ms(lambda: fb.run_backward(grad_image, info, info is not None), 10))
     cpu_baseline = None
     if not args.no_cpu_baseline:
         import oracle
@@ -108,7 +112,8 @@ def bench_training(args, scene_cpu, scene, settings):
         "unit": "ms/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"{scene.name} {MODE_NAMES[args.mode]} K={args.K} forward+backward, {fb.n} Gaussians, "
-                               f"{scene.width}x{scene.height}", "n_instances": fb.n_instances},
+                               f"{scene.width}x{scene.height}", "n_instances": fb.n_instances,
+                   "densification_rows": args.densification_rows},
         "stages": {"blend_forward_ms": round(fwd_blend, 4), "backward_ms": round(bwd, 4)},
         "cpu_baseline": cpu_baseline}))
 

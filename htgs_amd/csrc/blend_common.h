@@ -6,32 +6,7 @@
 namespace htgs {
 
 // ---------------------------------------------------------------------------------------------
-// plane form: the Gaussian's record as preprocess wrote it (backward kernels)
-// ---------------------------------------------------------------------------------------------
-template <int N>
-struct Stage {
-    float4 v1[N], v2[N], v4[N], mt3[N], col[N];
-};
-
-// Stages one Gaussian record per lane.
-template <int N>
-__device__ __forceinline__ void stage_load(Stage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
-                                           uint32_t fetch, uint32_t last, int slot, uint32_t *idx_out)
-{
-    if (fetch < last) {
-        const uint32_t g = inst[fetch];
-        const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
-        st.v1[slot] = rec[0];
-        st.v2[slot] = rec[1];
-        st.v4[slot] = rec[2];
-        st.mt3[slot] = rec[3];
-        st.col[slot] = rec[4];
-        if (idx_out) idx_out[slot] = g;
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// tile-relative form (forward direction).  With px = px0 - dx VPMT4, py = py0 - dy VPMT4, where px0 / py0 are
+// tile-relative form.  With px = px0 - dx VPMT4, py = py0 - dy VPMT4, where px0 / py0 are
 // the reference's planes (R/include/hybrid_blend/kernels/inference.cuh:137-141) through the tile centre and
 // (dx, dy) is the pixel's offset from it,
 //     d = cross(px.n, py.n)     = A  + dy B  + dx C

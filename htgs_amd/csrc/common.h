@@ -2,11 +2,9 @@
 //
 // Rounding convention.  The whole library is compiled with -ffp-contract=off, so a fused
 // multiply-add exists exactly where __builtin_fmaf is written.  The per-Gaussian stage uses none
-// (operand order of the reference source, R/include/kernel_utils.cuh).  The per-pixel stage has two
-// forms of the reference's ray / Gaussian evaluation: the plane form (frag_cutoff / frag_depth /
-// frag_alpha), kept by the backward pass because it needs the intermediates, and the tile-relative
-// form (TileFrag, blend_common.h) used by every forward-direction kernel, in which |m|^2, |d|^2 and
-// MT3.(d x m) are quadratics of the pixel offset from the tile centre.  log, exp and 2^x are the
+// (operand order of the reference source, R/include/kernel_utils.cuh).  The per-pixel stage evaluates
+// the reference's ray / Gaussian expressions in the tile-relative form (TileFrag, blend_common.h), in which |m|^2, |d|^2 and
+// MT3.(d x m) are quadratics of the pixel offset from the tile centre.  log and 2^x are the
 // polynomial routines below, sqrt and division are correctly rounded
 // (-fhip-fp32-correctly-rounded-divide-sqrt; rcp_exact is the same quotient, cheaper).  The CPU
 // checker used by the test-suite follows the same convention, which is what makes tile counts, sort
@@ -74,25 +72,6 @@ __device__ __forceinline__ float d_logf(float x)
     return fe * 0.693359375f + (lnm + fe * -2.12194440e-4f);
 }
 
-// e^x for x in [-87, 0]: n = rint(x log2 e), r = x - n ln 2, 1 + r + r^2 P(r), scaled through the exponent
-__device__ __forceinline__ float d_expf(float x)
-{
-    const float t = x * 1.44269504088896341f;
-    const float n = __builtin_rintf(t);
-    float r = __builtin_fmaf(n, -0.693359375f, x);
-    r = __builtin_fmaf(n, 2.12194440e-4f, r);
-    float p = 1.9875691500e-4f;
-    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
-    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
-    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
-    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
-    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
-    const float r2 = r * r;
-    const float y = __builtin_fmaf(p, r2, r) + 1.0f;
-    const int ni = (int)n;
-    return bits_to_float((uint32_t)((int)float_to_bits(y) + ni * 8388608));
-}
-
 // 2^t for t in [-126, 1): n = rint(t), r = t - n, degree-5 polynomial of 2^r on [-1/2, 1/2] (relative error 2.7e-7)
 __device__ __forceinline__ float d_exp2(float t)
 {
@@ -126,54 +105,5 @@ __device__ __forceinline__ float rcp_exact(float x)
 
 __device__ __forceinline__ float clamp_pos(float v) { return v > 0.0f ? v : 0.0f; }
 __device__ __forceinline__ float saturate(float v) { return v > 0.0f ? (v < 1.0f ? v : 1.0f) : 0.0f; }
-
-struct Frag {
-    float G, alpha, depth;
-    float num, den, den_rcp;
-    float px[4], py[4], m[3], d[3];
-};
-
-// Ray / Gaussian evaluation of every blend kernel (R/include/hybrid_blend/kernels/inference.cuh:137-155):
-// planes through the pixel in the Gaussian's local frame, distance of their intersection line from the
-// origin, Gaussian weight at the point of maximum contribution.  The camera-space depth of that point is
-// computed separately (frag_depth) because the modes need it at different places.
-template <int MODE>
-__device__ __forceinline__ bool frag_cutoff(const float4 &V1, const float4 &V2, const float4 &V4,
-                                            float fx, float fy, Frag &o)
-{
-    o.px[0] = __builtin_fmaf(-V4.x, fx, V1.x); o.px[1] = __builtin_fmaf(-V4.y, fx, V1.y);
-    o.px[2] = __builtin_fmaf(-V4.z, fx, V1.z); o.px[3] = __builtin_fmaf(-V4.w, fx, V1.w);
-    o.py[0] = __builtin_fmaf(-V4.x, fy, V2.x); o.py[1] = __builtin_fmaf(-V4.y, fy, V2.y);
-    o.py[2] = __builtin_fmaf(-V4.z, fy, V2.z); o.py[3] = __builtin_fmaf(-V4.w, fy, V2.w);
-    const float *px = o.px, *py = o.py;
-    o.m[0] = __builtin_fmaf(px[3], py[0], -(px[0] * py[3]));
-    o.m[1] = __builtin_fmaf(px[3], py[1], -(px[1] * py[3]));
-    o.m[2] = __builtin_fmaf(px[3], py[2], -(px[2] * py[3]));
-    o.d[0] = __builtin_fmaf(px[1], py[2], -(px[2] * py[1]));
-    o.d[1] = __builtin_fmaf(px[2], py[0], -(px[0] * py[2]));
-    o.d[2] = __builtin_fmaf(px[0], py[1], -(px[1] * py[0]));
-    o.num = __builtin_fmaf(o.m[2], o.m[2], __builtin_fmaf(o.m[1], o.m[1], o.m[0] * o.m[0]));
-    o.den = __builtin_fmaf(o.d[2], o.d[2], __builtin_fmaf(o.d[1], o.d[1], o.d[0] * o.d[0]));
-    return !(o.num > ModeCfg<MODE>::cutoff_sq * o.den);
-}
-
-__device__ __forceinline__ float frag_depth(const float4 &MT3, const Frag &o)
-{
-    const float *m = o.m, *d = o.d;
-    const float e0 = __builtin_fmaf(d[1], m[2], -(d[2] * m[1])) * o.den_rcp;
-    const float e1 = __builtin_fmaf(d[2], m[0], -(d[0] * m[2])) * o.den_rcp;
-    const float e2 = __builtin_fmaf(d[0], m[1], -(d[1] * m[0])) * o.den_rcp;
-    return __builtin_fmaf(MT3.z, e2, __builtin_fmaf(MT3.y, e1, MT3.x * e0)) + MT3.w;
-}
-
-// alpha of the fragment; false if below the mode's threshold.  Needs o.den_rcp.
-template <int MODE>
-__device__ __forceinline__ bool frag_alpha(float opacity, Frag &o)
-{
-    o.G = d_expf((-0.5f * o.num) * o.den_rcp);
-    const float a = opacity * o.G;
-    o.alpha = a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha;
-    return !(o.alpha < ModeCfg<MODE>::min_alpha);
-}
 
 }  // namespace htgs
