@@ -224,7 +224,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
                 a0 += t.x * alpha; a1 += t.y * alpha; a2 += t.z * alpha;         // :244
                 const float oma = 1.0f - alpha;
                 dL_dalpha = t.w + (col.x * t.x + col.y * t.y + col.z * t.z)
-                          + s_tail_a[p] * rcp_exact(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255
+                          + s_tail_a[p] * rcp_refined(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);   // :253-255; [1e-8, 1] is inside the refined reciprocal's exact range
             }
             if (dL_dalpha == 0.0f) continue;                                     // :258
             a_op += dL_dalpha * G;                                               // :262
@@ -395,7 +395,7 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
                     acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                        // :171-174
                     n0 = __builtin_fmaf(bw, col.x, n0); n1 = __builtin_fmaf(bw, col.y, n1); n2 = __builtin_fmaf(bw, col.z, n2);   // :178
                     const float oma = 1.0f - alpha;
-                    const float omar = rcp_exact(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);
+                    const float omar = rcp_refined(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);    // [1e-8, 1]: exact there
                     const float dL_dalpha = (T * col.x - (e0 - n0) * omar) * g0 + (T * col.y - (e1 - n1) * omar) * g1
                                           + (T * col.z - (e2 - n2) * omar) * g2;                // :181
                     if (dL_dalpha != 0.0f) {
