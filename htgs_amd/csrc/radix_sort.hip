@@ -118,19 +118,22 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
         key[r] = valid ? keys_in[i] : (KeyT)0;
         val[r] = valid ? vals_in[i] : 0u;
         const uint32_t d = digit_of(key[r], shift, mask);
-        // lanes of this wave holding the same digit
-        uint64_t peers = __ballot(valid);
+        // lanes of this wave holding the same digit: per digit bit, keep the lanes whose bit equals this lane's.
+        // (bit as 0 / ~0 by a signed bit-field extract; keep = peers & ~(vote ^ bit) is one three-input operation per half)
+        const uint64_t present = __ballot(valid);
+        uint32_t peers_lo = (uint32_t)present, peers_hi = (uint32_t)(present >> 32);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            const bool bit = (d >> b) & 1u;
-            const uint64_t vote = __ballot(bit);
-            peers &= bit ? vote : ~vote;
+            const uint32_t bit = (uint32_t)__builtin_amdgcn_sbfe((int)d, b, 1);
+            const uint64_t vote = __ballot(bit != 0u);
+            peers_lo &= ~((uint32_t)vote ^ bit);
+            peers_hi &= ~((uint32_t)(vote >> 32) ^ bit);
         }
-        const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
         uint32_t seen = 0;
         if (valid) {
             seen = counts[wave][d];
-            if (below == 0) counts[wave][d] = seen + (uint32_t)__builtin_popcountll(peers);
+            if (below == 0) counts[wave][d] = seen + (uint32_t)(__builtin_popcount(peers_lo) + __builtin_popcount(peers_hi));
         }
         rank[r] = seen + below;
     }
