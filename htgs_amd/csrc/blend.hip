@@ -26,7 +26,7 @@ __device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__
 // else is merged order-independently into one tail fragment behind them.
 // ---------------------------------------------------------------------------------------------
 template <int K, bool FAST>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_hybrid_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
 {
