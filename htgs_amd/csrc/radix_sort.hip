@@ -17,10 +17,10 @@ constexpr int kSortItems = 16;                              // rounds per wave
 constexpr int kRadix = 256;
 constexpr int kDigitWaves = kRadix / kWave;                 // the waves whose threads own one digit each
 constexpr int kScanThreads = 256;
-// Items per block = threads x 16.  Longer blocks give longer runs per digit, i.e. fuller cache lines in the
-// scatter; 8-byte keys stay at 256 threads so that two blocks still fit a CU's LDS.
-template <typename KeyT> struct SortShape { static constexpr int threads = sizeof(KeyT) == 8 ? 256 : 512; };
-constexpr int kSortTileMin = 256 * kSortItems;              // the smallest block (sizes the histogram scratch)
+// Items per block = threads x 16 = 8192.  Longer blocks give longer runs per digit, i.e. fuller cache lines in the
+// scatter; two blocks fit a CU's LDS for every key width (8-byte keys share one array between keys and values).
+template <typename KeyT> struct SortShape { static constexpr int threads = 512; };
+constexpr int kSortTileMin = 256 * kSortItems;              // sizes the histogram scratch (half a block: room to spare)
 
 template <typename KeyT>
 __device__ __forceinline__ uint32_t digit_of(KeyT k, int shift, uint32_t mask) { return (uint32_t)(k >> shift) & mask; }
@@ -101,7 +101,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
     __shared__ uint32_t global_base[kRadix];           // where the block's run of each digit starts in the output
     __shared__ uint32_t wave_sums[kDigitWaves], wave_sums_g[kDigitWaves];
     // The block's items grouped by digit (stable).  8-byte keys: the values follow the keys through the same memory, in a
-    // second round, which lets four blocks instead of two share a CU's LDS (sort of 9 M pairs 0.61 -> 0.50 ms); for the
+    // second round, which halves the block's LDS and allows 8192-item blocks here as well (sort of 9 M pairs 0.61 -> 0.47 ms); for the
     // short keys the second round costs more than the third resident block gains (0.24 -> 0.29 ms), so keys and values
     // have their own arrays there.
     constexpr bool kTwoRounds = sizeof(KeyT) == 8;
