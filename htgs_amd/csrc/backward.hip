@@ -124,46 +124,52 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
     const size_t np = (size_t)width * height;
-    if (wave == 0) {
+    {
+        // per-pixel terms into LDS: lane = pixel; the tail's by the first wave, the K core slots shared out over the four
         const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-        float4 tail = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        float tail_a = 0.0f;
         const bool inside = x < width && y < height;
         const size_t pix = inside ? (size_t)width * y + x : 0;
         float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f;
         if (inside) { g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix]; }
-        if (inside && kHasTail) {
-            const float r0 = tail_info[pix], r1 = tail_info[np + pix], r2 = tail_info[2 * np + pix];
-            const float asr = tail_info[3 * np + pix], T_tail = tail_info[4 * np + pix], T_core = tail_info[5 * np + pix];
-            const float w_tail = T_core * asr;                                   // backward.cuh:166
-            const float full = w_tail * (1.0f - T_tail);                         // :168
-            const float rdg = r0 * g0 + r1 * g1 + r2 * g2;
-            tail = make_float4(full * g0, full * g1, full * g2, -full * asr * rdg);   // :170-172
-            tail_a = w_tail * T_tail * rdg;                                      // :173
-        }
-        s_tail[lane] = tail;
-        s_tail_a[lane] = tail_a;
-        if (HELPER) {
-            // dL/dVPMT4.w = -x dL/dpx.w - y dL/dpy.w (:288), and dL/dposition = VPM[:, :3]^T of the three w components (:292-305)
-            const float fx = (float)x, fy = (float)y;
+        if (wave == 0) {
+            float4 tail = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            float tail_a = 0.0f;
+            if (inside && kHasTail) {
+                const float r0 = tail_info[pix], r1 = tail_info[np + pix], r2 = tail_info[2 * np + pix];
+                const float asr = tail_info[3 * np + pix], T_tail = tail_info[4 * np + pix], T_core = tail_info[5 * np + pix];
+                const float w_tail = T_core * asr;                                   // backward.cuh:166
+                const float full = w_tail * (1.0f - T_tail);                         // :168
+                const float rdg = r0 * g0 + r1 * g1 + r2 * g2;
+                tail = make_float4(full * g0, full * g1, full * g2, -full * asr * rdg);   // :170-172
+                tail_a = w_tail * T_tail * rdg;                                      // :173
+            }
+            s_tail[lane] = tail;
+            s_tail_a[lane] = tail_a;
+            if (HELPER) {
+                // dL/dVPMT4.w = -x dL/dpx.w - y dL/dpy.w (:288), and dL/dposition = VPM[:, :3]^T of the three w components (:292-305)
+                const float fx = (float)x, fy = (float)y;
 #pragma unroll
-            for (int k = 0; k < 3; ++k) {
-                s_pos[lane][k] = __builtin_fmaf(-fx, VPM[12 + k], VPM[k]);
-                s_pos[lane][3 + k] = __builtin_fmaf(-fy, VPM[12 + k], VPM[4 + k]);
+                for (int k = 0; k < 3; ++k) {
+                    s_pos[lane][k] = __builtin_fmaf(-fx, VPM[12 + k], VPM[k]);
+                    s_pos[lane][3 + k] = __builtin_fmaf(-fy, VPM[12 + k], VPM[4 + k]);
+                }
             }
         }
         if (K > 0) {
 #pragma unroll
-            for (int i = 0; i < KS; ++i) {
-                uint32_t idx = 0xffffffffu;
-                float4 c = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-                if (inside) {
-                    idx = core_idx[(size_t)i * np + pix];
-                    const float4 info = core_info[(size_t)i * np + pix];
-                    c = make_float4(info.w * g0, info.w * g1, info.w * g2, info.x * g0 + info.y * g1 + info.z * g2);   // :154-155
+            for (int i0 = 0; i0 < KS; i0 += kBackwardWaves) {
+                const int i = i0 + (int)wave;
+                if (i < KS) {
+                    uint32_t idx = 0xffffffffu;
+                    float4 c = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    if (inside) {
+                        idx = core_idx[(size_t)i * np + pix];
+                        const float4 info = core_info[(size_t)i * np + pix];
+                        c = make_float4(info.w * g0, info.w * g1, info.w * g2, info.x * g0 + info.y * g1 + info.z * g2);   // :154-155
+                    }
+                    s_idx[lane * KS + i] = idx == 0xffffffffu ? idx : (idx << kSlotBits) | (uint32_t)i;
+                    s_core[lane * KS + i] = c;
                 }
-                s_idx[lane * KS + i] = idx == 0xffffffffu ? idx : (idx << kSlotBits) | (uint32_t)i;
-                s_core[lane * KS + i] = c;
             }
         }
     }
