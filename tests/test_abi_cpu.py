@@ -111,3 +111,12 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_native, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _native.lib()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One frame is rendered on one GPU; asking bench.py for more must end with a message, not with a wrong figure."""
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 2
+    assert "--gpus must be 1" in out.stderr and out.stdout.strip() == ""
