@@ -106,7 +106,7 @@ __device__ __forceinline__ void moments_to_rows(const float4 &V1, const float4 &
 // the fourth components of the fragment's dL/dVPMT rows, which need m and the two plane normals at the pixel.
 // ---------------------------------------------------------------------------------------------
 template <int K, int MODE, bool HELPER>
-__global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_waves_per_eu(5))) blend_tail_backward_moments_kernel(
+__global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_moments_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
     const float *__restrict__ grad_image, const float *__restrict__ VPM, const uint32_t *__restrict__ offsets,
