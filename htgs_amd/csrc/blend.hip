@@ -7,6 +7,8 @@
 // An 8x8 tile is exactly one wave64: one workgroup = one wave, Gaussian records are staged 64 at a
 // time in LDS (every lane then reads the same address, a broadcast), the K-buffer lives in VGPRs.
 // The 16x16 tiles of the global-ordering mode use four waves and a workgroup barrier.
+// Every kernel has a second instantiation, FAST, for the image-only path of the reference's fast_inference
+// kernels (R/include/<mode>/kernels/fast_inference.cuh): hardware reciprocal and 2^x, no depth.
 #include "blend_common.h"
 
 namespace htgs {
