@@ -256,6 +256,8 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_momen
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
     const size_t np = (size_t)width * height;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    if (first == last) return;               // nothing was drawn into this tile (whole workgroup)
     {
         // per-pixel terms into LDS: lane = pixel; the tail's by the first wave, the K core slots shared out over the four
         const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
@@ -308,7 +310,6 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) blend_tail_backward_momen
     __syncthreads();
 
     const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
-    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first + 64 * wave; base < last; base += 64 * kBackwardWaves) {
         // a short batch (the ragged end of the tile's list) shares the wave among two or four groups of pixels
         const uint32_t n_here = last - base;                                  // wave-uniform
