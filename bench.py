@@ -33,7 +33,7 @@ FLOPS_PER_EVAL = 46
 # same counters on a plain 1 GiB copy (fetch x 2.000, write x 1.000); profiles/inference_cfg2_3M_1080p_hybrid_k16.md
 MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3198286548}
 # VALUBusy of the blend kernel by the profiler's formula, SQ_ACTIVE_INST_VALU x 4 / (SIMDs x kernel cycles), capped at 1
-# (same profile; indicative: partly filled waves retire instructions in fewer than four cycles)
+# (same profile; indicative, not a calibrated share of time)
 MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 1.0}
 
 
