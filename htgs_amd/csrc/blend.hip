@@ -54,13 +54,13 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
-            const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
-            uint32_t addr = stage_address(st);
-            for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+            const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+            while (hits) {
+                const uint32_t addr = stage_next_hit(hits, stage_base);
                 TileFrag f;
                 if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
                 f.den_rcp = frag_rcp<FAST>(f.den);
@@ -158,12 +158,12 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
-            const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
-            uint32_t addr = stage_address(st);
-            for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+            const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+            while (hits) {
+                const uint32_t addr = stage_next_hit(hits, stage_base);
                 TileFrag f;
                 if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
                 f.den_rcp = frag_rcp<FAST>(f.den);
@@ -231,12 +231,12 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
-            const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
-            uint32_t addr = stage_address(st);
-            for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+            const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+            while (hits) {
+                const uint32_t addr = stage_next_hit(hits, stage_base);
                 TileFrag f;
                 if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
                 f.den_rcp = frag_rcp<FAST>(f.den);
@@ -314,6 +314,44 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
+// Self-check of the staging cull (tile_stage_load with CULL): every instance of every 8x8 tile is evaluated at all 64
+// pixels with the blend kernels' own cut-off and alpha tests and the outcome is compared with the verdict of the lane
+// that staged it.  counts: instances looked at, instances that reach no pixel, reported misses, wrong misses.
+template <int MODE>
+__global__ void __launch_bounds__(64) check_tile_cull_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t grid_w,
+    unsigned long long *__restrict__ counts)
+{
+    __shared__ TileStage<64> st;
+    const uint32_t tile = blockIdx.x, lane = threadIdx.x;
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
+    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    unsigned long long seen = 0, empty = 0, missed = 0, wrong = 0;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 64) {
+        __syncthreads();
+        const uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        __syncthreads();
+        const int nb = last - base < 64u ? (int)(last - base) : 64;
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+            TileFrag f;
+            bool pass = tile_frag_cutoff<64>(addr, pt, f);
+            if (pass) {
+                f.den_rcp = rcp_exact(f.den);
+                pass = tile_frag_alpha<MODE>(stage_opacity<64>(addr), f);
+            }
+            const bool any = __any(pass), miss = !((hits >> j) & 1);
+            ++seen; empty += !any; missed += miss; wrong += miss && any;
+        }
+    }
+    if (lane == 0 && seen) {
+        atomicAdd(counts, seen); atomicAdd(counts + 1, empty); atomicAdd(counts + 2, missed);
+        if (wrong) atomicAdd(counts + 3, wrong);
+    }
+}
+
 template <int K, bool FAST>
 static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
@@ -389,4 +427,23 @@ extern "C" int htgs_blend(const htgs_frame *f, int selector)
     if (f->fast_math) launch_blend<true>(f, selector, grid_w, n_tiles);
     else launch_blend<false>(f, selector, grid_w, n_tiles);
     return check_launch("blend");
+}
+
+extern "C" int htgs_check_tile_cull(const htgs_frame *f, int selector, unsigned long long *counts)
+{
+    if (!f || !counts) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: null pointer");
+    if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
+    if (f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING) return fail(HTGS_ERR_MODE, "htgs_check_tile_cull: the 16x16-tile mode does not cull");
+    if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: bad argument");
+    if (!f->ranges || (f->n_instances > 0 && (!f->vals[selector] || !f->prim))) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: null pointer");
+    const uint32_t grid_w = div_up(f->width, 8), n_tiles = grid_w * div_up(f->height, 8);
+    hipStream_t s = (hipStream_t)f->stream;
+    const float4 *prim = (const float4 *)f->prim;
+    if (f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K)
+        hipLaunchKernelGGL(check_tile_cull_kernel<HTGS_MODE_ALPHA_BLEND_FIRST_K>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], prim, grid_w, counts);
+    else if (f->mode == HTGS_MODE_OIT_BLEND)
+        hipLaunchKernelGGL(check_tile_cull_kernel<HTGS_MODE_OIT_BLEND>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], prim, grid_w, counts);
+    else
+        hipLaunchKernelGGL(check_tile_cull_kernel<HTGS_MODE_HYBRID_BLEND>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], prim, grid_w, counts);
+    return check_launch("check_tile_cull");
 }

@@ -71,13 +71,58 @@ __device__ __forceinline__ void tile_quadratics(const TileGeometry &g, float (&n
     d[3] = dotf(g.C, g.C); d[4] = 2.0f * dotf(g.B, g.C); d[5] = dotf(g.B, g.B);
 }
 
+// True when no pixel of the tile can pass both the cut-off and the alpha test of an instance, given the
+// coefficients of |m|^2 / cut-off (n) and |d|^2 (d) and the opacity.  The cut-off is 2 ln(1 / min_alpha) in every
+// mode, so opacity * exp(-rho^2 / 2) >= min_alpha is n / d <= 1 + log2(opacity) / log2(1 / min_alpha) =: r, and both
+// tests together are  Q = n - min(r, 1) d <= 0.  Q is a quadratic of the pixel offset; per pixel row its least value
+// over the row's pixels is at the pixel next to the vertex (or at a row end), so one evaluation per row gives the
+// least Q over the tile.  The margin (1e-5 of the sum of the magnitudes of all terms, with r raised by 1e-5) is an
+// order of magnitude above the rounding of the per-pixel evaluation, of 2^x and of this routine; non-finite
+// coefficients never report a miss.
+template <int MODE>
+__device__ __forceinline__ bool tile_misses(const float (&n)[6], const float (&d)[6], float opacity)
+{
+    constexpr int rows = ModeCfg<MODE>::tile;
+    constexpr float h = 0.5f * (float)(rows - 1);
+    float r = __builtin_fmaf(__builtin_amdgcn_logf(opacity), -1.0f / ModeCfg<MODE>::exp2_scale, 1.0f);
+    r = r < 1.0f ? r : 1.0f;                       // (also a NaN opacity: the cut-off alone decides)
+    r = r > -1.0f ? r : -1.0f;
+    r += 1e-5f;
+    float q[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) q[i] = __builtin_fmaf(-r, d[i], n[i]);
+    const float s0 = __builtin_fabsf(n[0]) + __builtin_fabsf(d[0]);
+    const float s1 = (__builtin_fabsf(n[1]) + __builtin_fabsf(d[1])) + (__builtin_fabsf(n[2]) + __builtin_fabsf(d[2]));
+    const float s2 = ((__builtin_fabsf(n[3]) + __builtin_fabsf(d[3])) + (__builtin_fabsf(n[4]) + __builtin_fabsf(d[4]))) +
+                     (__builtin_fabsf(n[5]) + __builtin_fabsf(d[5]));
+    const float margin = 1e-5f * __builtin_fmaf(h * h, s2, __builtin_fmaf(h, s1, s0));
+    const bool convex = q[3] > 0.0f;
+    const float to_vertex = -0.5f * __builtin_amdgcn_rcpf(q[3]);
+    float least = __FLT_MAX__;
+#pragma nounroll
+    for (int row = 0; row < rows; ++row) {           // (kept a loop: unrolled, the rows crowd the callers' K-buffers out of registers)
+        const float y = (float)row - h;
+        const float b = __builtin_fmaf(q[4], y, q[1]);
+        const float c = __builtin_fmaf(y, __builtin_fmaf(q[5], y, q[2]), q[0]);
+        float xv = __builtin_rintf(__builtin_fmaf(b, to_vertex, 0.5f)) - 0.5f;
+        xv = __builtin_fminf(__builtin_fmaxf(xv, -h), h);
+        const float xe = b > 0.0f ? -h : h;
+        const float x = convex ? xv : xe;
+        least = __builtin_fminf(least, __builtin_fmaf(x, __builtin_fmaf(q[3], x, b), c));
+    }
+    return least > margin;
+}
+
 // (the same arithmetic as tile_geometry / tile_quadratics, written out so that every row is stored as soon as it is
 // complete: the kernels that call this hold a K-buffer in registers)
-template <int MODE, int N, bool DEPTH>
-__device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
+// Returns whether the slot holds an instance that can reach a pixel of the tile: always true for a loaded slot
+// unless CULL asks for tile_misses.  What that leaves out contributes to no pixel, so a walk over the hits alone
+// gives the results of the full walk bit for bit.
+template <int MODE, int N, bool DEPTH, bool CULL = false>
+__device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                 uint32_t fetch, uint32_t last, int slot, float cx, float cy)
 {
-    if (fetch >= last) return;
+    if (fetch >= last) return false;
     const uint32_t g = inst[fetch];
     const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
     const float4 r1 = rec[0], r2 = rec[1], r4 = rec[2], r3 = rec[3], col = rec[4];
@@ -98,10 +143,6 @@ __device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *
         Bm[k] = __builtin_fmaf(px0[k], V4[3], -(px0[3] * V4[k]));
         Cm[k] = __builtin_fmaf(V4[k], py0[3], -(V4[3] * py0[k]));
     }
-    constexpr float kc = ModeCfg<MODE>::cutoff_rcp;
-    st.q[0][slot] = make_float4(dotf(Am, Am) * kc, (2.0f * dotf(Am, Cm)) * kc, (2.0f * dotf(Am, Bm)) * kc, dotf(Cm, Cm) * kc);
-    st.q[1][slot] = make_float4((2.0f * dotf(Bm, Cm)) * kc, dotf(Bm, Bm) * kc, dotf(A, A), 2.0f * dotf(A, C));
-    st.q[2][slot] = make_float4(2.0f * dotf(A, B), dotf(C, C), 2.0f * dotf(B, C), dotf(B, B));
     float zxy = 0.0f, zyy = 0.0f;
     if (DEPTH) {
         const float MT3[3] = { r3.x, r3.y, r3.z };
@@ -115,6 +156,14 @@ __device__ __forceinline__ void tile_stage_load(TileStage<N> &st, const float4 *
     }
     st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
     st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
+    constexpr float kc = ModeCfg<MODE>::cutoff_rcp;
+    const float n[6] = { dotf(Am, Am) * kc, (2.0f * dotf(Am, Cm)) * kc, (2.0f * dotf(Am, Bm)) * kc,
+                         dotf(Cm, Cm) * kc, (2.0f * dotf(Bm, Cm)) * kc, dotf(Bm, Bm) * kc };
+    const float d[6] = { dotf(A, A), 2.0f * dotf(A, C), 2.0f * dotf(A, B), dotf(C, C), 2.0f * dotf(B, C), dotf(B, B) };
+    st.q[0][slot] = make_float4(n[0], n[1], n[2], n[3]);
+    st.q[1][slot] = make_float4(n[4], n[5], d[0], d[1]);
+    st.q[2][slot] = make_float4(d[2], d[3], d[4], d[5]);
+    return CULL ? !tile_misses<MODE>(n, d, col.w) : true;
 }
 
 // the pixel's offset from the tile centre (exact)
@@ -150,6 +199,16 @@ typedef __attribute__((address_space(3))) const float lds_float;
 template <int N>
 __device__ __forceinline__ uint32_t stage_address(const TileStage<N> &st) { return (uint32_t)(uintptr_t)(lds_float4 *)&st.q[0][0]; }
 __device__ __forceinline__ void stage_advance(uint32_t &addr) { asm volatile("v_add_u32 %0, 16, %0" : "+v"(addr)); }
+// the walk over the hits of a batch: takes the lowest set bit of the (wave-uniform) mask and returns the LDS address
+// of that slot's q[0] entry, again through an opaque move so that one VGPR serves every read of the iteration
+__device__ __forceinline__ uint32_t stage_next_hit(uint64_t &hits, uint32_t stage_base)
+{
+    const uint32_t at = stage_base + 16u * (uint32_t)__builtin_ctzll(hits);
+    hits &= hits - 1;
+    uint32_t addr;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(addr) : "s"(at));
+    return addr;
+}
 template <int N, int ROW>
 __device__ __forceinline__ float4 stage_row(uint32_t addr)
 {

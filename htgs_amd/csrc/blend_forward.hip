@@ -43,11 +43,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
-        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
-        uint32_t addr = stage_address(st);
-        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+        while (hits) {
+            const uint32_t addr = stage_next_hit(hits, stage_base);
             TileFrag f;
             if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
@@ -165,11 +165,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<MODE, 64, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
-        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
-        uint32_t addr = stage_address(st);
-        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+        while (hits) {
+            const uint32_t addr = stage_next_hit(hits, stage_base);
             TileFrag f;
             if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
@@ -255,11 +255,11 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        tile_stage_load<MODE, 64, false>(st, prim, inst, base + lane, last, lane, cx, cy);
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
-        const int nb = __builtin_amdgcn_readfirstlane(last - base < 64u ? (int)(last - base) : 64);
-        uint32_t addr = stage_address(st);
-        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+        while (hits) {
+            const uint32_t addr = stage_next_hit(hits, stage_base);
             TileFrag f;
             if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
             f.den_rcp = rcp_exact(f.den);
