@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
@@ -158,7 +158,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
@@ -231,7 +231,7 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
@@ -331,7 +331,7 @@ __global__ void __launch_bounds__(64) check_tile_cull_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        const uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        const uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         uint32_t addr = stage_address(st);

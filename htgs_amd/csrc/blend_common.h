@@ -116,9 +116,11 @@ __device__ __forceinline__ bool tile_misses(const float (&n)[6], const float (&d
 // (the same arithmetic as tile_geometry / tile_quadratics, written out so that every row is stored as soon as it is
 // complete: the kernels that call this hold a K-buffer in registers)
 // Returns whether the slot holds an instance that can reach a pixel of the tile: always true for a loaded slot
-// unless CULL asks for tile_misses.  What that leaves out contributes to no pixel, so a walk over the hits alone
-// gives the results of the full walk bit for bit.
-template <int MODE, int N, bool DEPTH, bool CULL = false>
+// unless CULL asks for tile_misses -- for walks that apply the cut-off and the alpha threshold (kCullAlpha), or the
+// cut-off alone (kCullCutoff: the test with opacity 1).  What that leaves out contributes to no pixel, so a walk over
+// the hits alone gives the results of the full walk bit for bit.
+enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2 };
+template <int MODE, int N, bool DEPTH, int CULL = kCullNone>
 __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                 uint32_t fetch, uint32_t last, int slot, float cx, float cy)
 {
@@ -163,7 +165,7 @@ __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *
     st.q[0][slot] = make_float4(n[0], n[1], n[2], n[3]);
     st.q[1][slot] = make_float4(n[4], n[5], d[0], d[1]);
     st.q[2][slot] = make_float4(d[2], d[3], d[4], d[5]);
-    return CULL ? !tile_misses<MODE>(n, d, col.w) : true;
+    return CULL == kCullNone ? true : !tile_misses<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
 }
 
 // the pixel's offset from the tile centre (exact)

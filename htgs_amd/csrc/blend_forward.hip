@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         while (hits) {
@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         while (hits) {
@@ -255,7 +255,7 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         while (hits) {

@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, kCore, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, kCore, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         while (hits) {
@@ -91,10 +91,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     if (inside && alpha_sum >= weight_threshold) tail_weight = (T_core * (1.0f - T_tail)) * (1.0f / alpha_sum);
     const bool active = inside && tail_weight >= weight_threshold;
     if (!__any(active)) return;
-    // second walk over the tile's list: alpha * tail weight for every fragment that passes the cut-off
+    // second walk over the tile's list: alpha * tail weight for every fragment that passes the cut-off (no alpha
+    // threshold here, R/include/hybrid_blend/kernels/update_max_weights.cuh:197-204)
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, kCullCutoff>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         while (hits) {

@@ -31,6 +31,25 @@ def test_max_weights_bit_exact(cuda, config, n, K, mode):
     assert (want > start).sum() > n // 50
 
 
+@pytest.mark.parametrize("threshold", [1e-4, 0.0])
+@pytest.mark.parametrize("mode", [0, 3])
+def test_weight_threshold_below_the_alpha_threshold(cuda, mode, threshold):
+    """The tail's second walk has no alpha threshold (only the cut-off), so with a weight threshold under 1/255 a
+    fragment too faint for the blend still raises its Gaussian's weight; faint Gaussians make that the common case."""
+    print(f"case mode={mode} threshold={threshold}", flush=True)
+    n = 20_000
+    scene = make_scene(1, n)
+    scene.opacities.mul_(torch.rand(n, 1, generator=torch.Generator().manual_seed(5)) ** 3)
+    want = np.zeros(n, dtype=np.float32)
+    oracle.update_max_weights(oracle_frame(scene, mode, 8), want, *[t.numpy() for t in scene.gaussians()[:4]], threshold)
+    sg = scene.to(cuda)
+    got = torch.zeros(n, 1, device=cuda)
+    update_max_weights(got, *sg.gaussians()[:4], sg.settings(RasterizerMode(mode), 8), threshold)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(got.cpu().numpy().reshape(-1).view(np.uint32), want.view(np.uint32))
+    assert ((want > 0) & (want < 1.0 / 255.0)).sum() > n // 100
+
+
 def test_two_views_accumulate(cuda):
     scene = make_scene(0, 4000).to(cuda)
     mw = torch.zeros(4000, device=cuda)
