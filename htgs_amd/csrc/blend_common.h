@@ -113,12 +113,12 @@ __device__ __forceinline__ bool tile_misses(const float (&n)[6], const float (&d
     return least > margin;
 }
 
-// (the same arithmetic as tile_geometry / tile_quadratics, written out so that every row is stored as soon as it is
-// complete: the kernels that call this hold a K-buffer in registers)
-// Returns whether the slot holds an instance that can reach a pixel of the tile: always true for a loaded slot
-// unless CULL asks for tile_misses -- for walks that apply the cut-off and the alpha threshold (kCullAlpha), or the
-// cut-off alone (kCullCutoff: the test with opacity 1).  What that leaves out contributes to no pixel, so a walk over
-// the hits alone gives the results of the full walk bit for bit.
+// Stages instance `fetch` of the sorted list in slot `slot` (the same arithmetic as tile_geometry / tile_quadratics,
+// written out so that every row is stored as soon as it is complete: the kernels that call this hold a K-buffer in
+// registers).  Returns whether the slot holds an instance that can reach a pixel of the tile: always true for a
+// loaded slot unless CULL asks for tile_misses -- for walks that apply the cut-off and the alpha threshold
+// (kCullAlpha), or the cut-off alone (kCullCutoff: the test with opacity 1).  What that leaves out contributes to
+// no pixel, so a walk over the hits alone gives the results of the full walk bit for bit.
 enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2 };
 template <int MODE, int N, bool DEPTH, int CULL = kCullNone>
 __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
