@@ -31,7 +31,7 @@ FP32_PEAK_TFLOPS = 157.3
 FLOPS_PER_EVAL = 46
 # HBM bytes of one blend launch of the default workload: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
 # same counters on a plain 1 GiB copy (fetch x 2.000, write x 1.000); profiles/inference_cfg2_3M_1080p_hybrid_k16.md
-MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3791557452}
+MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3205669118}
 # VALUBusy of the blend kernel by the profiler's formula, SQ_ACTIVE_INST_VALU x 4 / (SIMDs x kernel cycles), capped at 1
 # (same profile; indicative, not a calibrated share of time)
 MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 1.0}

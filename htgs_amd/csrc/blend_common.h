@@ -127,7 +127,12 @@ __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *
     if (fetch >= last) return false;
     const uint32_t g = inst[fetch];
     const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
-    const float4 r1 = rec[0], r2 = rec[1], r4 = rec[2], r3 = rec[3], col = rec[4];
+    // (with CULL the record's colour row is fetched when it is needed, behind a compiler fence: it comes from a cache
+    // line the other rows have just brought in, and four registers less at the peak keep the callers' K-buffers out
+    // of scratch memory inside the batch loop)
+    const float4 r1 = rec[0], r2 = rec[1], r4 = rec[2], r3 = rec[3];
+    float4 col;
+    if (CULL == kCullNone) col = rec[4];
     const float V1[4] = { r1.x, r1.y, r1.z, r1.w }, V2[4] = { r2.x, r2.y, r2.z, r2.w }, V4[4] = { r4.x, r4.y, r4.z, r4.w };
     float px0[4], py0[4];
 #pragma unroll
@@ -156,8 +161,6 @@ __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *
         zxy = dotf(PB, Cm) + dotf(PC, Bm);
         zyy = dotf(PB, Bm);
     }
-    st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
-    st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
     constexpr float kc = ModeCfg<MODE>::cutoff_rcp;
     const float n[6] = { dotf(Am, Am) * kc, (2.0f * dotf(Am, Cm)) * kc, (2.0f * dotf(Am, Bm)) * kc,
                          dotf(Cm, Cm) * kc, (2.0f * dotf(Bm, Cm)) * kc, dotf(Bm, Bm) * kc };
@@ -165,6 +168,12 @@ __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *
     st.q[0][slot] = make_float4(n[0], n[1], n[2], n[3]);
     st.q[1][slot] = make_float4(n[4], n[5], d[0], d[1]);
     st.q[2][slot] = make_float4(d[2], d[3], d[4], d[5]);
+    if (CULL != kCullNone) {
+        asm volatile("" ::: "memory");
+        col = rec[4];
+    }
+    st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
+    st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
     return CULL == kCullNone ? true : !tile_misses<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
 }
 
