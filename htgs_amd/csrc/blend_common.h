@@ -265,9 +265,18 @@ __device__ __forceinline__ bool tile_frag_alpha(float opacity, TileFrag &o)
     return !(o.alpha < ModeCfg<MODE>::min_alpha);
 }
 
-// exchange two VGPRs in the active lanes (one instruction instead of a select pair)
-__device__ __forceinline__ void vswap(float &a, float &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
-__device__ __forceinline__ void vswap(uint32_t &a, uint32_t &b) { asm volatile("v_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+// exchange two VGPRs in the active lanes: three moves through a scratch register (a wave64 v_mov_b32 holds the
+// vector ALU for two cycles, v_swap_b32 for eight, v_cndmask_b32 for four)
+__device__ __forceinline__ void vswap(float &a, float &b)
+{
+    float t;
+    asm volatile("v_mov_b32 %2, %0\n\tv_mov_b32 %0, %1\n\tv_mov_b32 %1, %2" : "+v"(a), "+v"(b), "=&v"(t));
+}
+__device__ __forceinline__ void vswap(uint32_t &a, uint32_t &b)
+{
+    uint32_t t;
+    asm volatile("v_mov_b32 %2, %0\n\tv_mov_b32 %0, %1\n\tv_mov_b32 %1, %2" : "+v"(a), "+v"(b), "=&v"(t));
+}
 
 // Sorted insertion into a K-slot buffer walks the slots front to back carrying the displaced entry; the kernels
 // take the slots four at a time and the whole wave skips a group that no active lane can change (the carried

@@ -72,10 +72,13 @@ __device__ __forceinline__ float d_logf(float x)
     return fe * 0.693359375f + (lnm + fe * -2.12194440e-4f);
 }
 
-// 2^t for t in [-126, 1): n = rint(t), r = t - n, degree-5 polynomial of 2^r on [-1/2, 1/2] (relative error 2.7e-7)
+// 2^t for t in [-126, 1): n = rint(t), r = t - n, degree-5 polynomial of 2^r on [-1/2, 1/2] (relative error 2.7e-7).
+// rint is taken by adding and subtracting 1.5 * 2^23 (exact for |t| < 2^22, ties to even like rint), which also leaves
+// n in the low bits of the sum for the exponent: two full-rate additions instead of v_rndne_f32 and v_cvt_i32_f32.
 __device__ __forceinline__ float d_exp2(float t)
 {
-    const float n = __builtin_rintf(t);
+    const float shifted = t + 12582912.0f;
+    const float n = shifted - 12582912.0f;
     const float r = t - n;
     float p = 1.3381302124e-3f;
     p = __builtin_fmaf(p, r, 9.6663683653e-3f);
@@ -83,8 +86,7 @@ __device__ __forceinline__ float d_exp2(float t)
     p = __builtin_fmaf(p, r, 2.4022349715e-1f);
     p = __builtin_fmaf(p, r, 6.9314718246e-1f);
     p = __builtin_fmaf(p, r, 1.0f);
-    const int ni = (int)n;
-    return bits_to_float((uint32_t)((int)float_to_bits(p) + ni * 8388608));
+    return bits_to_float(float_to_bits(p) + (float_to_bits(shifted) << 23));
 }
 
 // 1 / x.  v_rcp_f32 followed by one fused Newton step is the correctly rounded quotient for every x with
