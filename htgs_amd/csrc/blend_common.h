@@ -106,11 +106,9 @@ __device__ __forceinline__ bool tile_misses(const float (&n)[6], const float (&d
         const float c = __builtin_fmaf(y, __builtin_fmaf(q[5], y, q[2]), q[0]);
         float xv = __builtin_rintf(__builtin_fmaf(b, to_vertex, 0.5f)) - 0.5f;
         xv = __builtin_fminf(__builtin_fmaxf(xv, -h), h);
-        const float xe = b > 0.0f ? -h : h;
-        const float x = convex ? xv : xe;
-        least = __builtin_fminf(least, __builtin_fmaf(x, __builtin_fmaf(q[3], x, b), c));
+        least = __builtin_fminf(least, __builtin_fmaf(xv, __builtin_fmaf(q[3], xv, b), c));
     }
-    return least > margin;
+    return convex && least > margin;                 // (a quadratic that is not convex along the rows is never left out)
 }
 
 // Stages instance `fetch` of the sorted list in slot `slot` (the same arithmetic as tile_geometry / tile_quadratics,
