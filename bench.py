@@ -23,7 +23,8 @@ sys.path.insert(0, ROOT)
 
 MODE_NAMES = {0: "HYBRID_BLEND", 1: "ALPHA_BLEND_FIRST_K", 2: "ALPHA_BLEND_GLOBAL_ORDERING", 3: "OIT_BLEND"}
 HBM_PEAK_GBS = 8000.0
-# fp32 vector peak as published (157.3 TFLOP/s counts packed FP32; plain FMA issue is half of it)
+# fp32 vector peak as published: 1024 SIMDs x 32 lanes x 2 flops x 2.4 GHz, i.e. one wave64 v_fma_f32 per two cycles
+# and SIMD (measured: 2.2-2.5 cycles)
 FP32_PEAK_TFLOPS = 157.3
 # flops of the mandatory part of one pixel/instance evaluation as the reference states it (the two planes, m, d,
 # |m|^2, |d|^2, cut-off test: R/include/hybrid_blend/kernels/inference.cuh:137-147).  The kernels reach the same
@@ -31,10 +32,10 @@ FP32_PEAK_TFLOPS = 157.3
 FLOPS_PER_EVAL = 46
 # HBM bytes of one blend launch of the default workload: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
 # same counters on a plain 1 GiB copy (fetch x 2.000, write x 1.000); profiles/inference_cfg2_3M_1080p_hybrid_k16.md
-MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3205669118}
-# VALUBusy of the blend kernel by the profiler's formula, SQ_ACTIVE_INST_VALU x 4 / (SIMDs x kernel cycles), capped at 1
-# (same profile; indicative, not a calibrated share of time)
-MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 1.0}
+MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3000585476}
+# share of the blend dispatch's SIMD-cycles (GRBM_GUI_ACTIVE) that the loop's instruction mix accounts for when priced
+# with the issue costs of single instructions measured on this device (same profile): 220 of 256 cycles per loop turn
+MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 0.86}
 
 
 def parse_args():
@@ -47,6 +48,8 @@ def parse_args():
     ap.add_argument("--mode", type=int, default=0)
     ap.add_argument("--K", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--issue-cost", action="store_true",
+                    help="measure how many cycles single vector instructions hold a SIMD (library's own micro-kernels) and exit")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 1 GiB copy kernel a few times (reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--train", action="store_true", help="time diff_rasterize forward + backward instead of rasterize")
@@ -134,6 +137,27 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.issue_cost:
+        # how long one wave64 vector instruction holds its SIMD: 32768 waves (eight resident per SIMD) x 500 turns x 64 copies
+        from htgs_amd import _native
+        lib, stream = _native.lib(), torch.cuda.current_stream(dev).cuda_stream
+        n_blocks, turns, clock_ghz = 8192, 500, 2.4
+        out = torch.empty(n_blocks * 256, dtype=torch.float32, device=dev)
+        table, i = {}, 0
+        while lib.htgs_issue_cost_name(i) is not None:
+            for _ in range(10):
+                _native.check(lib.htgs_issue_cost_launch(i, out.data_ptr(), n_blocks, turns, stream))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                _native.check(lib.htgs_issue_cost_launch(i, out.data_ptr(), n_blocks, turns, stream))
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / 10
+            table[lib.htgs_issue_cost_name(i).decode()] = round(ms * 1e-3 * clock_ghz * 1e9 * 1024 / (n_blocks * 4 * turns * 64), 2)
+            i += 1
+        print(json.dumps({"issue_cost": "cycles per wave64 instruction and SIMD at 2.4 GHz", "instructions": table}))
+        return
     if args.calibrate:
         from htgs_amd import _native
         n_bytes = 1 << 30                      # larger than the 256 MB memory-side cache: both streams come from HBM
