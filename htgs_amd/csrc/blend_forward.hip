@@ -17,7 +17,7 @@ __device__ __forceinline__ float one_minus_alpha_rcp(float one_minus_alpha)
 }
 
 template <int K>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 4 : 3))) blend_hybrid_forward_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_forward_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, uint32_t *__restrict__ core_idx, float4 *__restrict__ core_info, float *__restrict__ tail_info,
     uint32_t width, uint32_t height, uint32_t grid_w)
