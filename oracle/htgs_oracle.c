@@ -142,10 +142,14 @@ O_EXPORT float o_expf(float x)
 
 /* 2^t for t in [-126, 1): n = rint(t), r = t - n (exact), degree-5 polynomial of 2^r on [-1/2, 1/2]
  * (interpolated at Chebyshev nodes, relative error 2.7e-7), scaled by 2^n through the exponent field.
+ * rint(t) is taken as (t + 1.5 * 2^23) - 1.5 * 2^23 (equal to rintf for |t| < 2^22, ties to even), and the low bits of
+ * the sum are n for the exponent field: the arithmetic of the HIP routine, operation for operation, so that the
+ * two agree on every input, in range or not.
  * pinned by: tests compare with 2.0**t in float64 on [-20, 0.5] (<= 3e-7 relative). */
 O_EXPORT float o_exp2(float t)
 {
-    const float n = rintf(t);
+    const float shifted = t + 12582912.0f;
+    const float n = shifted - 12582912.0f;
     const float r = t - n;
     float p = 1.3381302124e-3f;
     p = fmaf(p, r, 9.6663683653e-3f);
@@ -153,8 +157,7 @@ O_EXPORT float o_exp2(float t)
     p = fmaf(p, r, 2.4022349715e-1f);
     p = fmaf(p, r, 6.9314718246e-1f);
     p = fmaf(p, r, 1.0f);
-    const int32_t ni = (int32_t)n;
-    return bits_to_float((uint32_t)((int32_t)float_to_bits(p) + ni * 8388608));
+    return bits_to_float(float_to_bits(p) + (float_to_bits(shifted) << 23));
 }
 
 static inline float clamp_pos(float v) { return v > 0.0f ? v : 0.0f; }              /* fmaxf(v, 0) with NaN -> 0 */
