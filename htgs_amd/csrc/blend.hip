@@ -73,18 +73,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 tail2 = __builtin_fmaf(p3, col.z, tail2);
                 if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
                     float pi = col.w;
-#pragma unroll
-                    for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
-                        if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
-#pragma unroll
-                        for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
-                            if (depth < cd[i]) {
-                                vswap(depth, cd[i]);
-                                vswap(p3, ca[i]);
-                                vswap(pi, ci[i]);
-                            }
-                        }
-                    }
+                    core_exchange_walk<K>(depth, p3, pi, cd, ca, ci);
                 }
                 // (depth, p3) is the fragment itself, the entry it pushed out of the core, or an empty slot (alpha 0)
                 tail3 += p3;
@@ -172,18 +161,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
                 float alpha = f.alpha;
                 uint32_t idx = stage_index<64>(addr);
-#pragma unroll
-                for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
-                    if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
-#pragma unroll
-                    for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
-                        if (depth < cd[i]) {
-                            vswap(depth, cd[i]);
-                            vswap(alpha, ca[i]);
-                            vswap(idx, ci[i]);
-                        }
-                    }
-                }
+                core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
             }
         }
     }

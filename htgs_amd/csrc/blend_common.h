@@ -263,22 +263,37 @@ __device__ __forceinline__ bool tile_frag_alpha(float opacity, TileFrag &o)
     return !(o.alpha < ModeCfg<MODE>::min_alpha);
 }
 
-// exchange two VGPRs in the active lanes: three moves through a scratch register (a wave64 v_mov_b32 holds the
-// vector ALU for two cycles, v_swap_b32 for eight, v_cndmask_b32 for four)
-__device__ __forceinline__ void vswap(float &a, float &b)
-{
-    float t;
-    asm volatile("v_mov_b32 %2, %0\n\tv_mov_b32 %0, %1\n\tv_mov_b32 %1, %2" : "+v"(a), "+v"(b), "=&v"(t));
-}
-__device__ __forceinline__ void vswap(uint32_t &a, uint32_t &b)
-{
-    uint32_t t;
-    asm volatile("v_mov_b32 %2, %0\n\tv_mov_b32 %0, %1\n\tv_mov_b32 %1, %2" : "+v"(a), "+v"(b), "=&v"(t));
-}
-
-// Sorted insertion into a K-slot buffer walks the slots front to back carrying the displaced entry; the kernels
-// take the slots four at a time and the whole wave skips a group that no active lane can change (the carried
-// depth is not below the group's last slot).
+// Sorted insertion into a K-slot buffer (depth, alpha, index per slot) walks the slots front to back carrying the
+// displaced entry (the reference's exchange walk); the slots are taken four at a time and the whole wave skips a group
+// that no active lane can change (the carried depth is not below the group's last slot).  One slot: v_cmpx narrows
+// exec to the lanes whose carried depth is below the slot's, three moves through a scratch register exchange each
+// of the three registers (a wave64 v_mov_b32 holds the vector ALU for two cycles, v_swap_b32 for eight,
+// v_cndmask_b32 for four), and exec is restored.  On return (depth, alpha, index) is what the walk pushed out.
 constexpr int kInsertGroup = 4;
+template <typename IndexT>
+__device__ __forceinline__ void exchange_step(float &D, float &A, IndexT &I, float &d, float &a, IndexT &x, uint64_t all)
+{
+    static_assert(sizeof(IndexT) == 4, "one register");
+    float t;
+    asm volatile("v_cmpx_lt_f32 vcc, %[D], %[d]\n\t"
+                 "v_mov_b32 %[t], %[d]\n\tv_mov_b32 %[d], %[D]\n\tv_mov_b32 %[D], %[t]\n\t"
+                 "v_mov_b32 %[t], %[a]\n\tv_mov_b32 %[a], %[A]\n\tv_mov_b32 %[A], %[t]\n\t"
+                 "v_mov_b32 %[t], %[x]\n\tv_mov_b32 %[x], %[I]\n\tv_mov_b32 %[I], %[t]\n\t"
+                 "s_mov_b64 exec, %[all]"
+                 : [D] "+v"(D), [A] "+v"(A), [I] "+v"(I), [d] "+v"(d), [a] "+v"(a), [x] "+v"(x), [t] "=&v"(t)
+                 : [all] "s"(all)
+                 : "vcc");
+}
+template <int K, typename IndexT>
+__device__ __forceinline__ void core_exchange_walk(float &depth, float &alpha, IndexT &index, float (&cd)[K], float (&ca)[K], IndexT (&ci)[K])
+{
+    const uint64_t all = __ballot(true);               // the lanes that called
+#pragma unroll
+    for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
+        if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
+#pragma unroll
+        for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) exchange_step(depth, alpha, index, cd[i], ca[i], ci[i], all);
+    }
+}
 
 }  // namespace htgs

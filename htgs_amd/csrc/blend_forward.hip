@@ -60,18 +60,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             tail2 = __builtin_fmaf(p3, col.z, tail2);
             if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
                 uint32_t idx = stage_index<64>(addr);
-#pragma unroll
-                for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
-                    if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
-#pragma unroll
-                    for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
-                        if (depth < cd[i]) {
-                            vswap(depth, cd[i]);
-                            vswap(p3, c3[i]);
-                            vswap(idx, ci[i]);
-                        }
-                    }
-                }
+                core_exchange_walk<K>(depth, p3, idx, cd, c3, ci);
             }
             tail3 += p3;
             T_tail *= 1.0f - p3;
@@ -178,18 +167,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
             float alpha = f.alpha;
             uint32_t idx = stage_index<64>(addr);
-#pragma unroll
-            for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
-                if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
-#pragma unroll
-                for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) {
-                    if (depth < cd[i]) {
-                        vswap(depth, cd[i]);
-                        vswap(alpha, ca[i]);
-                        vswap(idx, ci[i]);
-                    }
-                }
-            }
+            core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
         }
     }
     if (!inside) return;

@@ -60,18 +60,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth<64>(addr, pt, f);
             if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
                 uint32_t idx = stage_index<64>(addr);
-#pragma unroll
-                for (int g0 = 0; g0 < KS; g0 += kInsertGroup) {
-                    if (KS > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < KS ? g0 + kInsertGroup - 1 : KS - 1])) continue;
-#pragma unroll
-                    for (int i = g0; i < g0 + kInsertGroup && i < KS; ++i) {
-                        if (depth < cd[i]) {
-                            vswap(depth, cd[i]);
-                            vswap(alpha, ca[i]);
-                            vswap(idx, ci[i]);
-                        }
-                    }
-                }
+                core_exchange_walk<KS>(depth, alpha, idx, cd, ca, ci);
             }
             if (kTail) { alpha_sum += alpha; T_tail *= 1.0f - alpha; }
         }
