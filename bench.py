@@ -32,7 +32,7 @@ FP32_PEAK_TFLOPS = 157.3
 FLOPS_PER_EVAL = 46
 # HBM bytes of one blend launch of the default workload: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
 # same counters on a plain 1 GiB copy (fetch x 2.000, write x 1.000); profiles/inference_cfg2_3M_1080p_hybrid_k16.md
-MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3000585476}
+MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3076682530}
 # share of the blend dispatch's SIMD-cycles (GRBM_GUI_ACTIVE) that the loop's instruction mix accounts for when priced
 # with the issue costs of single instructions measured on this device (same profile): 220 of 256 cycles per loop turn
 MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 0.86}
