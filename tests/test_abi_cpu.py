@@ -86,6 +86,26 @@ def test_entry_points_reject_bad_frames_without_touching_the_gpu():
     assert lib.htgs_preprocess(ctypes.byref(f)) == 2
 
 
+def test_measurement_and_self_check_entry_points_reject_bad_arguments():
+    lib = _native.lib()
+    names = []
+    while lib.htgs_issue_cost_name(len(names)) is not None:
+        names.append(lib.htgs_issue_cost_name(len(names)).decode())
+    assert names[0] == "v_fma_f32" and "v_mov_b32" in names and "v_swap_b32" in names and len(set(names)) == len(names)
+    assert lib.htgs_issue_cost_name(-1) is None
+    assert lib.htgs_issue_cost_launch(len(names), None, 1, 1, None) == 2          # no such instruction (and no buffer)
+    assert lib.htgs_issue_cost_launch(0, None, 1, 1, None) == 2
+    f = _native.Frame()
+    f.mode = 2
+    f.width = f.height = 64
+    assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, None) == 2
+    counts = (ctypes.c_ulonglong * 4)()
+    assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, counts) == 1               # the 16x16-tile mode does not cull
+    assert b"does not cull" in lib.htgs_last_error()
+    assert lib.htgs_check_reciprocal(None, None) == 2
+    assert lib.htgs_copy_bytes(None, None, 16, None) == 2
+
+
 def test_python_api_surface_and_validation():
     import HTGSCudaBackend.torch_bindings as alias
     import htgs_amd

@@ -91,6 +91,22 @@ def test_refined_reciprocal_equals_division_on_the_whole_guarded_range(cuda):
     assert wrong == 0
 
 
+def test_issue_cost_micro_kernels_run(cuda):
+    """The measurement aid behind ``bench.py --issue-cost``: every micro-kernel launches and fills its output."""
+    from htgs_amd import _native
+    lib = _native.lib()
+    marker = 0x7FC12345                                   # a NaN pattern no kernel produces
+    out = torch.empty(4 * 256, dtype=torch.int32, device=cuda)
+    i = 0
+    while lib.htgs_issue_cost_name(i) is not None:
+        out.fill_(marker)
+        _native.check(lib.htgs_issue_cost_launch(i, out.data_ptr(), 4, 2, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert not bool((out == marker).any()), lib.htgs_issue_cost_name(i)
+        i += 1
+    assert i >= 10
+
+
 def test_fast_rasterize_agrees_with_rasterize_to_rounding(cuda):
     """The image-only fast path uses the hardware's reciprocal and 2^x (one ulp each): the image is the exact one to
     rounding, except where a fragment sits within an ulp of an alpha threshold (1/255: worth 4e-3 of a colour; 1/20, the
