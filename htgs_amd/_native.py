@@ -85,6 +85,8 @@ SYMBOLS = {
     "htgs_sort_tmp_words": (ctypes.c_size_t, [ctypes.c_uint64]),
     "htgs_preprocess": (ctypes.c_int, [_FRAME_P]),
     "htgs_scan_offsets": (ctypes.c_int, [_FRAME_P]),
+    "htgs_scan_offsets_static": (ctypes.c_int, [_FRAME_P]),
+    "htgs_scan_static_max_primitives": (ctypes.c_int, []),
     "htgs_create_instances": (ctypes.c_int, [_FRAME_P]),
     "htgs_sort_instances": (ctypes.c_int, [_FRAME_P, ctypes.POINTER(ctypes.c_int)]),
     "htgs_extract_ranges": (ctypes.c_int, [_FRAME_P, ctypes.c_int]),
