@@ -49,7 +49,7 @@ def parse_args():
     ap.add_argument("--K", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--issue-cost", action="store_true",
-                    help="measure how many cycles single vector instructions hold a SIMD (library's own micro-kernels) and exit")
+                    help="measure how many cycles single vector instructions hold a SIMD (micro-kernels of the separate probe library) and exit")
     ap.add_argument("--calibrate", action="store_true",
                     help="only run the plain 1 GiB copy kernel a few times (reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--train", action="store_true", help="time diff_rasterize forward + backward instead of rasterize")
@@ -139,34 +139,34 @@ def main():
     torch.cuda.set_device(dev)
     if args.issue_cost:
         # how long one wave64 vector instruction holds its SIMD: 32768 waves (eight resident per SIMD) x 500 turns x 64 copies
-        from htgs_amd import _native
-        lib, stream = _native.lib(), torch.cuda.current_stream(dev).cuda_stream
+        from htgs_amd import diagnostics
+        lib, stream = diagnostics.lib(), torch.cuda.current_stream(dev).cuda_stream
         n_blocks, turns, clock_ghz = 8192, 500, 2.4
         out = torch.empty(n_blocks * 256, dtype=torch.float32, device=dev)
         table, i = {}, 0
-        while lib.htgs_issue_cost_name(i) is not None:
+        while lib.htgs_probe_issue_cost_name(i) is not None:
             for _ in range(10):
-                _native.check(lib.htgs_issue_cost_launch(i, out.data_ptr(), n_blocks, turns, stream))
+                assert lib.htgs_probe_issue_cost_launch(i, out.data_ptr(), n_blocks, turns, stream) == 0
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(10):
-                _native.check(lib.htgs_issue_cost_launch(i, out.data_ptr(), n_blocks, turns, stream))
+                assert lib.htgs_probe_issue_cost_launch(i, out.data_ptr(), n_blocks, turns, stream) == 0
             e1.record()
             torch.cuda.synchronize()
             ms = e0.elapsed_time(e1) / 10
-            table[lib.htgs_issue_cost_name(i).decode()] = round(ms * 1e-3 * clock_ghz * 1e9 * 1024 / (n_blocks * 4 * turns * 64), 2)
+            table[lib.htgs_probe_issue_cost_name(i).decode()] = round(ms * 1e-3 * clock_ghz * 1e9 * 1024 / (n_blocks * 4 * turns * 64), 2)
             i += 1
         print(json.dumps({"issue_cost": "cycles per wave64 instruction and SIMD at 2.4 GHz", "instructions": table}))
         return
     if args.calibrate:
-        from htgs_amd import _native
+        from htgs_amd import diagnostics
         n_bytes = 1 << 30                      # larger than the 256 MB memory-side cache: both streams come from HBM
         src = torch.empty(n_bytes // 4, dtype=torch.float32, device=dev).fill_(1.0)
         dst = torch.empty_like(src)
         for _ in range(5):
-            _native.check(_native.lib().htgs_copy_bytes(dst.data_ptr(), src.data_ptr(), n_bytes, torch.cuda.current_stream(dev).cuda_stream))
+            assert diagnostics.lib().htgs_probe_copy_bytes(dst.data_ptr(), src.data_ptr(), n_bytes, torch.cuda.current_stream(dev).cuda_stream) == 0
         torch.cuda.synchronize()
-        print(json.dumps({"calibration": "copy_bytes_kernel", "bytes_read": n_bytes, "bytes_written": n_bytes, "launches": 5}))
+        print(json.dumps({"calibration": "copy_bytes_kernel (libhtgs_probes.so)", "bytes_read": n_bytes, "bytes_written": n_bytes, "launches": 5}))
         return
     scene_cpu = make_scene(args.config, args.n)
     scene = scene_cpu.to(dev)

@@ -107,9 +107,6 @@ SYMBOLS = {
                                              ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_void_p]),
     "htgs_check_reciprocal": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p]),
     "htgs_check_tile_cull": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]),
-    "htgs_copy_bytes": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
-    "htgs_issue_cost_name": (ctypes.c_char_p, [ctypes.c_int]),
-    "htgs_issue_cost_launch": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
 }
 
 _lib = None

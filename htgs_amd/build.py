@@ -1,6 +1,7 @@
-"""Builds ``libhtgs_amd.so`` (gfx950 only) from ``csrc/*.hip`` with hipcc.
+"""Builds ``libhtgs_amd.so`` (gfx950 only) from ``csrc/*.hip`` with hipcc, and the separate measurement-probe library
+``diagnostics/libhtgs_probes.so`` from ``diagnostics/probes.hip``.
 
-The library is built in-tree next to this file.  ``python -m htgs_amd.build`` rebuilds it.
+Both are built in-tree.  ``python -m htgs_amd.build`` rebuilds them.
 """
 from __future__ import annotations
 
@@ -13,6 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libhtgs_amd.so")
 OBJ_DIR = os.path.join(HERE, "build")
+PROBES_SRC = os.path.join(HERE, "diagnostics", "probes.hip")
+PROBES_LIB_PATH = os.path.join(HERE, "diagnostics", "libhtgs_probes.so")
 
 # -ffp-contract=off: a fused multiply-add exists only where the sources write __builtin_fmaf, which is what
 #   makes tile counts and accept/reject decisions reproducible (see csrc/common.h).
@@ -59,11 +62,14 @@ def build(verbose: bool = False) -> str:
             print(" ".join(cmd))
         _run(cmd)
 
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
-        list(pool.map(compile_one, zip(srcs, objs)))
-    tmp = LIB_PATH + ".tmp"
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wno-unused-command-line-argument", *objs, "-o", tmp])
-    os.replace(tmp, LIB_PATH)
+    probes_obj = os.path.join(OBJ_DIR, "probes.o")
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs) + 1)) as pool:
+        list(pool.map(compile_one, [*zip(srcs, objs), (PROBES_SRC, probes_obj)]))
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wno-unused-command-line-argument"]
+    for lib_objs, path in ((objs, LIB_PATH), ([probes_obj], PROBES_LIB_PATH)):
+        tmp = path + ".tmp"
+        _run([*link, *lib_objs, "-o", tmp])
+        os.replace(tmp, path)
     return LIB_PATH
 
 

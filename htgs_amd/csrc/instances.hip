@@ -56,11 +56,15 @@ __global__ void __launch_bounds__(kScanBlock) scan_reduce_kernel(const uint32_t 
     if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 
-// pass 2: one block turns the tile sums into exclusive tile offsets and publishes the grand total
+// pass 2: one block turns the tile sums into exclusive tile offsets and publishes the grand total.  Offsets are
+// 32-bit as in the reference; a frame whose counts add up to more than 2^32 - 2 publishes 0xffffffff, which no valid
+// frame produces, so that the host can refuse it instead of sizing its buffers from a wrapped sum.
 __global__ void __launch_bounds__(kScanBlock) scan_tiles_kernel(uint32_t *__restrict__ tile_sums, int n_tiles, uint32_t *__restrict__ total_out)
 {
     __shared__ uint32_t wave_sums[kScanBlock / kWave];
+    __shared__ unsigned long long s_wide[kScanBlock];
     uint32_t carry = 0;
+    unsigned long long wide = 0;             // this thread's share of the same sum without wrap-around
     for (int start = 0; start < n_tiles; start += kScanBlock) {
         const int i = start + threadIdx.x;
         const uint32_t v = i < n_tiles ? tile_sums[i] : 0u;
@@ -68,8 +72,15 @@ __global__ void __launch_bounds__(kScanBlock) scan_tiles_kernel(uint32_t *__rest
         const uint32_t inc = block_inclusive_scan(v, wave_sums, &total);
         if (i < n_tiles) tile_sums[i] = carry + inc - v;
         carry += total;
+        wide += v;
     }
-    if (threadIdx.x == 0) *total_out = carry;
+    s_wide[threadIdx.x] = wide;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long sum = 0;
+        for (int t = 0; t < kScanBlock; ++t) sum += s_wide[t];
+        *total_out = sum > 0xfffffffeull ? 0xffffffffu : carry;
+    }
 }
 
 // pass 3: scan inside each tile, add the tile offset.  Thread t owns items [t*8, t*8+8) of the tile.
@@ -234,6 +245,9 @@ static int launch_scan(const htgs_frame *f, uint32_t *tile_sums, const char *who
 {
     hipStream_t s = (hipStream_t)f->stream;
     const int n = f->n_primitives;
+    // a block's 2048 counts, each at most the number of tiles, must fit 32 bits for the overflow check of the total
+    if (f->width > 0 && f->height > 0 && (uint64_t)div_up(f->width, 8) * (uint64_t)div_up(f->height, 8) > (1ull << 20))
+        return fail(HTGS_ERR_ARGUMENT, "%s: more than 2^20 tiles (images beyond 8192 x 8192 pixels are not supported)", who);
     const int tiles = n > 0 ? div_up(n, kScanTile) : 0;
     if (n > 0 && (!f->n_touched || !f->offsets)) return fail(HTGS_ERR_ARGUMENT, "%s: null pointer", who);
     if (tiles > 0) hipLaunchKernelGGL(scan_reduce_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, n);
@@ -280,7 +294,7 @@ extern "C" int htgs_create_instances(const htgs_frame *f)
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_create_instances: null frame");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (f->n_primitives <= 0 || f->n_instances == 0) return HTGS_OK;
-    if (f->n_instances > 0xffffffffull) return fail(HTGS_ERR_ARGUMENT, "htgs_create_instances: more than 2^32-1 instances");
+    if (f->n_instances > 0xfffffffeull) return fail(HTGS_ERR_ARGUMENT, "htgs_create_instances: more than 2^32-2 instances");
     if (!f->n_touched || !f->offsets || !f->bounds || !f->prim || !f->keys[0] || !f->vals[0])
         return fail(HTGS_ERR_ARGUMENT, "htgs_create_instances: null pointer");
     hipStream_t s = (hipStream_t)f->stream;

@@ -272,7 +272,7 @@ extern "C" int htgs_sort_instances(const htgs_frame *f, int *selector)
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     *selector = 0;
     if (f->n_instances == 0) return HTGS_OK;
-    if (f->n_instances > 0xffffffffull) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: more than 2^32-1 instances");
+    if (f->n_instances > 0xfffffffeull) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: more than 2^32-2 instances");
     if (!f->keys[0] || !f->keys[1] || !f->vals[0] || !f->vals[1] || !f->sort_tmp)
         return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: null pointer");
     if (((uintptr_t)f->keys[0] | (uintptr_t)f->keys[1]) & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: keys must be 16-byte aligned");

@@ -17,6 +17,9 @@ import torch
 from .torch_bindings.rasterization import RasterizerMode, RasterizerSettings
 
 SH_C0 = 0.28209479177387814
+# focal length (pixels) of the 6 M stress scene: the value at which a visible Gaussian of that scene covers 16 tiles of
+# 8x8 pixels on average (the scene is specified by its distributions and by 8-20 tiles per Gaussian, not by a focal length)
+CFG3_FOCAL = 35.0
 
 
 @dataclass
@@ -130,14 +133,13 @@ def make_scene(config: int, n: Optional[int] = None) -> Scene:
         xy_near = (torch.rand(n, 2, generator=g) * 2.0 - 1.0) * 0.5
         pos[near, 2] = z_near[near]
         pos[near, :2] = xy_near[near]
+        # log-scales ~ N(-3, 0.8) for every Gaussian, the near-plane group included: those are the ellipsoids that
+        # cross the near plane, reach NDC z < -1 or cover the whole tile grid
         scales = torch.exp(torch.randn(n, 3, generator=g) * 0.8 - 3.0)
-        # the near group keeps the projected size of a Gaussian at the cluster centre (4 units): without this a
-        # single near Gaussian covers thousands of tiles and the scene leaves the stated 8-20 tiles per Gaussian
-        scales[near] *= (pos[near, 2:3] / 4.0)
         rot = _unit_quaternions(n, g)
         opac = torch.sigmoid(torch.randn(n, 1, generator=g) * 1.5)
         sh_0, sh_rest = _sh(n, 3, g)
-        M, VPM, cam = pinhole(1600, 1066, 100.0, 100.0, 800.0, 533.0, 0.2, 1000.0)
+        M, VPM, cam = pinhole(1600, 1066, CFG3_FOCAL, CFG3_FOCAL, 800.0, 533.0, 0.2, 1000.0)
         return Scene("cfg3-6M-stress", pos.contiguous(), scales, rot, opac, sh_0, sh_rest, M, VPM, cam, 1600, 1066, 0.2, 1000.0, 16, 16)
     if config == 4:
         return _cluster_scene("cfg4-1M-1080p-train", 4, n or 1_000_000, 1920, 1080, 1500.0, 16)

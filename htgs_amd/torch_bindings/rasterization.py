@@ -8,6 +8,7 @@ torch only owns the device memory and the stream, every kernel is hand-written H
 from __future__ import annotations
 
 import ctypes
+import threading
 from enum import Enum
 from typing import NamedTuple, Optional
 
@@ -61,28 +62,44 @@ def _ptr(t: Optional[torch.Tensor]) -> int:
     return 0 if t is None or t.numel() == 0 else t.data_ptr()
 
 
+MAX_INSTANCES = 0xfffffffe
+
+
+def checked_instance_count(published: int) -> int:
+    """The instance count the scan published.  Offsets into the instance list are 32-bit, as in the reference
+    (R/include/hybrid_blend/buffer_utils.h:22-54); the scan publishes 0xffffffff for a frame whose tile counts add up
+    to more than ``MAX_INSTANCES``, and such a frame is refused instead of being rendered from wrapped offsets."""
+    if published < 0 or published > MAX_INSTANCES:
+        raise RuntimeError(f"the frame needs more than {MAX_INSTANCES} (tile, Gaussian) instances; offsets are 32-bit -- "
+                           "render fewer Gaussians per call or a smaller image")
+    return published
+
+
 class ScratchPool:
-    """Grow-only device scratch that inference frames on one (device, stream) reuse, so that a steady stream of
-    ``rasterize`` calls allocates nothing but its outputs.  Work is ordered by the stream, which is what makes the
-    reuse safe; frames issued on another stream get another pool.  Training frames do not use it (their scratch
-    has to survive until backward)."""
+    """Grow-only device scratch that inference frames on one (device, stream, host thread) reuse, so that a steady
+    stream of ``rasterize`` calls allocates nothing but its outputs.  A frame is issued front to back by one thread and
+    ordered by the stream, which is what makes the reuse safe; frames issued on another stream or by another thread
+    get another pool.  Training frames do not use it (their scratch has to survive until backward)."""
 
     _pools: dict = {}
+    _lock = threading.Lock()
 
     def __init__(self):
         self.buffers: dict = {}
 
     @classmethod
     def current(cls, device: torch.device) -> "ScratchPool":
-        key = (device.index, torch.cuda.current_stream(device).cuda_stream)
-        pool = cls._pools.get(key)
-        if pool is None:
-            pool = cls._pools[key] = ScratchPool()
+        key = (device.index, torch.cuda.current_stream(device).cuda_stream, threading.get_ident())
+        with cls._lock:
+            pool = cls._pools.get(key)
+            if pool is None:
+                pool = cls._pools[key] = ScratchPool()
         return pool
 
     @classmethod
     def clear(cls):
-        cls._pools.clear()
+        with cls._lock:
+            cls._pools.clear()
 
     def get(self, name: str, numel: int, dtype: torch.dtype, device: torch.device, headroom: float = 0.0) -> torch.Tensor:
         buf = self.buffers.get(name)
@@ -198,7 +215,7 @@ class FrameBuffers:
     def read_instance_count(self) -> int:
         """The frame's only host/device synchronisation (the reference's cudaMemcpy at
         R/src/hybrid_blend/inference.cu:118-119)."""
-        return int(self.n_instances_dev.item()) & 0xffffffff if self.n > 0 else 0
+        return checked_instance_count(int(self.n_instances_dev.item()) & 0xffffffff) if self.n > 0 else 0
 
     def alloc_instances(self, n_instances: int):
         dev = self.device
@@ -311,7 +328,8 @@ class FrameBuffers:
 
 class _Rasterize(torch.autograd.Function):
     """Differentiable render (reference: rasterization.py:45-113).  The frame object saved on ``ctx`` owns the
-    scratch that the reference returns to Python as four byte blobs."""
+    scratch that the reference returns to Python as four byte blobs and keeps in ``ctx.save_for_backward``
+    (:71-82); like those it lives as long as ``ctx``, so ``backward(retain_graph=True)`` can run again."""
 
     @staticmethod
     def forward(ctx, positions, scales, rotations, opacities, sh_0, sh_rest, densification_info, rasterizer_settings,
@@ -330,7 +348,6 @@ class _Rasterize(torch.autograd.Function):
     def backward(ctx, grad_image):
         _ = ctx.saved_tensors      # raises if an input was modified in place since forward
         grads = ctx.fb.run_backward(grad_image, ctx.densification_info, ctx.use_distance_scaling)
-        ctx.fb = None
         return (*grads, None, None, None)
 
 

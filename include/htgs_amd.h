@@ -200,18 +200,6 @@ int htgs_check_reciprocal(unsigned long long *counts, void *stream);
  * caller): instances looked at, instances that reach no pixel, instances left out, instances left out wrongly (0). */
 int htgs_check_tile_cull(const htgs_frame *f, int selector, unsigned long long *counts);
 
-/* Measurement aid, no counterpart in the reference: how long one vector instruction holds a SIMD.  Launch number
- * `instruction` (0 .. until htgs_issue_cost_name returns NULL) runs n_blocks workgroups of four waves, each wave
- * `turns` loop turns of 64 copies of that instruction; out receives n_blocks * 256 floats.  Timed by the caller
- * (bench.py --issue-cost): cycles per instruction and SIMD = time * clock * 1024 SIMDs / (n_blocks * 4 * turns * 64). */
-const char *htgs_issue_cost_name(int instruction);
-int htgs_issue_cost_launch(int instruction, float *out, int n_blocks, int turns, void *stream);
-
-/* Measurement aid, no counterpart in the reference: a plain device-to-device copy of n_bytes (multiple of 16)
- * with one 16-byte load and store per thread.  Hardware counters read on it calibrate the same counters read on
- * the rasterizer's kernels (bench.py --calibrate). */
-int htgs_copy_bytes(void *dst, const void *src, size_t n_bytes, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

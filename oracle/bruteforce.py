@@ -282,3 +282,24 @@ def max_weights(fr: Fragments, mode: int, K: int, weight_threshold: float):
             W = torch.maximum(W, alpha * tail_weight[:, None] * inside_cutoff)
     raw = W.max(dim=0).values
     return torch.where(raw >= weight_threshold, raw, torch.zeros_like(raw)), raw
+
+
+def per_fragment_position_gradient_l1(positions, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam_position, mode: int,
+                                      active_sh_bases: int, width: int, height: int, near_plane: float, far_plane: float,
+                                      K: int, grad_image: torch.Tensor) -> torch.Tensor:
+    """Third densification statistic by its definition (R/include/hybrid_blend/kernels/backward.cuh:292-306): for every
+    Gaussian g the sum over pixels p of  | d L_p / d position_g |_1 , where L_p = sum_c grad_image[c,p] image[c,p] is the
+    loss carried by pixel p alone and the derivative is the geometric one (through the fragment's alpha; the colour's
+    view dependence is added elsewhere and is not part of it).  One autograd pass per pixel through the float64
+    evaluator; nothing of the reference's hand-derived chain is used.  Returns [G] (no distance scaling)."""
+    pos = positions.to(F64).clone().requires_grad_(True)
+    fr = evaluate(pos, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam_position, mode, active_sh_bases, width, height,
+                  near_plane, far_plane)
+    fr.rgb = fr.rgb.detach()
+    image, _, _, _ = render(fr, mode, K, False, clamp=False)
+    per_pixel = (image * grad_image.to(F64)).sum(0).reshape(-1)            # L_p, [P]
+    out = torch.zeros(pos.shape[0], dtype=F64)
+    for p in torch.nonzero(per_pixel.detach() != 0).reshape(-1).tolist():
+        (g,) = torch.autograd.grad(per_pixel[p], pos, retain_graph=True)
+        out += g.abs().sum(1)
+    return out

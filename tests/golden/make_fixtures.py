@@ -1,8 +1,9 @@
 """Writes tests/golden/small_scene.npz: known answers for a 140-Gaussian scene, from the independent float64
 evaluator (oracle/bruteforce.py: textbook ray / Gaussian maximum, dense compositing by the definition of each blend
 mode, gradients by torch.autograd).  The fixture holds the inputs, and per blend mode the image, the depth, the
-pixels whose accept / reject decisions are not within 1e-4 of a threshold (only those are compared), and the six
-gradients of sum(image * grad_image) over those pixels.
+pixels whose accept / reject decisions are not within 1e-4 of a threshold (only those are compared), the six
+gradients of sum(image * grad_image) over those pixels, and the third densification statistic (per Gaussian, the sum
+over those pixels of the 1-norm of the pixel's own position gradient).
 
 The reference ships no test vectors; these are this repository's own, frozen so that a change of the CPU checker and
 of the kernels in the same direction still has something to answer to.  Run from the repository root:
@@ -45,6 +46,10 @@ def main():
         out[f"mask_{mode}"] = mask.numpy()
         for name, leaf in zip(NAMES, leaves):
             out[f"grad_{name}_{mode}"] = leaf.grad.numpy().astype(np.float32)
+        # third densification statistic (sum over pixels of |dL_p / dposition|_1), same upstream gradient and mask
+        out[f"dens_l1_{mode}"] = bf.per_fragment_position_gradient_l1(
+            *sc.gaussians(), sc.M, sc.VPM, sc.cam_position, mode, sc.active_sh_bases, sc.width, sc.height, sc.near_plane,
+            sc.far_plane, K, grad_image.double() * mask.double()).numpy().astype(np.float32)
         print(f"mode {mode}: {float(mask.double().mean()):.3f} of the pixels compared, image max {float(image.detach().max()):.3f}")
     np.savez_compressed(os.path.join(HERE, "small_scene.npz"), **out)
 

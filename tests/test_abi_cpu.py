@@ -19,8 +19,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "htgs_amd.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(htgs_[a-z0-9_]+)\s*\(", text)))
 
@@ -33,6 +33,26 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(handle, name), f"{name} is declared in include/htgs_amd.h but not exported"
     assert sorted(_native.SYMBOLS) == names, "htgs_amd/_native.py must bind exactly the declared entry points"
     _native.lib()
+
+
+def test_probe_library_is_separate_and_exports_its_header():
+    """The measurement probes live in their own library and header, not in the drop-in boundary."""
+    from htgs_amd import diagnostics
+    names = declared_functions(os.path.join(ROOT, "include", "htgs_probes.h"))
+    assert sorted(diagnostics.SYMBOLS) == names and len(names) == 3
+    product = ctypes.CDLL(_native.LIB_PATH)
+    for name in names:
+        assert hasattr(diagnostics.lib(), name)
+        assert not hasattr(product, name)
+    lib = diagnostics.lib()
+    probes = []
+    while lib.htgs_probe_issue_cost_name(len(probes)) is not None:
+        probes.append(lib.htgs_probe_issue_cost_name(len(probes)).decode())
+    assert probes[0] == "v_fma_f32" and "v_mov_b32" in probes and "v_swap_b32" in probes and len(set(probes)) == len(probes)
+    assert lib.htgs_probe_issue_cost_name(-1) is None
+    assert lib.htgs_probe_issue_cost_launch(len(probes), None, 1, 1, None) == 2        # no such instruction (and no buffer)
+    assert lib.htgs_probe_issue_cost_launch(0, None, 1, 1, None) == 2
+    assert lib.htgs_probe_copy_bytes(None, None, 16, None) == 2
 
 
 def test_frame_struct_layout_matches_the_header(tmp_path):
@@ -86,15 +106,29 @@ def test_entry_points_reject_bad_frames_without_touching_the_gpu():
     assert lib.htgs_preprocess(ctypes.byref(f)) == 2
 
 
-def test_measurement_and_self_check_entry_points_reject_bad_arguments():
+def test_instance_counts_beyond_32_bit_offsets_are_refused():
+    """Offsets into the instance list are 32-bit, as in the reference; 0xffffffff is what the scan publishes when the
+    tile counts do not fit.  The host refuses it, and so do the entry points that take the count."""
+    from htgs_amd.torch_bindings.rasterization import MAX_INSTANCES, checked_instance_count
+    assert MAX_INSTANCES == 2 ** 32 - 2
+    assert checked_instance_count(0) == 0 and checked_instance_count(MAX_INSTANCES) == MAX_INSTANCES
+    for bad in (MAX_INSTANCES + 1, 2 ** 32, 2 ** 40, -1):
+        with pytest.raises(RuntimeError, match="instances"):
+            checked_instance_count(bad)
     lib = _native.lib()
-    names = []
-    while lib.htgs_issue_cost_name(len(names)) is not None:
-        names.append(lib.htgs_issue_cost_name(len(names)).decode())
-    assert names[0] == "v_fma_f32" and "v_mov_b32" in names and "v_swap_b32" in names and len(set(names)) == len(names)
-    assert lib.htgs_issue_cost_name(-1) is None
-    assert lib.htgs_issue_cost_launch(len(names), None, 1, 1, None) == 2          # no such instruction (and no buffer)
-    assert lib.htgs_issue_cost_launch(0, None, 1, 1, None) == 2
+    f = _native.Frame()
+    f.mode, f.width, f.height, f.n_primitives = 0, 1920, 1080, 1
+    sel = ctypes.c_int(0)
+    for n in (2 ** 32 - 1, 2 ** 32, 2 ** 33 + 5):
+        f.n_instances = n
+        assert lib.htgs_create_instances(ctypes.byref(f)) == 2 and b"2^32-2 instances" in lib.htgs_last_error()
+        assert lib.htgs_sort_instances(ctypes.byref(f), ctypes.byref(sel)) == 2 and b"2^32-2 instances" in lib.htgs_last_error()
+    f.n_instances = 2 ** 32 - 2              # allowed: the next complaint is about the (null) buffers
+    assert lib.htgs_create_instances(ctypes.byref(f)) == 2 and b"null pointer" in lib.htgs_last_error()
+
+
+def test_self_check_entry_points_reject_bad_arguments():
+    lib = _native.lib()
     f = _native.Frame()
     f.mode = 2
     f.width = f.height = 64
@@ -103,7 +137,6 @@ def test_measurement_and_self_check_entry_points_reject_bad_arguments():
     assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, counts) == 1               # the 16x16-tile mode does not cull
     assert b"does not cull" in lib.htgs_last_error()
     assert lib.htgs_check_reciprocal(None, None) == 2
-    assert lib.htgs_copy_bytes(None, None, 16, None) == 2
 
 
 def test_python_api_surface_and_validation():

@@ -129,3 +129,30 @@ def test_scale_modifier_and_rotated_camera(cuda, mode):
     got = gpu_stages(scene.to(cuda), mode, 16, scale_modifier=0.6)
     check_against_oracle(got, ref)
     assert ref["image"].max() > 0.05
+
+
+def test_scan_publishes_a_marker_when_the_instance_count_does_not_fit_32_bits(cuda):
+    """Offsets are 32-bit (as in the reference); tile counts (each at most 2^20, the largest supported tile grid) that
+    add up to more than 2^32 - 2 make the scan publish 0xffffffff, which the host refuses, instead of a wrapped total."""
+    import ctypes
+    from htgs_amd import _native
+    from htgs_amd.torch_bindings.rasterization import checked_instance_count
+    lib = _native.lib()
+    for counts, want in (([0x7fffffff, 0x7fffffff, 0], 0xfffffffe), ([0x7fffffff, 0x7fffffff, 1], 0xffffffff),
+                         ([1 << 20] * 5000, 0xffffffff), ([1 << 20] * 4095 + [(1 << 20) - 2], 0xfffffffe), ([3] * 5000, 15000)):
+        n = len(counts)
+        c = torch.tensor(counts, dtype=torch.int64).to(torch.int32).to(cuda)
+        offsets = torch.empty(n, dtype=torch.int32, device=cuda)
+        total = torch.zeros(1, dtype=torch.int32, device=cuda)
+        tmp = torch.empty(lib.htgs_scan_tmp_words(n), dtype=torch.int32, device=cuda)
+        f = _native.Frame()
+        f.n_primitives, f.n_touched, f.offsets, f.n_instances_dev, f.scan_tmp = n, c.data_ptr(), offsets.data_ptr(), total.data_ptr(), tmp.data_ptr()
+        f.stream = torch.cuda.current_stream(cuda).cuda_stream
+        _native.check(lib.htgs_scan_offsets(ctypes.byref(f)))
+        got = int(total.item()) & 0xffffffff
+        assert got == want
+        if want == 0xffffffff:
+            with pytest.raises(RuntimeError, match="instances"):
+                checked_instance_count(got)
+        else:
+            assert checked_instance_count(got) == want

@@ -2,7 +2,7 @@
 and the densification side outputs, against the CPU oracle on the same seeded inputs.
 
 Tolerances: image 1e-4 max abs; gradients 1e-3 relative (the GPU path sums a Gaussian's contributions in another
-order than the oracle; the global-ordering mode also uses float atomics).  "Relative" is taken per tensor against its largest reference entry, and element-wise with
+order than the oracle; no mode uses atomics, so the sums are reproducible run to run).  "Relative" is taken per tensor against its largest reference entry, and element-wise with
 rtol 1e-3 plus a small absolute term tied to that scale, because individual entries are sums with cancellation."""
 import numpy as np
 import pytest
@@ -96,3 +96,26 @@ def test_no_densification_tensor_and_untouched_inputs(cuda):
     for a, b in zip(before, leaves):
         assert torch.equal(a, b.detach())
         assert torch.isfinite(b.grad).all()
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_backward_twice_through_a_retained_graph(cuda, mode):
+    """The reference keeps everything backward needs in ctx.save_for_backward (torch_bindings/rasterization.py:71-82),
+    so a second backward through a retained graph works; here the frame stays on ctx.  Both passes are compared with
+    the oracle, each with its own upstream gradient."""
+    scene = make_scene(0, 3000)
+    arrays = [t.numpy() for t in scene.gaussians()]
+    fwd = oracle.forward(oracle_frame(scene, mode, 4), *arrays)
+    sg = scene.to(cuda)
+    leaves = [t.clone().requires_grad_(True) for t in sg.gaussians()]
+    image = diff_rasterize(*leaves, torch.empty(0, device=cuda), sg.settings(RasterizerMode(mode), 4), False)
+    for seed, retain in ((21, True), (22, False)):
+        print(f"case mode={mode} pass seed={seed}", flush=True)
+        grad_image = torch.randn(3, scene.height, scene.width, generator=torch.Generator().manual_seed(seed))
+        want = oracle.backward(fwd, grad_image.numpy(), *arrays)
+        for leaf in leaves:
+            leaf.grad = None
+        (image * grad_image.to(cuda)).sum().backward(retain_graph=retain)
+        torch.cuda.synchronize()
+        for name, leaf in zip(NAMES, leaves):
+            assert_grad_close(name, leaf.grad.cpu().numpy(), want[name])
