@@ -11,7 +11,8 @@ with S = R diag(s^2) R^T, evaluates every Gaussian at every pixel (no tiles, no 
 instances) and composites with the *definition* of each blend mode (reference README.md:17-20 and the
 constants of R/include/<mode>/config.h).  Written in torch so that autograd provides reference gradients.
 
-Everything is dense [pixels, Gaussians]; meant for a few hundred Gaussians and a few thousand pixels.
+Everything is dense [pixels, Gaussians]; meant for a few hundred Gaussians and a few thousand pixels (or, with an
+explicit pixel list and a pre-selected subset of the Gaussians, for patches of a large frame).
 """
 from __future__ import annotations
 
@@ -79,7 +80,10 @@ class Fragments:
 
 
 def evaluate(positions, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam_position, mode: int, active_sh_bases: int,
-             width: int, height: int, near_plane: float, far_plane: float, scale_modifier: float = 1.0) -> Fragments:
+             width: int, height: int, near_plane: float, far_plane: float, scale_modifier: float = 1.0,
+             pixels: torch.Tensor = None) -> Fragments:
+    """Every Gaussian at every pixel of the width x height image, or, with ``pixels`` ([P,2] integer (x, y)), at those
+    pixels only (the result then describes a 1 x P image)."""
     positions, scales, rotations = positions.to(F64), scales.to(F64), rotations.to(F64)
     opacities = opacities.to(F64).reshape(-1)
     sh_0, sh_rest = sh_0.to(F64), sh_rest.to(F64)
@@ -87,7 +91,11 @@ def evaluate(positions, scales, rotations, opacities, sh_0, sh_rest, M, VPM, cam
     VP = VPM @ torch.linalg.inv(M)                       # intrinsics with the half-pixel shift (Renderer.py:38-44)
     fx, fy, cxs, cys = VP[0, 0], VP[1, 1], VP[0, 2], VP[1, 2]
     Rc, tc = M[:3, :3], M[:3, 3]
-    ys, xs = torch.meshgrid(torch.arange(height, dtype=F64), torch.arange(width, dtype=F64), indexing="ij")
+    if pixels is None:
+        ys, xs = torch.meshgrid(torch.arange(height, dtype=F64), torch.arange(width, dtype=F64), indexing="ij")
+    else:
+        xs, ys = pixels[:, 0].to(F64).reshape(1, -1), pixels[:, 1].to(F64).reshape(1, -1)
+        height, width = 1, xs.shape[1]
     dir_c = torch.stack([(xs - cxs) / fx, (ys - cys) / fy, torch.ones_like(xs)], dim=-1).reshape(-1, 3)   # [P,3]
     origin = -Rc.T @ tc
     dir_w = dir_c @ Rc                                    # rows: Rc^T dir_c
@@ -303,3 +311,26 @@ def per_fragment_position_gradient_l1(positions, scales, rotations, opacities, s
         (g,) = torch.autograd.grad(per_pixel[p], pos, retain_graph=True)
         out += g.abs().sum(1)
     return out
+
+
+def near_ray(positions, scales, M, VPM, centre_xy, radius_px: float, cutoff: float = 3.4, slack: float = 1.5) -> torch.Tensor:
+    """Indices of the Gaussians that can reach a pixel within ``radius_px`` of the pixel ``centre_xy``: those whose centre
+    lies within  cutoff * largest scale + slack * (distance along the ray) * radius_px / focal  of the ray through
+    ``centre_xy`` (Euclidean distance in float64; sqrt(2 ln 255) = 3.33 standard deviations is the farthest a fragment is
+    accepted).  A generous, formula-free pre-selection so that the dense evaluator can be run on patches of frames with
+    millions of Gaussians; leaving out a Gaussian that contributes shows up as a mismatch, not as a silent pass."""
+    positions, scales = positions.to(F64), scales.to(F64)
+    M, VPM = M.to(F64).reshape(4, 4), VPM.to(F64).reshape(4, 4)
+    VP = VPM @ torch.linalg.inv(M)
+    fx, fy, cxs, cys = VP[0, 0], VP[1, 1], VP[0, 2], VP[1, 2]
+    Rc, tc = M[:3, :3], M[:3, 3]
+    d = torch.stack([(centre_xy[0] - cxs) / fx, (centre_xy[1] - cys) / fy, torch.ones((), dtype=F64)])
+    norm = d.norm()
+    d = (Rc.T @ d) / norm
+    delta = positions - (-Rc.T @ tc)
+    t = delta @ d
+    dist = (delta - t[:, None] * d[None, :]).norm(dim=1)
+    # a pixel radius_px away sees the ray tilted by at most radius_px / (focal * |d|) ... times |d|^2 off axis: use the
+    # looser radius_px * |d| / focal
+    reach = cutoff * scales.max(dim=1).values + slack * t.abs() * radius_px * norm / torch.minimum(fx, fy)
+    return torch.nonzero(dist <= reach).reshape(-1)

@@ -1137,6 +1137,8 @@ static void scale_rotation_grad(const oracle_cam *c, const float *scale, const f
  * first_k:      R/include/alpha_blend_first_k/kernels/backward.cuh:60-206
  * global:       R/include/alpha_blend_global_ordering/kernels/backward.cuh:60-251
  * Sums are formed in a fixed order (tile by tile, the reference uses atomics). */
+#define ATOMIC_ADD(target, value) do { const float v_ = (value); _Pragma("omp atomic") target += v_; } while (0)
+
 O_EXPORT void oracle_blend_backward(
     const oracle_cam *c, int n, const uint32_t *ranges, const uint32_t *inst,
     const float *VPMT1, const float *VPMT2, const float *VPMT4, const float *rgba,
@@ -1154,6 +1156,7 @@ O_EXPORT void oracle_blend_backward(
 
     if (mode == MODE_FIRST_K) {
         /* one stored fragment at a time, backward.cuh:81-205 */
+        #pragma omp parallel for schedule(static)
         for (size_t frag = 0; frag < np * (size_t)K; ++frag) {
             const size_t pix = frag / K, slot = frag % K;
             const uint32_t g = core_idx[slot * np + pix];
@@ -1161,7 +1164,7 @@ O_EXPORT void oracle_blend_backward(
             const float fx = (float)(pix % c->width), fy = (float)(pix / c->width);
             const float gp[3] = { grad_image[pix], grad_image[np + pix], grad_image[2 * np + pix] };
             const float *info = core_info + 4 * (slot * np + pix);
-            for (int k = 0; k < 3; ++k) grad_rgb[3 * (size_t)g + k] += info[3] * gp[k];
+            for (int k = 0; k < 3; ++k) ATOMIC_ADD(grad_rgb[3 * (size_t)g + k], info[3] * gp[k]);
             const float dL_dalpha = dot3(info, gp);
             if (dL_dalpha == 0.0f) continue;
             fragment f;
@@ -1180,20 +1183,21 @@ O_EXPORT void oracle_blend_backward(
             f.G = o_expf((-0.5f * f.num) * f.den_rcp);
             frag_grads fg;
             fragment_backward(&f, rgba[4 * (size_t)g + 3], dL_dalpha, fx, fy, &fg);
-            grad_opacities[g] += fg.opacity;
+            ATOMIC_ADD(grad_opacities[g], fg.opacity);
             float dp[3];
             position_grad(c, &fg, dp);
-            for (int k = 0; k < 3; ++k) grad_positions[3 * (size_t)g + k] += dp[k];
+            for (int k = 0; k < 3; ++k) ATOMIC_ADD(grad_positions[3 * (size_t)g + k], dp[k]);
             const float c1[3] = { fg.dV1[0], fg.dV2[0], fg.dV4[0] }, c2[3] = { fg.dV1[1], fg.dV2[1], fg.dV4[1] }, c3[3] = { fg.dV1[2], fg.dV2[2], fg.dV4[2] };
             float ds[3], dq[4];
             scale_rotation_grad(c, scales + 3 * (size_t)g, rotations + 4 * (size_t)g, c1, c2, c3, ds, dq);
-            for (int k = 0; k < 3; ++k) grad_scales[3 * (size_t)g + k] += ds[k];
-            for (int k = 0; k < 4; ++k) grad_rotations[4 * (size_t)g + k] += dq[k];
-            if (helper) helper[g] += fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]);
+            for (int k = 0; k < 3; ++k) ATOMIC_ADD(grad_scales[3 * (size_t)g + k], ds[k]);
+            for (int k = 0; k < 4; ++k) ATOMIC_ADD(grad_rotations[4 * (size_t)g + k], dq[k]);
+            if (helper) ATOMIC_ADD(helper[g], fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]));
         }
         return;
     }
 
+    #pragma omp parallel for schedule(dynamic, 4)
     for (int t = 0; t < grid_w * grid_h; ++t) {
         const int tx = t % grid_w, ty = t / grid_w;
         const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
@@ -1213,7 +1217,7 @@ O_EXPORT void oracle_blend_backward(
                     if (!reeval_fragment(c, &in, g, x, y, mode, &f)) continue;
                     const float bw = T * f.alpha;
                     const float *col = rgba + 4 * g;
-                    for (int k = 0; k < 3; ++k) grad_rgb[3 * g + k] += bw * gp[k];
+                    for (int k = 0; k < 3; ++k) ATOMIC_ADD(grad_rgb[3 * g + k], bw * gp[k]);
                     for (int k = 0; k < 3; ++k) rgb_new[k] = fmaf(bw, col[k], rgb_new[k]);
                     const float oma = 1.0f - f.alpha;
                     const float omar = 1.0f / (oma > ONE_MINUS_ALPHA_EPS ? oma : ONE_MINUS_ALPHA_EPS);
@@ -1223,16 +1227,16 @@ O_EXPORT void oracle_blend_backward(
                     if (dL_dalpha != 0.0f) {
                         frag_grads fg;
                         fragment_backward(&f, col[3], dL_dalpha, fx, fy, &fg);
-                        grad_opacities[g] += fg.opacity;
+                        ATOMIC_ADD(grad_opacities[g], fg.opacity);
                         float dp[3];
                         position_grad(c, &fg, dp);
-                        for (int k = 0; k < 3; ++k) grad_positions[3 * g + k] += dp[k];
+                        for (int k = 0; k < 3; ++k) ATOMIC_ADD(grad_positions[3 * g + k], dp[k]);
                         const float c1[3] = { fg.dV1[0], fg.dV2[0], fg.dV4[0] }, c2[3] = { fg.dV1[1], fg.dV2[1], fg.dV4[1] }, c3[3] = { fg.dV1[2], fg.dV2[2], fg.dV4[2] };
                         float ds[3], dq[4];
                         scale_rotation_grad(c, scales + 3 * g, rotations + 4 * g, c1, c2, c3, ds, dq);
-                        for (int k = 0; k < 3; ++k) grad_scales[3 * g + k] += ds[k];
-                        for (int k = 0; k < 4; ++k) grad_rotations[4 * g + k] += dq[k];
-                        if (helper) helper[g] += fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]);
+                        for (int k = 0; k < 3; ++k) ATOMIC_ADD(grad_scales[3 * g + k], ds[k]);
+                        for (int k = 0; k < 4; ++k) ATOMIC_ADD(grad_rotations[4 * g + k], dq[k]);
+                        if (helper) ATOMIC_ADD(helper[g], fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]));
                     }
                     T *= oma;
                     if (T < TRANSMITTANCE_THRESHOLD) break;
@@ -1286,14 +1290,14 @@ O_EXPORT void oracle_blend_backward(
                 a_help += fabsf(dp[0]) + fabsf(dp[1]) + fabsf(dp[2]);
             }
             for (int k = 0; k < 3; ++k) {
-                grad_rgb[3 * g + k] += a_rgb[k];
-                grad_positions[3 * g + k] += a_pos[k];
-                grad_VPMT[(size_t)(0 + k) * n + g] += a_V1[k];
-                grad_VPMT[(size_t)(3 + k) * n + g] += a_V2[k];
-                grad_VPMT[(size_t)(6 + k) * n + g] += a_V4[k];
+                ATOMIC_ADD(grad_rgb[3 * g + k], a_rgb[k]);
+                ATOMIC_ADD(grad_positions[3 * g + k], a_pos[k]);
+                ATOMIC_ADD(grad_VPMT[(size_t)(0 + k) * n + g], a_V1[k]);
+                ATOMIC_ADD(grad_VPMT[(size_t)(3 + k) * n + g], a_V2[k]);
+                ATOMIC_ADD(grad_VPMT[(size_t)(6 + k) * n + g], a_V4[k]);
             }
-            grad_opacities[g] += a_op;
-            if (helper) helper[g] += a_help;
+            ATOMIC_ADD(grad_opacities[g], a_op);
+            if (helper) ATOMIC_ADD(helper[g], a_help);
         }
     }
 }

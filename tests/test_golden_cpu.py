@@ -26,3 +26,8 @@ def test_oracle_reproduces_the_frozen_float64_answers(mode):
         want = z[f"grad_{name}_{mode}"].reshape(got[name].shape)
         scale = max(np.abs(want).max(), 1e-12)
         assert np.abs(got[name] - want).max() / scale < 2e-5, (name, np.abs(got[name] - want).max(), scale)
+    # third densification statistic: per Gaussian, the sum over the compared pixels of |dL_p/dposition|_1
+    info = np.zeros((3, sc.positions.shape[0]), np.float32)
+    oracle.backward(fwd, z["grad_image"] * mask, *arrays, densification_info=info, use_distance_scaling=False)
+    want = z[f"dens_l1_{mode}"]
+    assert np.abs(info[2] - want).max() / np.abs(want).max() < 1e-4, np.abs(info[2] - want).max()

@@ -74,6 +74,39 @@ def test_stress_scene_properties(cuda):
     print(f"  instances {n_inst}, mean tiles per visible Gaussian {n_inst / max(1, int((pre['n_touched'] > 0).sum())):.1f}", flush=True)
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_full_size_training_step_against_oracle(cuda, mode):
+    """The training configuration at its full size (1 M Gaussians, 1920x1080, K=16, upstream gradient ~N(0,1)): unclamped
+    image within 1e-4, the six gradients within 1e-3 relative, the densification statistics of the mode the scene is
+    specified for.  The oracle applies the reference's per-fragment chain (R/include/hybrid_blend/kernels/backward.cuh:104-331)."""
+    from test_gpu_training import NAMES, assert_grad_close
+    print(f"case config=4 mode={mode} (full size, forward + backward)", flush=True)
+    scene = make_scene(4)
+    arrays = [t.numpy() for t in scene.gaussians()]
+    fwd = oracle.forward(oracle_frame(scene, mode, 16), *arrays)
+    grad_image = torch.randn(3, scene.height, scene.width, generator=torch.Generator().manual_seed(4))
+    rows = 3 if mode == 0 else 0
+    info_ref = np.zeros((rows, scene.positions.shape[0]), np.float32) if rows else None
+    want = oracle.backward(fwd, grad_image.numpy(), *arrays, densification_info=info_ref, use_distance_scaling=True)
+    sg = scene.to(cuda)
+    fb = FrameBuffers(*sg.gaussians(), sg.settings(RasterizerMode(mode), 16), True, False, train=True)
+    image = fb.run_forward()
+    info = torch.zeros((rows, fb.n), device=cuda) if rows else None
+    grads = fb.run_backward(grad_image.to(cuda), info, True)
+    torch.cuda.synchronize()
+    assert fb.n_instances == len(fwd["keys"])
+    err = float(np.abs(image.cpu().numpy() - fwd["image"]).max())
+    print(f"  instances {fb.n_instances}, image max|err| {err:.3g}", flush=True)
+    assert err <= 1e-4
+    for name, got in zip(NAMES, grads):
+        assert_grad_close(name, got.cpu().numpy(), want[name])
+    if rows:
+        got_info = info.cpu().numpy()
+        np.testing.assert_array_equal(got_info[0], info_ref[0])
+        for r in (1, 2):
+            np.testing.assert_allclose(got_info[r], info_ref[r], rtol=2e-3, atol=2e-4 * float(np.abs(info_ref[r]).max()))
+
+
 def test_frames_are_reproducible_bit_for_bit(cuda):
     scene = make_scene(1, 300_000).to(cuda)
     for mode in range(4):
