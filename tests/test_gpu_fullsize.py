@@ -94,7 +94,7 @@ def test_full_size_training_step_against_oracle(cuda, mode):
     info = torch.zeros((rows, fb.n), device=cuda) if rows else None
     grads = fb.run_backward(grad_image.to(cuda), info, True)
     torch.cuda.synchronize()
-    assert fb.n_instances == len(fwd["keys"])
+    assert fb.n_instances == len(fwd["sorted_keys"])
     err = float(np.abs(image.cpu().numpy() - fwd["image"]).max())
     print(f"  instances {fb.n_instances}, image max|err| {err:.3g}", flush=True)
     assert err <= 1e-4
