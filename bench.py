@@ -30,12 +30,29 @@ FP32_PEAK_TFLOPS = 157.3
 # |m|^2, |d|^2, cut-off test: R/include/hybrid_blend/kernels/inference.cuh:137-147).  The kernels reach the same
 # decision with two quadratics (21 flops), so this prices the problem, not the instructions issued.
 FLOPS_PER_EVAL = 46
-# HBM bytes of one blend launch of the default workload: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the
-# same counters on a plain 1 GiB copy (fetch x 2.000, write x 1.000); profiles/inference_cfg2_3M_1080p_hybrid_k16.md
-MEASURED_BLEND_TRAFFIC = {(2, 0, 16, None): 3076682530}
-# share of the blend dispatch's SIMD-cycles (GRBM_GUI_ACTIVE) that the loop's instruction mix accounts for when priced
-# with the issue costs of single instructions measured on this device (same profile): 220 of 256 cycles per loop turn
-MEASURED_BLEND_VALU_BUSY = {(2, 0, 16, None): 0.86}
+# CPU baseline: one warm-up run, then this many timed runs; the median is reported
+CPU_REPS = 3
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "counters.json")
+
+
+def measured_traffic(workload_key: str):
+    """HBM bytes of the dominant kernel's launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, as recorded in
+    profiles/counters.json by ``python -m htgs_amd.diagnostics.counters`` -- or None when that file was recorded on
+    other kernel sources than the ones in this tree (the figure would describe other code)."""
+    try:
+        with open(COUNTERS_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    from htgs_amd.build import csrc_digest
+    if rec.get("csrc_sha256") != csrc_digest():
+        return None
+    entry = rec.get("launches", {}).get(workload_key)
+    return None if entry is None else entry.get("traffic_bytes")
+
+
+def workload_key(config, n, mode, K, what) -> str:
+    return f"cfg{config}" + (f"-n{n}" if n else "") + f"/mode{mode}/K{K}/{what}"
 
 
 def parse_args():
@@ -99,18 +116,43 @@ def bench_training(args, scene_cpu, scene, settings):
     fb.run_forward()
     fwd_blend = statistics.median(event_ms(fb.blend_forward, 10))
     bwd = statistics.median(event_ms(lambda: fb.run_backward(grad_image, info, info is not None), 10))
+    fb.run_backward(grad_image, info, info is not None)
+    bwd_blend_samples = event_ms(fb.blend_backward, 10)
+    bwd_blend = statistics.median(bwd_blend_samples)
+    bwd_prim = statistics.median(event_ms(fb.preprocess_backward, 10))
+    # roofline of the dominant kernel (the backward blend): it evaluates every (pixel, instance) pair again, priced as
+    # in the inference line; its algorithmic bytes are the gathered records, the per-pixel records of the forward pass,
+    # the upstream gradient and one 64-byte gradient row per instance
+    n_inst, P, K = fb.n_instances, fb.width * fb.height, fb.lib.htgs_effective_k(args.K)
+    tile_px = fb.tile * fb.tile
+    avg_ms = sum(bwd_blend_samples) / len(bwd_blend_samples)
+    records = {0: (20 * K + 24) * P, 1: 20 * K * P, 2: 12 * P, 3: 24 * P}[args.mode]
+    algo_bytes = 84 * n_inst + records + 12 * P + 64 * n_inst + (4 * n_inst if args.densification_rows == 3 else 0)
+    tflops = FLOPS_PER_EVAL * tile_px * n_inst / (avg_ms / 1e3) / 1e12
+    roofline = {"kernel": "blend_backward", "bound": "valu_fp32", "achieved": round(tflops, 3), "peak": FP32_PEAK_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(tflops / FP32_PEAK_TFLOPS, 4),
+                "traffic": measured_traffic(workload_key(args.config, args.n, args.mode, args.K, f"train{args.densification_rows}")),
+                "launch_ms": round(avg_ms, 4), "evals_per_launch": tile_px * n_inst, "algo_GB": round(algo_bytes / 1e9, 4),
+                "algo_GBps": round(algo_bytes / 1e9 / (avg_ms / 1e3), 1)}
     cpu_baseline = None
     if not args.no_cpu_baseline:
         import oracle
         fr = oracle.Frame(scene_cpu.M.numpy(), scene_cpu.VPM.numpy(), scene_cpu.cam_position.numpy(), args.mode, args.K,
                           scene_cpu.active_sh_bases, scene_cpu.width, scene_cpu.height, scene_cpu.near_plane, scene_cpu.far_plane)
         arrays = [t.numpy() for t in scene_cpu.gaussians()]
-        t0 = time.perf_counter()
-        fwd = oracle.forward(fr, *arrays)
-        oracle.backward(fwd, grad_image.cpu().numpy(), *arrays)
-        cpu_s = time.perf_counter() - t0
-        cpu_baseline = {"value": round(cpu_s * 1e3, 1), "unit": "ms/step", "cores": oracle.num_threads(), "kind": "port",
-                        "sample": "one whole forward + backward of the same workload; the C oracle's blend backward is single-threaded"}
+        gi = grad_image.cpu().numpy()
+        runs = []
+        for _ in range(1 + CPU_REPS):                       # the first run is the warm-up
+            t0 = time.perf_counter()
+            fwd = oracle.forward(fr, *arrays)
+            t1 = time.perf_counter()
+            oracle.backward(fwd, gi, *arrays)
+            runs.append((time.perf_counter() - t0, t1 - t0))
+        runs = sorted(runs[1:])
+        total_s, fwd_s = runs[len(runs) // 2]
+        cpu_baseline = {"value": round(total_s * 1e3, 1), "unit": "ms/step", "cores": oracle.num_threads(), "kind": "port",
+                        "stages_ms": {"forward": round(fwd_s * 1e3, 1), "backward": round((total_s - fwd_s) * 1e3, 1)},
+                        "sample": f"whole forward + backward of the same workload, C oracle with OpenMP; median of {CPU_REPS} runs after one warm-up"}
     print(json.dumps({
         "metric": f"training step (diff_rasterize forward + backward) {MODE_NAMES[args.mode]} K={args.K}", "value": round(ms_per_step, 4),
         "unit": "ms/step", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -118,8 +160,23 @@ def bench_training(args, scene_cpu, scene, settings):
         "config": {"workload": f"{scene.name} {MODE_NAMES[args.mode]} K={args.K} forward+backward, {fb.n} Gaussians, "
                                f"{scene.width}x{scene.height}", "n_instances": fb.n_instances,
                    "densification_rows": args.densification_rows},
-        "stages": {"blend_forward_ms": round(fwd_blend, 4), "backward_ms": round(bwd, 4)},
+        "stages": {"blend_forward_ms": round(fwd_blend, 4), "backward_ms": round(bwd, 4), "blend_backward_ms": round(bwd_blend, 4),
+                   "preprocess_backward_ms": round(bwd_prim, 4)},
+        "roofline": roofline,
         "cpu_baseline": cpu_baseline}))
+
+
+def cpu_frame(oracle, fr, arrays):
+    """One inference frame on the CPU oracle, stage by stage; seconds per stage (same stages as the GPU breakdown)."""
+    t = [time.perf_counter()]
+    pre = oracle.preprocess(fr, *arrays); t.append(time.perf_counter())
+    offsets = oracle.inclusive_scan(pre["n_touched"]); t.append(time.perf_counter())
+    keys, vals = oracle.create_instances(fr, pre, offsets); t.append(time.perf_counter())
+    skeys, svals = oracle.sort_pairs(keys, vals, oracle.end_bit(fr)); t.append(time.perf_counter())
+    ranges = oracle.extract_ranges(fr, skeys); t.append(time.perf_counter())
+    oracle.blend(fr, pre, ranges, svals, True, False); t.append(time.perf_counter())
+    names = ("preprocess", "scan", "create_instances", "sort", "extract_ranges", "blend")
+    return {n: t[i + 1] - t[i] for i, n in enumerate(names)}
 
 
 def main():
@@ -224,7 +281,7 @@ def main():
         "preprocess": N * (56 + 12 * (B - 1) * (B > 1)) + 4 * N + 88 * n_vis,   # 80 B record + 8 B bounds per visible Gaussian
         "scan": 8 * N,
         "create_instances": 16 * n_vis + (kb + 4) * n_inst,
-        "sort": passes * 2 * (kb + 4) * n_inst + passes * kb * n_inst,
+        "sort": passes * 2 * (kb + 4) * n_inst + kb * n_inst,            # every pass moves the pairs once each way; the keys are read once more for the histograms
         "extract_ranges": kb * n_inst + 8 * T,
         "blend": 84 * n_inst + 16 * P,
     }
@@ -239,8 +296,7 @@ def main():
     roofline = {
         "kernel": "blend", "bound": "valu_fp32", "achieved": round(achieved_tflops, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved_tflops / FP32_PEAK_TFLOPS, 4),
-        "traffic": None if args.fast else MEASURED_BLEND_TRAFFIC.get((args.config, args.mode, args.K, args.n)),
-        "valu_busy": None if args.fast else MEASURED_BLEND_VALU_BUSY.get((args.config, args.mode, args.K, args.n)),
+        "traffic": measured_traffic(workload_key(args.config, args.n, args.mode, args.K, "fast_rasterize" if args.fast else "rasterize")),
         "launch_ms": round(blend_avg_ms, 4), "evals_per_launch": tile_px * n_inst,
     }
 
@@ -251,11 +307,12 @@ def main():
         fr = oracle.Frame(scene_cpu.M.numpy(), scene_cpu.VPM.numpy(), scene_cpu.cam_position.numpy(), args.mode, args.K,
                           scene_cpu.active_sh_bases, scene_cpu.width, scene_cpu.height, scene_cpu.near_plane, scene_cpu.far_plane)
         arrays = [t.numpy() for t in scene_cpu.gaussians()]
-        t0 = time.perf_counter()
-        oracle.render(fr, *arrays)
-        cpu_s = time.perf_counter() - t0
+        runs = [cpu_frame(oracle, fr, arrays) for _ in range(1 + CPU_REPS)][1:]         # the first run is the warm-up
+        totals = sorted(sum(r.values()) for r in runs)
+        cpu_s = totals[len(totals) // 2]
         cpu_baseline = {"value": round(1.0 / cpu_s, 4), "unit": "FPS", "cores": oracle.num_threads(), "kind": "port",
-                        "sample": f"one whole frame of the same workload, C oracle with OpenMP, {cpu_s:.2f} s"}
+                        "stages_ms": {k: round(statistics.median(r[k] for r in runs) * 1e3, 2) for k in runs[0]},
+                        "sample": f"whole frames of the same workload, C oracle with OpenMP; median of {CPU_REPS} runs after one warm-up, {cpu_s:.2f} s per frame"}
 
     line = {
         "metric": f"FPS {MODE_NAMES[args.mode]} K={args.K} fast_rasterize (image only, reduced accuracy)" if args.fast

@@ -32,6 +32,18 @@ def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def csrc_digest() -> str:
+    """SHA-256 over the kernel sources and the C ABI header: the code version a profile-derived figure is tied to."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in [*sources(), *sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")),
+                 os.path.join(os.path.dirname(HERE), "include", "htgs_amd.h")]:
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):

@@ -831,7 +831,7 @@ extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0 || f->n_primitives < 0)
         return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: bad argument");
     if (f->n_primitives == 0 || f->n_instances == 0) return HTGS_OK;
-    if (f->n_primitives > (1 << 27)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: more than 2^27 Gaussians");
+    if (f->n_primitives >= (1 << 27)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: 2^27 Gaussians or more");
     const bool needs_core = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K;
     const bool needs_tail = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_OIT_BLEND;
     if (!f->ranges || !f->vals[selector] || !f->prim || !f->grad_image || !f->VPM || !f->grad_rows || !f->offsets || !f->bounds ||

@@ -95,6 +95,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
         tail1 = __builtin_fmaf(-ca[i], cc[i].y, tail1);
         tail2 = __builtin_fmaf(-ca[i], cc[i].z, tail2);
     }
+    tail0 = clamp_pos(tail0); tail1 = clamp_pos(tail1); tail2 = clamp_pos(tail2);   // colours are >= 0, so is the exact difference
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         if (T_core >= kTransmittanceThreshold) {

@@ -82,6 +82,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
         tail1 = __builtin_fmaf(-c3[i], c1[i], tail1);
         tail2 = __builtin_fmaf(-c3[i], c2[i], tail2);
     }
+    tail0 = clamp_pos(tail0); tail1 = clamp_pos(tail1); tail2 = clamp_pos(tail2);   // colours are >= 0, so is the exact difference
     float r = 0.0f, g = 0.0f, b = 0.0f, T_core = 1.0f;
 #pragma unroll
     for (int i = 0; i < K; ++i) {

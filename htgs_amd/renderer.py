@@ -33,11 +33,11 @@ def view_projection(camera) -> np.ndarray:
 def extract_settings(view, mode: int, K: int, active_sh_bases: int, scale_modifier: float, device="cuda") -> RasterizerSettings:
     camera = view.camera
     if getattr(camera, "distortion", None) is not None:
-        warnings.warn("found distortion parameters that will be ignored by the rasterizer")
+        warnings.warn("the camera carries lens-distortion parameters; the rasterizer renders an undistorted pinhole image")
     try:
         rasterizer_mode = RasterizerMode(mode)
     except ValueError:
-        warnings.warn(f"Invalid rasterizer mode: {mode}. Defaulting to HYBRID_BLEND.")
+        warnings.warn(f"rasterizer mode {mode!r} does not exist (0-3); using HYBRID_BLEND")
         rasterizer_mode = RasterizerMode.HYBRID_BLEND
     M = np.asarray(view.w2c_numpy)
     VPM = view_projection(camera).astype(M.dtype) @ M

@@ -322,8 +322,17 @@ class FrameBuffers:
         f.densification_rows = rows
         f.dens_helper = _ptr(helper)
         f.use_distance_scaling = int(bool(use_distance_scaling))
+        self.grads = grads           # keeps the bound outputs alive for blend_backward / preprocess_backward
         _native.check(self.lib.htgs_backward(self._ref, self.selector))
         return grads
+
+    def blend_backward(self):
+        """The blend half of the last ``run_backward`` again, into the same buffers (per-stage timing)."""
+        _native.check(self.lib.htgs_blend_backward(self._ref, self.selector))
+
+    def preprocess_backward(self):
+        """The per-Gaussian half of the last ``run_backward`` again (densification_info is accumulated once more)."""
+        _native.check(self.lib.htgs_preprocess_backward(self._ref))
 
 
 class _Rasterize(torch.autograd.Function):

@@ -677,6 +677,7 @@ static void hybrid_pixel(const oracle_cam *c, const blend_in *in, uint32_t first
     }
     for (int i = 0; i < K; ++i)
         for (int k = 0; k < 3; ++k) tail[k] = fmaf(-core[i][3], core[i][k], tail[k]);
+    for (int k = 0; k < 3; ++k) tail[k] = tail[k] > 0.0f ? tail[k] : 0.0f;    /* colours are >= 0: so is the exact difference */
     float rgb[3] = { 0, 0, 0 }, depth_pixel = 0.0f, T_core = 1.0f;
     for (int i = 0; i < K && T_core >= TRANSMITTANCE_THRESHOLD; ++i) {                         /* :180 */
         const float w = T_core * core[i][3];
@@ -869,6 +870,7 @@ static void hybrid_pixel_forward(const blend_in *in, uint32_t first, uint32_t la
     }
     for (int i = 0; i < K; ++i)
         for (int k = 0; k < 3; ++k) tail[k] = fmaf(-core[i][3], core[i][k], tail[k]);
+    for (int k = 0; k < 3; ++k) tail[k] = tail[k] > 0.0f ? tail[k] : 0.0f;    /* colours are >= 0: so is the exact difference */
     float rgb[3] = { 0, 0, 0 }, T_core = 1.0f;
     for (int i = 0; i < K && T_core >= TRANSMITTANCE_THRESHOLD; ++i) {                         /* :184-190 */
         const float bw = T_core * core[i][3];

@@ -100,3 +100,46 @@ def test_third_densification_row_is_the_per_pixel_l1_norm_of_the_position_gradie
     oracle.backward(fwd, gi.numpy(), *arrays, densification_info=info, use_distance_scaling=scaling)
     assert np.abs(want).max() > 1.0 and (want > 0).sum() >= 8
     assert np.abs(info[2] - want).max() <= 1e-4 * np.abs(want).max(), (info[2], want)
+
+
+def faint_tail_scene(K: int, seed: int):
+    """K fairly opaque Gaussians over the middle of the image in front of six large ones whose alpha stays between
+    1/255 and 1/100: the case in which the colour sums of the hybrid tail (all fragments added, the core's share
+    subtracted at the end) cancel most."""
+    sc = small_scene(n=K + 6, seed=seed, sh_degree=1, width=32, height=24, focal=40.0, scale=(0.35, 0.55), z_range=(2.2, 3.0))
+    g = torch.Generator().manual_seed(seed + 1)
+    z = sc.positions @ sc.M[2, :3] + sc.M[2, 3]
+    centre = sc.cam_position[None, :] + z[:, None] * sc.M[2, :3][None, :]
+    sc.positions[:K] = centre[:K] + 0.4 * (sc.positions[:K] - centre[:K])
+    sc.opacities[:K] = 0.1 + 0.5 * torch.rand(K, 1, generator=g)
+    sc.opacities[K:] = 0.0045 + 0.0045 * torch.rand(6, 1, generator=g)
+    sc.scales[K:] *= 3.0
+    sc.positions[K:] += (7.0 - z[K:, None]) * sc.M[2, :3][None, :]                    # the faint ones behind the core
+    return sc
+
+
+@pytest.mark.parametrize("K", [4, 16])
+def test_hybrid_tail_with_a_strong_core_and_a_faint_tail(K):
+    """Image and gradients of HYBRID_BLEND against the float64 evaluator where the tail's colour sums are the small
+    difference of two large ones (every fragment's alpha * colour is added when it is evaluated and the K core entries'
+    share is taken out after the walk; the reference, R/include/hybrid_blend/kernels/inference.cuh:158-170, only ever
+    adds what is outside the core)."""
+    sc = faint_tail_scene(K, 100 + K)
+    arrays = [t.numpy() for t in sc.gaussians()]
+    fwd = oracle.forward(oracle_frame(sc, 0, K), *arrays)
+    tail = fwd["tail_info"].reshape(6, -1)
+    alpha_sum = 1.0 / np.maximum(tail[3], 1e-30)
+    in_core = (fwd["core_idx"].reshape(K, -1) != 0xffffffff).sum(0)
+    faint = (tail[3] > 0) & (alpha_sum < 0.1) & (tail[5] > 0.01) & (in_core >= min(K, 3))
+    assert faint.mean() > 0.15, "the scene is meant to have faint tails behind a partly transparent core"
+    assert (tail[:3] >= 0).all()
+    gi = torch.randn(3, sc.height, sc.width, generator=torch.Generator().manual_seed(1))
+    img, mask, want = autograd_reference(sc, 0, K, gi)
+    assert mask.float().mean() > 0.9
+    assert np.abs(fwd["image"] - img.numpy())[:, mask.numpy()].max() < 2e-5
+    got = oracle.backward(fwd, (gi * mask.float()).numpy(), *arrays)
+    for name, w in zip(NAMES, want):
+        g = got[name]
+        w = w.numpy().reshape(g.shape)
+        scale = max(np.abs(w).max(), 1e-12)
+        assert np.abs(g - w).max() / scale < 5e-5, (name, np.abs(g - w).max(), scale)

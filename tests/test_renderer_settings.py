@@ -51,5 +51,5 @@ def test_same_matrices_as_the_synthetic_scenes_and_mode_fallback():
     with warnings.catch_warnings(record=True) as caught:
         warnings.simplefilter("always")
         s = extract_settings(view, 7, 4, 1, 1.0, device="cpu")
-    assert s.mode is RasterizerMode.HYBRID_BLEND and any("Invalid rasterizer mode" in str(w.message) for w in caught)
+    assert s.mode is RasterizerMode.HYBRID_BLEND and any("HYBRID_BLEND" in str(w.message) for w in caught)
     assert torch.allclose(s.M, M) and torch.allclose(s.VPM, VPM, atol=1e-5) and torch.allclose(s.cam_position, position, atol=1e-6)
