@@ -20,10 +20,14 @@ PROBES_LIB_PATH = os.path.join(HERE, "diagnostics", "libhtgs_probes.so")
 # -ffp-contract=off: a fused multiply-add exists only where the sources write __builtin_fmaf, which is what
 #   makes tile counts and accept/reject decisions reproducible (see csrc/common.h).
 # -packed-fp32-ops disabled: no v_pk_{add,mul,fma}_f32.
+# -disable-promote-alloca-to-vector: the K-buffer arrays of the blend kernels (constant indices once the loops are
+#   unrolled) must end up as individual registers; promoted early to one 16- or 32-wide vector value they are allocated
+#   as a register tuple and spilled around the insertion chain.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-gpu-flush-denormals-to-zero",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-disable-promote-alloca-to-vector=1",
     "-Wno-unused-command-line-argument",
 ]
 

@@ -37,9 +37,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
     const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
+    uint32_t local_x, local_y;
+    quadrant_pixel(lane, local_x, local_y);
+    const uint32_t x = x0 + local_x, y = y0 + local_y;
     const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
+    const PixelTerms pt = pixel_terms(local_x, local_y, 8);
     const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
 
     float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f, depth_tail = 0.0f;
@@ -49,23 +51,29 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     // entry pushed out of the core needs no colour: its alpha and depth, which the tail also needs, are in the slot.
     float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
 #pragma unroll
-    for (int i = 0; i < K; ++i) { cd[i] = __FLT_MAX__; ca[i] = 0.0f; ci[i] = 0.0f; }
+    for (int i = 0; i < K; ++i) {
+        cd[i] = __FLT_MAX__; ca[i] = 0.0f; ci[i] = 0.0f;
+        asm volatile("" : "+v"(cd[i]), "+v"(ca[i]), "+v"(ci[i]));      // one register per slot, never a 16-wide tuple
+    }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            while (hits) {
-                const uint32_t addr = stage_next_hit(hits, stage_base);
+            const auto turn = [&](uint32_t addr) {
+                addr += stage_base;
+                // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
+                // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
+                // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
                 TileFrag f;
-                if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+                const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
                 f.den_rcp = frag_rcp<FAST>(f.den);
                 const float4 col = stage_row<64, 5>(addr);
-                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
+                if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach)) return;
                 float depth = tile_frag_depth<64>(addr, pt, f);
                 float p3 = f.alpha;
                 tail0 = __builtin_fmaf(p3, col.x, tail0);
@@ -77,8 +85,14 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 }
                 // (depth, p3) is the fragment itself, the entry it pushed out of the core, or an empty slot (alpha 0)
                 tail3 += p3;
-                if (!FAST && !median) depth_tail = __builtin_fmaf(depth, p3, depth_tail);
+                if (!FAST) depth_tail = __builtin_fmaf(depth, p3, depth_tail);      // (not used for the median depth)
                 T_tail *= 1.0f - p3;
+            };
+            for (;;) {
+                const uint32_t addr = quadrant_next_hit(hits);
+                const bool live = addr != kNoHit;
+                if (__ballot(live) == 0) break;                  // every quadrant has walked its hits
+                if (live) turn(addr);
             }
         }
     }

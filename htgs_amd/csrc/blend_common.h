@@ -111,6 +111,47 @@ __device__ __forceinline__ bool tile_misses(const float (&n)[6], const float (&d
     return convex && least > margin;                 // (a quadratic that is not convex along the rows is never left out)
 }
 
+// The same bound per 4x4 quadrant of the 8x8 tile: bit q = 2 (row >= 4) + (column >= 4) of the result is clear when no
+// pixel of that quadrant can pass.  Per pixel row the least value of Q over a quadrant's four pixels is at the one
+// nearest to the vertex, so two evaluations per row serve the row's two quadrants.
+template <int MODE>
+__device__ __forceinline__ uint32_t tile_quadrant_hits(const float (&n)[6], const float (&d)[6], float opacity)
+{
+    static_assert(ModeCfg<MODE>::tile == 8, "8x8 tiles");
+    constexpr float h = 3.5f;
+    float r = __builtin_fmaf(__builtin_amdgcn_logf(opacity), -1.0f / ModeCfg<MODE>::exp2_scale, 1.0f);
+    r = r < 1.0f ? r : 1.0f;
+    r = r > -1.0f ? r : -1.0f;
+    r += 1e-5f;
+    float q[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) q[i] = __builtin_fmaf(-r, d[i], n[i]);
+    const float s0 = __builtin_fabsf(n[0]) + __builtin_fabsf(d[0]);
+    const float s1 = (__builtin_fabsf(n[1]) + __builtin_fabsf(d[1])) + (__builtin_fabsf(n[2]) + __builtin_fabsf(d[2]));
+    const float s2 = ((__builtin_fabsf(n[3]) + __builtin_fabsf(d[3])) + (__builtin_fabsf(n[4]) + __builtin_fabsf(d[4]))) +
+                     (__builtin_fabsf(n[5]) + __builtin_fabsf(d[5]));
+    const float margin = 1e-5f * __builtin_fmaf(h * h, s2, __builtin_fmaf(h, s1, s0));
+    if (!(q[3] > 0.0f)) return 0xfu;                 // (not convex along the rows, or not a number: kept everywhere)
+    const float to_vertex = -0.5f * __builtin_amdgcn_rcpf(q[3]);
+    uint32_t bits = 0;
+#pragma nounroll
+    for (int half = 0; half < 2; ++half) {
+        float least_l = __FLT_MAX__, least_r = __FLT_MAX__;
+#pragma nounroll
+        for (int row = 0; row < 4; ++row) {
+            const float y = (float)(4 * half + row) - h;
+            const float b = __builtin_fmaf(q[4], y, q[1]);
+            const float c = __builtin_fmaf(y, __builtin_fmaf(q[5], y, q[2]), q[0]);
+            const float xv = __builtin_rintf(__builtin_fmaf(b, to_vertex, 0.5f)) - 0.5f;
+            const float xl = __builtin_fminf(__builtin_fmaxf(xv, -h), -0.5f), xr = __builtin_fminf(__builtin_fmaxf(xv, 0.5f), h);
+            least_l = __builtin_fminf(least_l, __builtin_fmaf(xl, __builtin_fmaf(q[3], xl, b), c));
+            least_r = __builtin_fminf(least_r, __builtin_fmaf(xr, __builtin_fmaf(q[3], xr, b), c));
+        }
+        bits |= (least_l > margin ? 0u : 1u << (2 * half)) | (least_r > margin ? 0u : 2u << (2 * half));
+    }
+    return bits;
+}
+
 // Stages instance `fetch` of the sorted list in slot `slot` (the same arithmetic as tile_geometry / tile_quadratics,
 // written out so that every row is stored as soon as it is complete: the kernels that call this hold a K-buffer in
 // registers).  Returns whether the slot holds an instance that can reach a pixel of the tile: always true for a
@@ -118,11 +159,12 @@ __device__ __forceinline__ bool tile_misses(const float (&n)[6], const float (&d
 // (kCullAlpha), or the cut-off alone (kCullCutoff: the test with opacity 1).  What that leaves out contributes to
 // no pixel, so a walk over the hits alone gives the results of the full walk bit for bit.
 enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2 };
-template <int MODE, int N, bool DEPTH, int CULL = kCullNone>
-__device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
-                                                uint32_t fetch, uint32_t last, int slot, float cx, float cy)
+// With QUADRANTS the result has one bit per 4x4 quadrant of the tile (tile_quadrant_hits) instead of one for the tile.
+template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false>
+__device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
+                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy)
 {
-    if (fetch >= last) return false;
+    if (fetch >= last) return 0;
     const uint32_t g = inst[fetch];
     const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
     // (with CULL the record's colour row is fetched when it is needed, behind a compiler fence: it comes from a cache
@@ -172,7 +214,9 @@ __device__ __forceinline__ bool tile_stage_load(TileStage<N> &st, const float4 *
     }
     st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
     st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
-    return CULL == kCullNone ? true : !tile_misses<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
+    if constexpr (CULL == kCullNone) return QUADRANTS ? 0xfu : 1u;
+    else if constexpr (QUADRANTS) return tile_quadrant_hits<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
+    else return (uint32_t)!tile_misses<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
 }
 
 // the pixel's offset from the tile centre (exact)
@@ -216,6 +260,53 @@ __device__ __forceinline__ uint32_t stage_next_hit(uint64_t &hits, uint32_t stag
     hits &= hits - 1;
     uint32_t addr;
     asm volatile("v_mov_b32 %0, %1" : "=v"(addr) : "s"(at));
+    return addr;
+}
+// Quadrant walk.  Lanes 16 q .. 16 q + 15 hold the 4x4 pixels of quadrant q of the tile and walk the hits of that
+// quadrant, in list order, in lock step with the other three quadrants: a turn of the loop serves up to four instances,
+// one per quadrant, and a batch takes as many turns as its busiest quadrant has hits (an instance reaches 1.9 of the four
+// quadrants on average, so this is well under the number of instances that reach the tile).  Every pixel still sees its
+// fragments in list order.  The four hit masks are wave-uniform (scalar registers).
+constexpr uint32_t kNoHit = 0xfffffff0u;           // 16 * s_ff1(0): the address a quadrant without a hit left gets
+struct QuadrantHits {
+    uint64_t h[4];
+};
+__device__ __forceinline__ void quadrant_pixel(uint32_t lane, uint32_t &local_x, uint32_t &local_y)
+{
+    local_x = ((lane >> 4) & 1) * 4 + (lane & 3);
+    local_y = (lane >> 5) * 4 + ((lane >> 2) & 3);
+}
+__device__ __forceinline__ QuadrantHits quadrant_ballot(uint32_t bits)
+{
+    QuadrantHits w;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) w.h[q] = __ballot((bits >> q) & 1);
+    return w;
+}
+__device__ __forceinline__ bool quadrant_pending(const QuadrantHits &w) { return (w.h[0] | w.h[1] | w.h[2] | w.h[3]) != 0; }
+// LDS address, relative to the stage, of the q[0] entry of the lane's quadrant's next hit, or kNoHit.  Per quadrant two
+// scalar instructions: s_ff1 gives the slot (-1 for an empty mask, which the shift turns into kNoHit) and s_bitset0
+// clears that bit (bit 63 of an empty mask).  A quadrant is one row of sixteen lanes to the data-parallel primitives, so
+// its lanes take the slot by a move with that row's mask: no exec writes, and the scalar unit, which the four SIMDs of a
+// compute unit share, is left to the loop's branches.
+__device__ __forceinline__ uint32_t quadrant_next_hit(QuadrantHits &w)
+{
+    uint32_t a0, a1, a2, a3, addr, t;
+    asm volatile("s_ff1_i32_b64 %[a0], %[h0]\n\ts_ff1_i32_b64 %[a1], %[h1]\n\ts_ff1_i32_b64 %[a2], %[h2]\n\ts_ff1_i32_b64 %[a3], %[h3]\n\t"
+                 "s_bitset0_b64 %[h0], %[a0]\n\ts_bitset0_b64 %[h1], %[a1]\n\ts_bitset0_b64 %[h2], %[a2]\n\ts_bitset0_b64 %[h3], %[a3]\n\t"
+                 "v_mov_b32 %[addr], %[a0]\n\t"
+                 "v_mov_b32 %[t], %[a1]\n\t"
+                 "s_nop 1\n\t"
+                 "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x2 bank_mask:0xf\n\t"
+                 "v_mov_b32 %[t], %[a2]\n\t"
+                 "s_nop 1\n\t"
+                 "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x4 bank_mask:0xf\n\t"
+                 "v_mov_b32 %[t], %[a3]\n\t"
+                 "s_nop 1\n\t"
+                 "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x8 bank_mask:0xf\n\t"
+                 "v_lshlrev_b32 %[addr], 4, %[addr]"
+                 : [a0] "=&s"(a0), [a1] "=&s"(a1), [a2] "=&s"(a2), [a3] "=&s"(a3), [addr] "=&v"(addr), [t] "=&v"(t),
+                   [h0] "+s"(w.h[0]), [h1] "+s"(w.h[1]), [h2] "+s"(w.h[2]), [h3] "+s"(w.h[3]));
     return addr;
 }
 template <int N, int ROW>
@@ -284,6 +375,27 @@ __device__ __forceinline__ void exchange_step(float &D, float &A, IndexT &I, flo
                  : [all] "s"(all)
                  : "vcc");
 }
+// four slots in one statement: exec is saved once and restored after every slot
+#define HTGS_EXCHANGE_SLOT(n)                                                                                            \
+    "v_cmpx_lt_f32 vcc, %[d], %[D" #n "]\n\t"                                                                           \
+    "v_mov_b32 %[t], %[D" #n "]\n\tv_mov_b32 %[D" #n "], %[d]\n\tv_mov_b32 %[d], %[t]\n\t"                              \
+    "v_mov_b32 %[t], %[A" #n "]\n\tv_mov_b32 %[A" #n "], %[a]\n\tv_mov_b32 %[a], %[t]\n\t"                              \
+    "v_mov_b32 %[t], %[I" #n "]\n\tv_mov_b32 %[I" #n "], %[x]\n\tv_mov_b32 %[x], %[t]\n\t"                              \
+    "s_mov_b64 exec, %[all]\n\t"
+template <typename IndexT>
+__device__ __forceinline__ void exchange_step4(float &d, float &a, IndexT &x, float &D0, float &A0, IndexT &I0, float &D1, float &A1, IndexT &I1,
+                                               float &D2, float &A2, IndexT &I2, float &D3, float &A3, IndexT &I3)
+{
+    static_assert(sizeof(IndexT) == 4, "one register");
+    float t;
+    uint64_t all;
+    asm volatile("s_mov_b64 %[all], exec\n\t" HTGS_EXCHANGE_SLOT(0) HTGS_EXCHANGE_SLOT(1) HTGS_EXCHANGE_SLOT(2) HTGS_EXCHANGE_SLOT(3)
+                 : [d] "+v"(d), [a] "+v"(a), [x] "+v"(x), [D0] "+v"(D0), [A0] "+v"(A0), [I0] "+v"(I0), [D1] "+v"(D1), [A1] "+v"(A1), [I1] "+v"(I1),
+                   [D2] "+v"(D2), [A2] "+v"(A2), [I2] "+v"(I2), [D3] "+v"(D3), [A3] "+v"(A3), [I3] "+v"(I3), [t] "=&v"(t), [all] "=&s"(all)
+                 :
+                 : "vcc");
+}
+#undef HTGS_EXCHANGE_SLOT
 template <int K, typename IndexT>
 __device__ __forceinline__ void core_exchange_walk(float &depth, float &alpha, IndexT &index, float (&cd)[K], float (&ca)[K], IndexT (&ci)[K])
 {
@@ -291,8 +403,13 @@ __device__ __forceinline__ void core_exchange_walk(float &depth, float &alpha, I
 #pragma unroll
     for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
         if (K > kInsertGroup && !__any(depth < cd[g0 + kInsertGroup - 1 < K ? g0 + kInsertGroup - 1 : K - 1])) continue;
+        if constexpr (K % kInsertGroup == 0 && kInsertGroup == 4) {
+            exchange_step4(depth, alpha, index, cd[g0], ca[g0], ci[g0], cd[g0 + 1], ca[g0 + 1], ci[g0 + 1], cd[g0 + 2], ca[g0 + 2], ci[g0 + 2],
+                           cd[g0 + 3], ca[g0 + 3], ci[g0 + 3]);
+        } else {
 #pragma unroll
-        for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) exchange_step(depth, alpha, index, cd[i], ca[i], ci[i], all);
+            for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) exchange_step(depth, alpha, index, cd[i], ca[i], ci[i], all);
+        }
     }
 }
 

@@ -57,6 +57,25 @@ PROBE_ISSUE_KERNEL(issue_cvt_kernel, PROBE_OP_CVT)
 PROBE_ISSUE_KERNEL(issue_lshladd_kernel, PROBE_OP_LSHLADD)
 PROBE_ISSUE_KERNEL(issue_rcp_kernel, PROBE_OP_RCP)
 PROBE_ISSUE_KERNEL(issue_exp_kernel, PROBE_OP_EXP)
+// the same instruction with part of the wave switched off: does a wave64 instruction with an empty half (or with one
+// row of sixteen lanes active) hold the SIMD for less time?
+#define PROBE_MASKED_KERNEL(name, op, mask)                                                                                       \
+    __global__ void __launch_bounds__(256) name(float *__restrict__ out, int turns)                                              \
+    {                                                                                                                            \
+        float a0 = threadIdx.x * 1e-3f, a1 = a0 + 1.0f, a2 = a0 + 2.0f, a3 = a0 + 3.0f, a4 = a0 + 4.0f, a5 = a0 + 5.0f,            \
+              a6 = a0 + 6.0f, a7 = a0 + 7.0f;                                                                                    \
+        const float m = 1.0001f, c = 0.5f;                                                                                       \
+        for (int i = 0; i < turns; ++i)                                                                                          \
+            asm volatile("s_mov_b64 s[40:41], exec\ns_mov_b64 exec, " mask "\n" PROBE_R64(op) "s_mov_b64 exec, s[40:41]\n"        \
+                         : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(a4), "+v"(a5), "+v"(a6), "+v"(a7)                       \
+                         : "v"(m), "v"(c)                                                                                        \
+                         : "vcc", "s40", "s41");                                                                                 \
+        out[blockIdx.x * 256 + threadIdx.x] = a0 + a1 + a2 + a3 + a4 + a5 + a6 + a7;                                             \
+    }
+PROBE_MASKED_KERNEL(issue_mov_half_kernel, PROBE_OP_MOV, "0xffffffff")
+PROBE_MASKED_KERNEL(issue_mov_row_kernel, PROBE_OP_MOV, "0xffff")
+PROBE_MASKED_KERNEL(issue_fma_half_kernel, PROBE_OP_FMA, "0xffffffff")
+PROBE_MASKED_KERNEL(issue_cmp_half_kernel, PROBE_OP_CMP, "0xffffffff")
 // (v_swap_b32 writes both operands: the second one is a ninth register of its own)
 __global__ void __launch_bounds__(256) issue_swap_kernel(float *__restrict__ out, int turns)
 {
@@ -72,6 +91,8 @@ static const IssueCase kIssueCases[] = {
     { "v_add_u32", issue_addu_kernel }, { "v_min_f32", issue_min_kernel }, { "v_cmp_lt_f32", issue_cmp_kernel },
     { "v_cndmask_b32", issue_cnd_kernel }, { "v_rndne_f32", issue_rnd_kernel }, { "v_cvt_i32_f32", issue_cvt_kernel },
     { "v_lshl_add_u32", issue_lshladd_kernel }, { "v_rcp_f32", issue_rcp_kernel }, { "v_exp_f32", issue_exp_kernel }, { "v_swap_b32", issue_swap_kernel },
+    { "v_mov_b32, lanes 0-31 only", issue_mov_half_kernel }, { "v_mov_b32, lanes 0-15 only", issue_mov_row_kernel },
+    { "v_fma_f32, lanes 0-31 only", issue_fma_half_kernel }, { "v_cmp_lt_f32, lanes 0-31 only", issue_cmp_half_kernel },
 };
 constexpr int kIssueCaseCount = (int)(sizeof(kIssueCases) / sizeof(kIssueCases[0]));
 
