@@ -36,13 +36,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    uint32_t local_x, local_y;
-    quadrant_pixel(lane, local_x, local_y);
-    const uint32_t x = x0 + local_x, y = y0 + local_y;
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(local_x, local_y, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const uint32_t x = px.x, y = px.y;
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
 
     float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f, depth_tail = 0.0f;
     // A core slot holds depth, alpha and the Gaussian's index (an exchange moves three registers); the colours are
@@ -64,8 +62,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
         {
             // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            const auto turn = [&](uint32_t addr) {
-                addr += stage_base;
+            quadrant_walk(hits, stage_base, [&](uint32_t addr) {
                 // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
                 // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
                 // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
@@ -87,13 +84,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 tail3 += p3;
                 if (!FAST) depth_tail = __builtin_fmaf(depth, p3, depth_tail);      // (not used for the median depth)
                 T_tail *= 1.0f - p3;
-            };
-            for (;;) {
-                const uint32_t addr = quadrant_next_hit(hits);
-                const bool live = addr != kNoHit;
-                if (__ballot(live) == 0) break;                  // every quadrant has walked its hits
-                if (live) turn(addr);
-            }
+            });
         }
     }
     if (!inside) return;
@@ -148,36 +139,38 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const uint32_t x = px.x, y = px.y;
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
 
     float ca[K], cd[K];
     uint32_t ci[K];
 #pragma unroll
-    for (int i = 0; i < K; ++i) { ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+    for (int i = 0; i < K; ++i) {
+        ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu;
+        asm volatile("" : "+v"(cd[i]), "+v"(ca[i]), "+v"(ci[i]));      // one register per slot
+    }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            while (hits) {
-                const uint32_t addr = stage_next_hit(hits, stage_base);
+            quadrant_walk(hits, stage_base, [&](uint32_t addr) {
                 TileFrag f;
-                if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+                const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
                 f.den_rcp = frag_rcp<FAST>(f.den);
                 float depth = tile_frag_depth<64>(addr, pt, f);
-                if (depth >= cd[K - 1]) continue;                      // depth test before the exponential (:151)
-                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
+                if (!(in_reach && depth < cd[K - 1])) return;          // depth test before the exponential (:151)
+                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) return;
                 float alpha = f.alpha;
                 uint32_t idx = stage_index<64>(addr);
                 core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
-            }
+            });
         }
     }
     if (!inside) return;
@@ -214,27 +207,26 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const uint32_t x = px.x, y = px.y;
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         {
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            while (hits) {
-                const uint32_t addr = stage_next_hit(hits, stage_base);
+            quadrant_walk(hits, stage_base, [&](uint32_t addr) {
                 TileFrag f;
-                if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+                const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
                 f.den_rcp = frag_rcp<FAST>(f.den);
                 const float4 col = stage_row<64, 5>(addr);
-                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) continue;
+                if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach)) return;
                 const float depth = FAST ? 0.0f : tile_frag_depth<64>(addr, pt, f);
                 a0 = __builtin_fmaf(f.alpha, col.x, a0);
                 a1 = __builtin_fmaf(f.alpha, col.y, a1);
@@ -242,7 +234,7 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
                 if (!FAST) a3 = __builtin_fmaf(f.alpha, depth, a3);
                 alpha_sum += f.alpha;
                 T *= 1.0f - f.alpha;
-            }
+            });
         }
     }
     if (!inside) return;
@@ -307,9 +299,10 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
-// Self-check of the staging cull (tile_stage_load with CULL): every instance of every 8x8 tile is evaluated at all 64
-// pixels with the blend kernels' own cut-off and alpha tests and the outcome is compared with the verdict of the lane
-// that staged it.  counts: instances looked at, instances that reach no pixel, reported misses, wrong misses.
+// Self-check of the staging cull (tile_stage_load with CULL, per quadrant): every instance of every 8x8 tile is evaluated
+// at all 64 pixels with the blend kernels' own cut-off and alpha tests and the outcome is compared, quadrant by quadrant,
+// with the verdict of the lane that staged it.  counts: instances looked at, instances that reach no pixel of the tile,
+// instances left out of all four quadrants, (instance, quadrant) pairs left out although a pixel there is reached.
 template <int MODE>
 __global__ void __launch_bounds__(64) check_tile_cull_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t grid_w,
@@ -317,14 +310,14 @@ __global__ void __launch_bounds__(64) check_tile_cull_kernel(
 {
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x, lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, 0xffffffffu, 0xffffffffu);
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
     unsigned long long seen = 0, empty = 0, missed = 0, wrong = 0;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        const uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const int nb = last - base < 64u ? (int)(last - base) : 64;
         uint32_t addr = stage_address(st);
@@ -335,8 +328,15 @@ __global__ void __launch_bounds__(64) check_tile_cull_kernel(
                 f.den_rcp = rcp_exact(f.den);
                 pass = tile_frag_alpha<MODE>(stage_opacity<64>(addr), f);
             }
-            const bool any = __any(pass), miss = !((hits >> j) & 1);
-            ++seen; empty += !any; missed += miss; wrong += miss && any;
+            const uint64_t reached = __ballot(pass);
+            bool kept = false;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bool keep = (hits.h[q] >> j) & 1;
+                kept = kept || keep;
+                wrong += !keep && ((reached >> (16 * q)) & 0xffffu) != 0;
+            }
+            ++seen; empty += reached == 0; missed += !kept;
         }
     }
     if (lane == 0 && seen) {

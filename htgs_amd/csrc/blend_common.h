@@ -292,9 +292,12 @@ __device__ __forceinline__ bool quadrant_pending(const QuadrantHits &w) { return
 __device__ __forceinline__ uint32_t quadrant_next_hit(QuadrantHits &w)
 {
     uint32_t a0, a1, a2, a3, addr, t;
+    // (two statements: one with scalar results only, which the compiler then knows to be wave-uniform)
     asm volatile("s_ff1_i32_b64 %[a0], %[h0]\n\ts_ff1_i32_b64 %[a1], %[h1]\n\ts_ff1_i32_b64 %[a2], %[h2]\n\ts_ff1_i32_b64 %[a3], %[h3]\n\t"
-                 "s_bitset0_b64 %[h0], %[a0]\n\ts_bitset0_b64 %[h1], %[a1]\n\ts_bitset0_b64 %[h2], %[a2]\n\ts_bitset0_b64 %[h3], %[a3]\n\t"
-                 "v_mov_b32 %[addr], %[a0]\n\t"
+                 "s_bitset0_b64 %[h0], %[a0]\n\ts_bitset0_b64 %[h1], %[a1]\n\ts_bitset0_b64 %[h2], %[a2]\n\ts_bitset0_b64 %[h3], %[a3]"
+                 : [a0] "=&s"(a0), [a1] "=&s"(a1), [a2] "=&s"(a2), [a3] "=&s"(a3),
+                   [h0] "+s"(w.h[0]), [h1] "+s"(w.h[1]), [h2] "+s"(w.h[2]), [h3] "+s"(w.h[3]));
+    asm volatile("v_mov_b32 %[addr], %[a0]\n\t"
                  "v_mov_b32 %[t], %[a1]\n\t"
                  "s_nop 1\n\t"
                  "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x2 bank_mask:0xf\n\t"
@@ -305,10 +308,28 @@ __device__ __forceinline__ uint32_t quadrant_next_hit(QuadrantHits &w)
                  "s_nop 1\n\t"
                  "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x8 bank_mask:0xf\n\t"
                  "v_lshlrev_b32 %[addr], 4, %[addr]"
-                 : [a0] "=&s"(a0), [a1] "=&s"(a1), [a2] "=&s"(a2), [a3] "=&s"(a3), [addr] "=&v"(addr), [t] "=&v"(t),
-                   [h0] "+s"(w.h[0]), [h1] "+s"(w.h[1]), [h2] "+s"(w.h[2]), [h3] "+s"(w.h[3]));
+                 : [addr] "=&v"(addr), [t] "=&v"(t)
+                 : [a0] "s"(a0), [a1] "s"(a1), [a2] "s"(a2), [a3] "s"(a3));
     return addr;
 }
+// The walk itself: turn(addr) is called, with the lanes of the quadrants that still have a hit, once per loop turn.
+template <typename Turn>
+__device__ __forceinline__ void quadrant_walk(QuadrantHits &hits, uint32_t stage_base, Turn &&turn)
+{
+    // (the exit is taken from the scalar masks, not from the lanes' addresses: an exit test that the optimizer can fold
+    // into the per-lane test below makes the loop, and the masks it carries, divergent in the compiler's eyes)
+    while (quadrant_pending(hits)) {
+        const uint32_t addr = quadrant_next_hit(hits);
+        if (addr != kNoHit) turn(addr + stage_base);
+    }
+}
+// pixel of a lane in an 8x8 tile that is walked by quadrants
+struct TilePixel {
+    uint32_t x, y;
+    bool inside;
+    PixelTerms pt;
+    float cx, cy;
+};
 template <int N, int ROW>
 __device__ __forceinline__ float4 stage_row(uint32_t addr)
 {
@@ -411,6 +432,21 @@ __device__ __forceinline__ void core_exchange_walk(float &depth, float &alpha, I
             for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) exchange_step(depth, alpha, index, cd[i], ca[i], ci[i], all);
         }
     }
+}
+
+__device__ __forceinline__ TilePixel quadrant_tile_pixel(uint32_t tile, uint32_t grid_w, uint32_t lane, uint32_t width, uint32_t height)
+{
+    TilePixel p;
+    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
+    uint32_t local_x, local_y;
+    quadrant_pixel(lane, local_x, local_y);
+    p.x = x0 + local_x;
+    p.y = y0 + local_y;
+    p.inside = p.x < width && p.y < height;
+    p.pt = pixel_terms(local_x, local_y, 8);
+    p.cx = tile_centre(x0, 8);
+    p.cy = tile_centre(y0, 8);
+    return p;
 }
 
 }  // namespace htgs

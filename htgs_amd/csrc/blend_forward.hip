@@ -26,11 +26,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const uint32_t x = px.x, y = px.y;
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
 
     float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f;
     // slots hold depth, alpha and index; colours are fetched at the end and the core's share of the colour sums is
@@ -38,21 +38,23 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     float c3[K], cd[K];
     uint32_t ci[K];
 #pragma unroll
-    for (int i = 0; i < K; ++i) { c3[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+    for (int i = 0; i < K; ++i) {
+        c3[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu;
+        asm volatile("" : "+v"(cd[i]), "+v"(c3[i]), "+v"(ci[i]));      // one register per slot
+    }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        while (hits) {
-            const uint32_t addr = stage_next_hit(hits, stage_base);
+        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
             TileFrag f;
-            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+            const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
             f.den_rcp = rcp_exact(f.den);
             const float4 col = stage_row<64, 5>(addr);
-            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+            if (!(tile_frag_alpha<MODE>(stage_opacity<64>(addr), f) && in_reach)) return;
             float depth = tile_frag_depth<64>(addr, pt, f);
             float p3 = f.alpha;
             tail0 = __builtin_fmaf(p3, col.x, tail0);
@@ -64,7 +66,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             }
             tail3 += p3;
             T_tail *= 1.0f - p3;
-        }
+        });
     }
     if (!inside) return;
 
@@ -141,35 +143,37 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const uint32_t x = px.x, y = px.y;
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
 
     float ca[K], cd[K];
     uint32_t ci[K];
 #pragma unroll
-    for (int i = 0; i < K; ++i) { ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+    for (int i = 0; i < K; ++i) {
+        ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu;
+        asm volatile("" : "+v"(cd[i]), "+v"(ca[i]), "+v"(ci[i]));      // one register per slot
+    }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, true, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        while (hits) {
-            const uint32_t addr = stage_next_hit(hits, stage_base);
+        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
             TileFrag f;
-            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+            const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
             f.den_rcp = rcp_exact(f.den);
             float depth = tile_frag_depth<64>(addr, pt, f);
-            if (depth >= cd[K - 1]) continue;
-            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+            if (!(in_reach && depth < cd[K - 1])) return;
+            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) return;
             float alpha = f.alpha;
             uint32_t idx = stage_index<64>(addr);
             core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
-        }
+        });
     }
     if (!inside) return;
 
@@ -224,32 +228,31 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const uint32_t x = px.x, y = px.y;
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        while (hits) {
-            const uint32_t addr = stage_next_hit(hits, stage_base);
+        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
             TileFrag f;
-            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+            const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
             f.den_rcp = rcp_exact(f.den);
             const float4 col = stage_row<64, 5>(addr);
-            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+            if (!(tile_frag_alpha<MODE>(stage_opacity<64>(addr), f) && in_reach)) return;
             a0 = __builtin_fmaf(f.alpha, col.x, a0);
             a1 = __builtin_fmaf(f.alpha, col.y, a1);
             a2 = __builtin_fmaf(f.alpha, col.z, a2);
             alpha_sum += f.alpha;
             T *= 1.0f - f.alpha;
-        }
+        });
     }
     if (!inside) return;
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;

@@ -27,35 +27,36 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     __shared__ TileStage<64> st;
     const uint32_t tile = blockIdx.x;
     const uint32_t lane = threadIdx.x;
-    const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
-    const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
-    const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(lane & 7, lane >> 3, 8);
-    const float cx = tile_centre(x0, 8), cy = tile_centre(y0, 8);
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    const bool inside = px.inside;
+    const PixelTerms pt = px.pt;
+    const float cx = px.cx, cy = px.cy;
 
     float alpha_sum = 0.0f, T_tail = 1.0f;
     float ca[KS], cd[KS];
     uint32_t ci[KS];
 #pragma unroll
-    for (int i = 0; i < KS; ++i) { ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu; }
+    for (int i = 0; i < KS; ++i) {
+        ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu;
+        asm volatile("" : "+v"(cd[i]), "+v"(ca[i]), "+v"(ci[i]));      // one register per slot
+    }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, kCore, kCullAlpha>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, kCore, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        while (hits) {
-            const uint32_t addr = stage_next_hit(hits, stage_base);
+        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
             TileFrag f;
-            if (!tile_frag_cutoff<64>(addr, pt, f)) continue;
+            bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
             f.den_rcp = rcp_exact(f.den);
             float depth = 0.0f;
             if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
                 depth = tile_frag_depth<64>(addr, pt, f);
-                if (depth >= cd[KS - 1]) continue;
+                in_reach = in_reach && depth < cd[KS - 1];
             }
-            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) continue;
+            if (!(tile_frag_alpha<MODE>(stage_opacity<64>(addr), f) && in_reach)) return;
             float alpha = f.alpha;
             if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth<64>(addr, pt, f);
             if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
@@ -63,7 +64,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 core_exchange_walk<KS>(depth, alpha, idx, cd, ca, ci);
             }
             if (kTail) { alpha_sum += alpha; T_tail *= 1.0f - alpha; }
-        }
+        });
     }
     float T_core = 1.0f;
     if (kCore && inside) {
@@ -84,18 +85,17 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     // threshold here, R/include/hybrid_blend/kernels/update_max_weights.cuh:197-204)
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        uint64_t hits = __ballot(tile_stage_load<MODE, 64, false, kCullCutoff>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullCutoff, true>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        while (hits) {
-            const uint32_t addr = stage_next_hit(hits, stage_base);
+        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
             TileFrag f;
-            if (!active || !tile_frag_cutoff<64>(addr, pt, f)) continue;
+            if (!active || !tile_frag_cutoff<64>(addr, pt, f)) return;
             const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * rcp_exact(f.den));
             const float a = stage_opacity<64>(addr) * G;
             const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
             if (!(w < weight_threshold)) raise_max(max_weights, stage_index<64>(addr), w);
-        }
+        });
     }
 }
 
