@@ -25,16 +25,29 @@ constexpr int kSortTileMin = 256 * kSortItems;              // sizes the histogr
 template <typename KeyT>
 __device__ __forceinline__ uint32_t digit_of(KeyT k, int shift, uint32_t mask) { return (uint32_t)(k >> shift) & mask; }
 
+// Workgroups go round the eight XCDs of the device in launch order, and each XCD has an L2 of its own.  Blocks that are
+// neighbours in the input write neighbouring runs of every digit, a run being shorter than a cache line or two; handing
+// every XCD a contiguous eighth of the input lets those partial lines meet in one L2 before they are written back.
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t launched, uint32_t n_blocks)
+{
+    const uint32_t per_xcd = (n_blocks + kXcds - 1) / kXcds;
+    return (launched % kXcds) * per_xcd + launched / kXcds;           // >= n_blocks: nothing to do
+}
+inline uint32_t xcd_padded_grid(uint32_t n_blocks) { return (n_blocks + kXcds - 1) / kXcds * kXcds; }
+
 template <typename KeyT>
 __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
                                                                                  uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
     constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems;
     __shared__ uint32_t counts[kRadix];
+    const uint32_t block = xcd_contiguous_block(blockIdx.x, n_blocks);
+    if (block >= n_blocks) return;
     if (threadIdx.x < kRadix) counts[threadIdx.x] = 0;
     __syncthreads();
     // the order of the keys does not matter here, so every thread reads 16-byte words: kPer keys at a time
-    const uint64_t base = (uint64_t)blockIdx.x * kSortTile;
+    const uint64_t base = (uint64_t)block * kSortTile;
     constexpr int kPer = 16 / sizeof(KeyT);
     if (base + kSortTile <= n) {
         const uint4 *words = reinterpret_cast<const uint4 *>(keys + base);      // kSortTile keys are a multiple of 16 bytes
@@ -54,7 +67,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_histogram_kern
         }
     }
     __syncthreads();
-    if (threadIdx.x < kRadix) hist[(size_t)threadIdx.x * n_blocks + blockIdx.x] = counts[threadIdx.x];
+    if (threadIdx.x < kRadix) hist[(size_t)threadIdx.x * n_blocks + block] = counts[threadIdx.x];
 }
 
 // block d scans row d of hist in place (exclusive) and writes the row total to totals[d]
@@ -109,10 +122,12 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
     KeyT *local_keys = reinterpret_cast<KeyT *>(local_raw);
     uint32_t *local_vals = reinterpret_cast<uint32_t *>(local_raw + (kTwoRounds ? 0 : kSortTile * sizeof(KeyT)));
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const uint32_t block = xcd_contiguous_block(blockIdx.x, n_blocks);
+    if (block >= n_blocks) return;
     for (int c = threadIdx.x; c < kSortWaves * kRadix; c += kSortThreads) (&counts[0][0])[c] = 0;
     __syncthreads();
 
-    const uint64_t block_base = (uint64_t)blockIdx.x * kSortTile;
+    const uint64_t block_base = (uint64_t)block * kSortTile;
     const uint64_t wave_base = block_base + (uint64_t)wave * (kWave * kSortItems);
     KeyT key[kSortItems];
     uint32_t val[kSortItems];
@@ -172,7 +187,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
                 if (w < wave) { before_l += wave_sums[w]; before_g += wave_sums_g[w]; }
             const uint32_t start = before_l + inc_local - block_count;
             digit_start[d] = start;
-            global_base[d] = before_g + inc_global - total + hist[(size_t)d * n_blocks + blockIdx.x];
+            global_base[d] = before_g + inc_global - total + hist[(size_t)d * n_blocks + block];
             uint32_t run = start;
 #pragma unroll
             for (int w = 0; w < kSortWaves; ++w) {
@@ -246,9 +261,9 @@ static int sort_pairs(const htgs_frame *f, int end_bit, int *selector)
         const uint32_t mask = (1u << bits) - 1u;
         const KeyT *kin = (const KeyT *)f->keys[cur];
         KeyT *kout = (KeyT *)f->keys[cur ^ 1];
-        hipLaunchKernelGGL((digit_histogram_kernel<KeyT>), dim3(n_blocks), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
+        hipLaunchKernelGGL((digit_histogram_kernel<KeyT>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
         hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
-        hipLaunchKernelGGL((digit_scatter_kernel<KeyT>), dim3(n_blocks), dim3(kSortThreads), 0, s, kin, f->vals[cur], kout, f->vals[cur ^ 1],
+        hipLaunchKernelGGL((digit_scatter_kernel<KeyT>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, f->vals[cur], kout, f->vals[cur ^ 1],
                            hist, totals, n, n_blocks, shift, mask);
         cur ^= 1;
     }
