@@ -259,7 +259,7 @@ def main():
     n_vis = int((fb.n_touched != 0).sum().item())
     N, P, T = fb.n, fb.width * fb.height, fb.n_tiles
     B, kb = settings.active_sh_bases, fb.key_bytes
-    passes = (fb.end_bit + 7) // 8
+    passes = fb.sort_passes
     # every repetition runs the whole frame in order, so that each stage sees the data (and the caches) it sees
     # in a real frame: a radix sort that is re-run on its own sorted output, say, would look twice as fast
     stage_fns = (("preprocess", fb.preprocess), ("scan", fb.scan), ("create_instances", fb.create_instances),

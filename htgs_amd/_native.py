@@ -81,6 +81,7 @@ SYMBOLS = {
     "htgs_effective_k": (ctypes.c_int, [ctypes.c_int]),
     "htgs_end_bit": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "htgs_key_bytes": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "htgs_sort_passes": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "htgs_scan_tmp_words": (ctypes.c_size_t, [ctypes.c_int]),
     "htgs_sort_tmp_words": (ctypes.c_size_t, [ctypes.c_uint64]),
     "htgs_preprocess": (ctypes.c_int, [_FRAME_P]),

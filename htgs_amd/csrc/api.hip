@@ -78,6 +78,13 @@ extern "C" int htgs_key_bytes(int mode, int width, int height)
     return htgs_end_bit(mode, width, height) <= 16 ? 2 : 4;
 }
 
+extern "C" int htgs_sort_passes(int mode, int width, int height)
+{
+    // 8 bits per pass, 9 for the 8-byte tile|depth keys (radix_sort.hip)
+    const int bits = htgs_key_bytes(mode, width, height) == 8 ? 9 : 8;
+    return (htgs_end_bit(mode, width, height) + bits - 1) / bits;
+}
+
 extern "C" int htgs_render_front(const htgs_frame *f)
 {
     int rc = htgs_preprocess(f);

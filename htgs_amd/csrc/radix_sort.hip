@@ -1,5 +1,5 @@
-// Stable least-significant-digit radix sort of (key, primitive index) pairs, 8 bits per pass, for
-// 16-, 32- and 64-bit keys.  Replaces cub::DeviceRadixSort::SortPairs(begin_bit = 0, end_bit)
+// Stable least-significant-digit radix sort of (key, primitive index) pairs for 16-, 32- and 64-bit keys: 8 bits per pass,
+// 9 bits for the 64-bit tile|depth keys (their 44 or 45 significant bits then take five passes instead of six).  Replaces cub::DeviceRadixSort::SortPairs(begin_bit = 0, end_bit)
 // at R/src/hybrid_blend/inference.cu:145-153 (64-bit tile|depth keys:
 // R/src/alpha_blend_global_ordering/inference.cu:117-124).
 //
@@ -14,8 +14,9 @@
 namespace htgs {
 
 constexpr int kSortItems = 16;                              // rounds per wave
-constexpr int kRadix = 256;
-constexpr int kDigitWaves = kRadix / kWave;                 // the waves whose threads own one digit each
+// digit width per key type; kRadix digits, the first kRadix threads of a block own one digit each
+template <typename KeyT> struct SortDigit { static constexpr int bits = sizeof(KeyT) == 8 ? 9 : 8; };
+constexpr int kMaxRadix = 512;
 constexpr int kScanThreads = 256;
 // Items per block = threads x 16 = 8192.  Longer blocks give longer runs per digit, i.e. fuller cache lines in the
 // scatter; two blocks fit a CU's LDS for every key width (8-byte keys share one array between keys and values).
@@ -40,7 +41,8 @@ template <typename KeyT>
 __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
                                                                                  uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
-    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems;
+    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems, kRadix = 1 << SortDigit<KeyT>::bits;
+    static_assert(kRadix <= kSortThreads, "one thread per digit");
     __shared__ uint32_t counts[kRadix];
     const uint32_t block = xcd_contiguous_block(blockIdx.x, n_blocks);
     if (block >= n_blocks) return;
@@ -109,7 +111,9 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
     const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
     constexpr int kSortThreads = SortShape<KeyT>::threads, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
-    __shared__ uint32_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the wave's base inside the block
+    constexpr int kBits = SortDigit<KeyT>::bits, kRadix = 1 << kBits, kDigitWaves = kRadix / kWave;
+    // (16-bit counters: a block holds 8192 items; with 512 digits and 8-byte keys two blocks still fit a CU's LDS)
+    __shared__ uint16_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the wave's base inside the block
     __shared__ uint32_t digit_start[kRadix];           // first slot of each digit in the block-local order
     __shared__ uint32_t global_base[kRadix];           // where the block's run of each digit starts in the output
     __shared__ uint32_t wave_sums[kDigitWaves], wave_sums_g[kDigitWaves];
@@ -124,7 +128,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const uint32_t block = xcd_contiguous_block(blockIdx.x, n_blocks);
     if (block >= n_blocks) return;
-    for (int c = threadIdx.x; c < kSortWaves * kRadix; c += kSortThreads) (&counts[0][0])[c] = 0;
+    for (int c = threadIdx.x; c < kSortWaves * kRadix / 2; c += kSortThreads) reinterpret_cast<uint32_t *>(&counts[0][0])[c] = 0;
     __syncthreads();
 
     const uint64_t block_base = (uint64_t)block * kSortTile;
@@ -144,7 +148,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
         const uint64_t present = __ballot(valid);
         uint32_t peers_lo = (uint32_t)present, peers_hi = (uint32_t)(present >> 32);
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
+        for (int b = 0; b < kBits; ++b) {
             const uint32_t bit = (uint32_t)__builtin_amdgcn_sbfe((int)d, b, 1);
             const uint64_t vote = __ballot(bit != 0u);
             peers_lo &= ~((uint32_t)vote ^ bit);
@@ -154,7 +158,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
         uint32_t seen = 0;
         if (valid) {
             seen = counts[wave][d];
-            if (below == 0) counts[wave][d] = seen + (uint32_t)(__builtin_popcount(peers_lo) + __builtin_popcount(peers_hi));
+            if (below == 0) counts[wave][d] = (uint16_t)(seen + (uint32_t)(__builtin_popcount(peers_lo) + __builtin_popcount(peers_hi)));
         }
         rank[r] = seen + below;
     }
@@ -192,7 +196,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
 #pragma unroll
             for (int w = 0; w < kSortWaves; ++w) {
                 const uint32_t c = counts[w][d];
-                counts[w][d] = run;
+                counts[w][d] = (uint16_t)run;
                 run += c;
             }
         }
@@ -212,9 +216,9 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
     __syncthreads();
     // ... then stream them out: neighbouring threads write neighbouring addresses inside each digit's run
     const uint32_t n_local = n - block_base < (uint64_t)kSortTile ? (uint32_t)(n - block_base) : (uint32_t)kSortTile;
-    uint32_t digits[kSortItems / 4];           // two rounds: the digits, four to a register, for the values' turn
+    uint32_t digits[kSortItems / 2];           // two rounds: the digits, two to a register, for the values' turn
 #pragma unroll
-    for (int r = 0; r < kSortItems / 4; ++r) digits[r] = 0u;
+    for (int r = 0; r < kSortItems / 2; ++r) digits[r] = 0u;
 #pragma unroll
     for (int r = 0; r < kSortItems; ++r) {
         const uint32_t i = (uint32_t)r * kSortThreads + threadIdx.x;
@@ -223,7 +227,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
             const uint32_t d = digit_of(k, shift, mask);
             const uint32_t pos = global_base[d] + (i - digit_start[d]);
             keys_out[pos] = k;
-            if (kTwoRounds) digits[r / 4] |= d << (8 * (r % 4));
+            if (kTwoRounds) digits[r / 2] |= d << (16 * (r % 2));
             else vals_out[pos] = local_vals[i];
         }
     }
@@ -239,7 +243,7 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
         for (int r = 0; r < kSortItems; ++r) {
             const uint32_t i = (uint32_t)r * kSortThreads + threadIdx.x;
             if (i < n_local) {
-                const uint32_t d = (digits[r / 4] >> (8 * (r % 4))) & 0xffu;
+                const uint32_t d = digits[r / 2] >> (16 * (r % 2)) & 0xffffu;
                 vals_out[global_base[d] + (i - digit_start[d])] = local_vals[i];
             }
         }
@@ -253,11 +257,12 @@ static int sort_pairs(const htgs_frame *f, int end_bit, int *selector)
     constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems;
     const uint64_t n = f->n_instances;
     const uint32_t n_blocks = (uint32_t)((n + kSortTile - 1) / kSortTile);
+    constexpr int kBits = SortDigit<KeyT>::bits, kRadix = 1 << kBits;
     uint32_t *hist = f->sort_tmp;
     uint32_t *totals = f->sort_tmp + (size_t)kRadix * n_blocks;
     int cur = 0;
-    for (int shift = 0; shift < end_bit; shift += 8) {
-        const int bits = end_bit - shift < 8 ? end_bit - shift : 8;
+    for (int shift = 0; shift < end_bit; shift += kBits) {
+        const int bits = end_bit - shift < kBits ? end_bit - shift : kBits;
         const uint32_t mask = (1u << bits) - 1u;
         const KeyT *kin = (const KeyT *)f->keys[cur];
         KeyT *kout = (KeyT *)f->keys[cur ^ 1];
@@ -278,7 +283,8 @@ using namespace htgs;
 extern "C" size_t htgs_sort_tmp_words(uint64_t n_instances)
 {
     const uint64_t n_blocks = (n_instances + kSortTileMin - 1) / kSortTileMin;
-    return (size_t)(kRadix * (n_blocks > 0 ? n_blocks : 1) + kRadix);
+    // (256 digits x blocks of half the real size = 512 digits x real blocks: either digit width fits)
+    return (size_t)(256 * (n_blocks > 0 ? n_blocks : 1) + 2 * kMaxRadix);
 }
 
 extern "C" int htgs_sort_instances(const htgs_frame *f, int *selector)

@@ -154,6 +154,7 @@ class FrameBuffers:
         self.n_tiles = self.grid_w * self.grid_h
         self.key_bytes = self.lib.htgs_key_bytes(mode, self.width, self.height)
         self.end_bit = self.lib.htgs_end_bit(mode, self.width, self.height)
+        self.sort_passes = self.lib.htgs_sort_passes(mode, self.width, self.height)
         self.to_chw = bool(to_chw)
 
         self.pool = pool
@@ -249,7 +250,7 @@ class FrameBuffers:
 
     def back(self):
         _native.check(self.lib.htgs_render_back(self._ref))
-        self.selector = ((self.end_bit + 7) // 8) & 1 if self.n_instances > 0 else 0
+        self.selector = self.sort_passes & 1 if self.n_instances > 0 else 0
 
     def run(self):
         self.front()

@@ -117,6 +117,8 @@ int htgs_effective_k(int K);
 int htgs_end_bit(int mode, int width, int height);
 /* 2, 4 or 8: ushort / uint / uint64_t keys (R/src/hybrid_blend/inference.cu:121-129) */
 int htgs_key_bytes(int mode, int width, int height);
+/* digit passes htgs_sort_instances takes (8 bits per pass, 9 for 8-byte keys); the sorted pairs end up in keys/vals[passes & 1] */
+int htgs_sort_passes(int mode, int width, int height);
 size_t htgs_scan_tmp_words(int n_primitives);
 size_t htgs_sort_tmp_words(uint64_t n_instances);
 
