@@ -45,6 +45,8 @@ class Frame(ctypes.Structure):
         ("scan_tmp", ctypes.c_void_p),
         ("n_instances_dev", ctypes.c_void_p),
         ("ranges", ctypes.c_void_p),
+        ("long_tiles", ctypes.c_void_p),
+        ("long_list_threshold", ctypes.c_int32),
         ("n_instances", ctypes.c_uint64),
         ("keys", ctypes.c_void_p * 2),
         ("vals", ctypes.c_void_p * 2),

@@ -27,38 +27,52 @@ __device__ __forceinline__ void store_pixel(float *__restrict__ image, float *__
 // HYBRID_BLEND: K nearest fragments with alpha >= 1/20 are alpha-blended in depth order, everything
 // else is merged order-independently into one tail fragment behind them.
 // ---------------------------------------------------------------------------------------------
-template <int K, bool FAST>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
-    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+// The tail of a pixel: colour sums (every fragment's alpha * colour; the final core's share is taken out when the pixel
+// is composited), alpha sum, depth sum and transmittance of what is not in the core.
+struct HybridTail {
+    float T, c0, c1, c2, alpha, depth;
+};
+__device__ __forceinline__ void hybrid_tail_init(HybridTail &t) { t.T = 1.0f; t.c0 = t.c1 = t.c2 = t.alpha = t.depth = 0.0f; }
+// what joins the tail: a fragment itself, the entry it pushed out of the core, or an empty slot (alpha 0)
+template <bool FAST>
+__device__ __forceinline__ void hybrid_tail_add(HybridTail &t, float depth, float alpha)
 {
-    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
-    __shared__ TileStage<64> st;
-    const uint32_t tile = blockIdx.x;
-    const uint32_t lane = threadIdx.x;
-    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
-    const uint32_t x = px.x, y = px.y;
-    const bool inside = px.inside;
-    const PixelTerms pt = px.pt;
-    const float cx = px.cx, cy = px.cy;
-
-    float T_tail = 1.0f, tail0 = 0.0f, tail1 = 0.0f, tail2 = 0.0f, tail3 = 0.0f, depth_tail = 0.0f;
-    // A core slot holds depth, alpha and the Gaussian's index (an exchange moves three registers); the colours are
-    // fetched once, when the sorted core is blended.  Every fragment's alpha * colour goes into the tail sums when it
-    // is evaluated, and the share of the fragments that end up in the core is taken out again at the end, so an
-    // entry pushed out of the core needs no colour: its alpha and depth, which the tail also needs, are in the slot.
-    float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
+    t.alpha += alpha;
+    if (!FAST) t.depth = __builtin_fmaf(depth, alpha, t.depth);      // (not used for the median depth)
+    t.T *= 1.0f - alpha;
+}
+template <int K>
+__device__ __forceinline__ void hybrid_core_init(float (&cd)[K], float (&ca)[K], float (&ci)[K])
+{
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         cd[i] = __FLT_MAX__; ca[i] = 0.0f; ci[i] = 0.0f;
         asm volatile("" : "+v"(cd[i]), "+v"(ca[i]), "+v"(ci[i]));      // one register per slot, never a 16-wide tuple
     }
+}
 
-    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+// The walk over instances [first, last) of a tile's list (whole batches of 64 from `first` on) by one wave: lanes =
+// pixels, by quadrants.  A core slot holds depth, alpha and the Gaussian's index (an exchange moves three registers); the
+// colours are fetched once, when the sorted core is blended.  Every fragment's alpha * colour goes into the tail sums
+// when it is evaluated, and the share of the fragments that end up in the core is taken out again at the end, so an
+// entry pushed out of the core needs no colour: its alpha and depth, which the tail also needs, are in the slot.
+// SOLO: the wave is the whole workgroup (its barriers are the workgroup's).
+// TIES (the walks of blend_hybrid_long_kernel): `tie` receives the least depth at which an entry was pushed out of the core
+// that is exactly as deep as the entry that is now last.  (A candidate as deep as the last slot of a share's own core
+// needs no note: at least K fragments of the share are not farther and came earlier, so it is in nobody's final core.)
+// PIXELS: only the pixels of the lanes in pixel_lanes are wanted; instances that do not reach one of them are left out
+// (the other lanes' cores and tails come out incomplete).
+template <int K, bool FAST, bool SOLO, bool TIES = false, bool PIXELS = false>
+__device__ __forceinline__ void hybrid_walk(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
+                                            uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K], float (&ca)[K],
+                                            float (&ci)[K], HybridTail &tail, float *tie = nullptr, uint64_t pixel_lanes = 0)
+{
+    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
     for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
+        if (SOLO) __syncthreads(); else wave_lds_sync();
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, PIXELS ? kCullPixels : kCullAlpha, true>(st, prim, inst, base + lane, last, lane,
+                                                                                                                 cx, cy, pixel_lanes));
+        if (SOLO) __syncthreads(); else wave_lds_sync();
         {
             // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
@@ -73,22 +87,29 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach)) return;
                 float depth = tile_frag_depth<64>(addr, pt, f);
                 float p3 = f.alpha;
-                tail0 = __builtin_fmaf(p3, col.x, tail0);
-                tail1 = __builtin_fmaf(p3, col.y, tail1);
-                tail2 = __builtin_fmaf(p3, col.z, tail2);
+                tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
+                tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
+                tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
                 if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
                     float pi = col.w;
                     core_exchange_walk<K>(depth, p3, pi, cd, ca, ci);
+                    if (TIES && p3 > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
                 }
-                // (depth, p3) is the fragment itself, the entry it pushed out of the core, or an empty slot (alpha 0)
-                tail3 += p3;
-                if (!FAST) depth_tail = __builtin_fmaf(depth, p3, depth_tail);      // (not used for the median depth)
-                T_tail *= 1.0f - p3;
+                hybrid_tail_add<FAST>(tail, depth, p3);
             });
         }
     }
-    if (!inside) return;
+}
 
+// core + tail -> pixel (R/include/hybrid_blend/kernels/inference.cuh:172-213)
+template <int K>
+__device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim, float (&cd)[K], float (&ca)[K], float (&ci)[K], HybridTail &tail,
+                                                 float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height,
+                                                 uint32_t x, uint32_t y, int chw, int median)
+{
+    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    float tail0 = tail.c0, tail1 = tail.c1, tail2 = tail.c2;
+    const float tail3 = tail.alpha, depth_tail = tail.depth, T_tail = tail.T;
     float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T_core = 1.0f;
     float4 cc[K];
 #pragma unroll
@@ -125,6 +146,129 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     }
     if (!median) depth_pixel = total_alpha > 0.0f ? depth_pixel / total_alpha : 0.0f;
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
+}
+
+// One wave per tile.  A tile whose list is longer than long_threshold is not walked here but put on the list of long tiles
+// (long_tiles[0] = their number and long_tiles[1] = a work counter, both zeroed with the ranges; long_tiles[2..] = the tiles) for blend_hybrid_long_kernel, if the
+// caller provided that list: one wave walks one tile at some 200 ns per instance once it has a SIMD to itself, so a single
+// list of 300 000 instances would otherwise hold the launch for 70 ms.
+template <int K, bool FAST>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold)
+{
+    __shared__ TileStage<64> st;
+    const uint32_t tile = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    if (long_tiles != nullptr && last - first > long_threshold) {
+        if (lane == 0) long_tiles[2 + atomicAdd(long_tiles, 1u)] = tile;
+        return;
+    }
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    HybridTail tail;
+    hybrid_tail_init(tail);
+    float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
+    hybrid_core_init<K>(cd, ca, ci);
+    hybrid_walk<K, FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
+    if (!px.inside) return;
+    hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+}
+
+// The long tiles: a workgroup of kLongWaves waves takes a tile, every wave walks a contiguous share of the list (whole
+// batches of 64) into a core and a tail of its own, and the shares are then merged into the first wave's, in list
+// order, through LDS: the entries of the incoming core enter the running core like fragments (what does not stay in
+// the core, of either, joins the tail), the tails add up.  The pixel gets the K nearest fragments of the whole list and
+// everything else in its tail, as in a single walk; what differs from the single walk is the order in which the tail's
+// sums are added (rounding) and which of two stored fragments of exactly equal depth is kept when a nearer one arrives.
+constexpr int kLongWaves = 16;
+constexpr uint32_t kLongListDefault = 8192;
+template <int K, bool FAST>
+__global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+{
+    __shared__ TileStage<64> st[kLongWaves];
+    __shared__ float s_merge[3 * K + 7][64];          // one wave's core, tail and least depth of a tie, lane-minor
+    __shared__ uint32_t s_next;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t n_long = long_tiles[0];
+    for (;;) {
+        // the workgroups take the tiles off the list one by one (their lists differ in length by orders of magnitude)
+        __syncthreads();
+        if (threadIdx.x == 0) s_next = atomicAdd(const_cast<uint32_t *>(long_tiles) + 1, 1u);
+        __syncthreads();
+        const uint32_t j = s_next;
+        if (j >= n_long) break;
+        const uint32_t tile = long_tiles[2 + j];
+        const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+        const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+        const uint32_t n_batches = (last - first + 63u) / 64u;
+        const uint32_t seg_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
+        uint32_t seg_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
+        seg_last = seg_last < last ? seg_last : last;
+        constexpr bool kTies = !FAST;
+        HybridTail tail;
+        hybrid_tail_init(tail);
+        float cd[K], ca[K], ci[K];
+        hybrid_core_init<K>(cd, ca, ci);
+        float tie = __FLT_MAX__;                        // least depth at which two fragments of equal depth met at the end of a core
+        hybrid_walk<K, FAST, false, kTies>(st[wave], inst, prim, seg_first, seg_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, &tie);
+        for (uint32_t s = 1; s < (uint32_t)kLongWaves; ++s) {
+            __syncthreads();                               // the buffer is free
+            if (wave == s) {
+#pragma unroll
+                for (int i = 0; i < K; ++i) { s_merge[3 * i][lane] = cd[i]; s_merge[3 * i + 1][lane] = ca[i]; s_merge[3 * i + 2][lane] = ci[i]; }
+                s_merge[3 * K][lane] = tail.T; s_merge[3 * K + 1][lane] = tail.c0; s_merge[3 * K + 2][lane] = tail.c1;
+                s_merge[3 * K + 3][lane] = tail.c2; s_merge[3 * K + 4][lane] = tail.alpha; s_merge[3 * K + 5][lane] = tail.depth;
+                s_merge[3 * K + 6][lane] = tie;
+            }
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int i = 0; i < K; ++i) {
+                    float depth = s_merge[3 * i][lane], alpha = s_merge[3 * i + 1][lane], index = s_merge[3 * i + 2][lane];
+                    if (alpha > 0.0f) {                    // a filled slot
+                        if (kTies && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
+                        if (depth < cd[K - 1]) {
+                            core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
+                            if (kTies && alpha > 0.0f && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
+                        }
+                        hybrid_tail_add<FAST>(tail, depth, alpha);
+                    }
+                }
+                tail.T *= s_merge[3 * K][lane];
+                tail.c0 += s_merge[3 * K + 1][lane]; tail.c1 += s_merge[3 * K + 2][lane]; tail.c2 += s_merge[3 * K + 3][lane];
+                tail.alpha += s_merge[3 * K + 4][lane]; tail.depth += s_merge[3 * K + 5][lane];
+                const float other = s_merge[3 * K + 6][lane];
+                tie = other < tie ? other : tie;
+            }
+        }
+        if (wave == 0) {
+            if (kTies) {
+                // Equal depths matter where they can change the final core: a tie no deeper than its last entry (both
+                // fragments of a deeper tie end in the tail either way), or two equal depths next to each other in it.
+                bool redo = tie <= cd[K - 1];
+#pragma unroll
+                for (int i = 0; i + 1 < K; ++i) redo = redo || (ca[i + 1] > 0.0f && cd[i] == cd[i + 1]);
+                const uint64_t redo_lanes = __ballot(redo);
+                if (redo_lanes != 0) {
+                    // The one case in which the merged walk and the single walk can keep different fragments, or keep them
+                    // in another order: the reference's insertion lets a displaced entry hop over a stored one of exactly
+                    // equal depth.  Such pixels (a handful per frame of very long lists) are walked again in one piece, by
+                    // this wave alone, over the instances that reach them; the others are finished first.
+                    if (px.inside && !redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+                    hybrid_tail_init(tail);
+                    hybrid_core_init<K>(cd, ca, ci);
+                    hybrid_walk<K, FAST, false, false, true>(st[0], inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, nullptr, redo_lanes);
+                    if (px.inside && redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+                    continue;
+                }
+            }
+            if (px.inside) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -348,9 +492,14 @@ __global__ void __launch_bounds__(64) check_tile_cull_kernel(
 template <int K, bool FAST>
 static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
+    const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth);
+                       f->use_median_depth, f->long_tiles, threshold);
+    if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
+        hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
+                           f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
+                           (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
 }
 template <int K, bool FAST>
 static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)

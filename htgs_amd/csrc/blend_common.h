@@ -158,11 +158,46 @@ __device__ __forceinline__ uint32_t tile_quadrant_hits(const float (&n)[6], cons
 // loaded slot unless CULL asks for tile_misses -- for walks that apply the cut-off and the alpha threshold
 // (kCullAlpha), or the cut-off alone (kCullCutoff: the test with opacity 1).  What that leaves out contributes to
 // no pixel, so a walk over the hits alone gives the results of the full walk bit for bit.
-enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2 };
+// the pixel's offset from the tile centre (exact)
+struct PixelTerms {
+    float X, Y;
+};
+__device__ __forceinline__ PixelTerms pixel_terms(uint32_t local_x, uint32_t local_y, int tile)
+{
+    PixelTerms p;
+    p.X = (float)local_x - 0.5f * (float)(tile - 1);
+    p.Y = (float)local_y - 0.5f * (float)(tile - 1);
+    return p;
+}
+__device__ __forceinline__ float tile_centre(uint32_t first_pixel, int tile) { return (float)first_pixel + 0.5f * (float)(tile - 1); }
+
+__device__ __forceinline__ float quad_eval(float c0, float cx, float cy, float cxx, float cxy, float cyy, const PixelTerms &p)
+{
+    const float tx = __builtin_fmaf(cxy, p.Y, __builtin_fmaf(cxx, p.X, cx));
+    const float ty = __builtin_fmaf(cyy, p.Y, cy);
+    return __builtin_fmaf(p.Y, ty, __builtin_fmaf(p.X, tx, c0));
+}
+
+// lane -> pixel of the quadrant walk (below): lanes 16 q .. 16 q + 15 hold the 4x4 pixels of quadrant q
+__device__ __forceinline__ void quadrant_pixel(uint32_t lane, uint32_t &local_x, uint32_t &local_y)
+{
+    local_x = ((lane >> 4) & 1) * 4 + (lane & 3);
+    local_y = (lane >> 5) * 4 + ((lane >> 2) & 3);
+}
+
+// kCullPixels: a slot counts for a quadrant when the instance passes the cut-off -- with the walk's own arithmetic -- at
+// one of the pixels named by pixel_lanes (a wave-uniform mask over the lanes of the quadrant walk) that lie in it.
+enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2, kCullPixels = 3 };
+
 // With QUADRANTS the result has one bit per 4x4 quadrant of the tile (tile_quadrant_hits) instead of one for the tile.
 template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
-                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy)
+                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes = 0);
+
+// (PixelTerms is complete by the time the template is instantiated)
+template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS>
+__device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
+                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes)
 {
     if (fetch >= last) return 0;
     const uint32_t g = inst[fetch];
@@ -215,28 +250,21 @@ __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const floa
     st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
     st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
     if constexpr (CULL == kCullNone) return QUADRANTS ? 0xfu : 1u;
+    else if constexpr (CULL == kCullPixels) {
+        static_assert(QUADRANTS, "per quadrant");
+        uint32_t bits = 0;
+        for (uint64_t m = pixel_lanes; m != 0; m &= m - 1) {      // (wave-uniform)
+            const uint32_t p = (uint32_t)__builtin_ctzll(m);
+            uint32_t local_x, local_y;
+            quadrant_pixel(p, local_x, local_y);
+            const PixelTerms pt = pixel_terms(local_x, local_y, 8);
+            const float num = quad_eval(n[0], n[1], n[2], n[3], n[4], n[5], pt), den = quad_eval(d[0], d[1], d[2], d[3], d[4], d[5], pt);
+            if (!(num > den)) bits |= 1u << (p >> 4);
+        }
+        return bits;
+    }
     else if constexpr (QUADRANTS) return tile_quadrant_hits<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
     else return (uint32_t)!tile_misses<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
-}
-
-// the pixel's offset from the tile centre (exact)
-struct PixelTerms {
-    float X, Y;
-};
-__device__ __forceinline__ PixelTerms pixel_terms(uint32_t local_x, uint32_t local_y, int tile)
-{
-    PixelTerms p;
-    p.X = (float)local_x - 0.5f * (float)(tile - 1);
-    p.Y = (float)local_y - 0.5f * (float)(tile - 1);
-    return p;
-}
-__device__ __forceinline__ float tile_centre(uint32_t first_pixel, int tile) { return (float)first_pixel + 0.5f * (float)(tile - 1); }
-
-__device__ __forceinline__ float quad_eval(float c0, float cx, float cy, float cxx, float cxy, float cyy, const PixelTerms &p)
-{
-    const float tx = __builtin_fmaf(cxy, p.Y, __builtin_fmaf(cxx, p.X, cx));
-    const float ty = __builtin_fmaf(cyy, p.Y, cy);
-    return __builtin_fmaf(p.Y, ty, __builtin_fmaf(p.X, tx, c0));
 }
 
 struct TileFrag {
@@ -271,11 +299,6 @@ constexpr uint32_t kNoHit = 0xfffffff0u;           // 16 * s_ff1(0): the address
 struct QuadrantHits {
     uint64_t h[4];
 };
-__device__ __forceinline__ void quadrant_pixel(uint32_t lane, uint32_t &local_x, uint32_t &local_y)
-{
-    local_x = ((lane >> 4) & 1) * 4 + (lane & 3);
-    local_y = (lane >> 5) * 4 + ((lane >> 2) & 3);
-}
 __device__ __forceinline__ QuadrantHits quadrant_ballot(uint32_t bits)
 {
     QuadrantHits w;
@@ -311,6 +334,14 @@ __device__ __forceinline__ uint32_t quadrant_next_hit(QuadrantHits &w)
                  : [addr] "=&v"(addr), [t] "=&v"(t)
                  : [a0] "s"(a0), [a1] "s"(a1), [a2] "s"(a2), [a3] "s"(a3));
     return addr;
+}
+// orders one wave's LDS writes before its later LDS reads (the LDS serves a wave's instructions in order; this only keeps
+// the compiler from moving them)
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 // The walk itself: turn(addr) is called, with the lanes of the quadrants that still have a hit, once per loop turn.
 template <typename Turn>

@@ -202,10 +202,12 @@ __global__ void __launch_bounds__(256) extract_ranges_kernel(const KeyT *__restr
     }
 }
 
-__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n)
+// zeroes p[0, n) and, if given, the two words at `also`
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n, uint32_t *also)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = 0;
+    if (i < 2 && also) also[i] = 0;
 }
 
 // Scratch of htgs_scan_offsets_static: the per-block sums of the scan, held in the library's own device image so
@@ -322,7 +324,7 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
     hipStream_t s = (hipStream_t)f->stream;
     const int tile = tile_size(f->mode);
     const size_t n_tiles = (size_t)div_up(f->width, tile) * div_up(f->height, tile);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((2 * n_tiles + 255) / 256)), dim3(256), 0, s, f->ranges, 2 * n_tiles);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((2 * n_tiles + 255) / 256)), dim3(256), 0, s, f->ranges, 2 * n_tiles, f->long_tiles);
     if (f->n_instances > 0) {
         if (!f->keys[selector]) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: null pointer");
         if ((uintptr_t)f->keys[selector] & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: keys must be 16-byte aligned");

@@ -70,6 +70,11 @@ typedef struct htgs_frame {
     uint32_t *n_instances_dev; /* [1] total number of instances, written by the scan */
     /* ---- per-tile scratch (PerTileBuffers, buffer_utils.h:86-94) ---- */
     uint32_t *ranges;          /* [n_tiles,2] first,last+1 into the sorted instance list */
+    uint32_t *long_tiles;      /* [2 + n_tiles] or NULL.  HYBRID_BLEND inference: tiles whose list is longer than
+                                  long_list_threshold are collected here (words 0 and 1: their number and a work
+                                  counter, zeroed by htgs_extract_ranges) and walked by several waves each, see htgs_blend.  NULL: every
+                                  tile is walked by one wave (no counterpart in the reference, which does that) */
+    int32_t long_list_threshold; /* 0 = the default (8192 instances) */
     /* ---- per-instance scratch (PerInstanceBuffers, buffer_utils.h:56-84) ---- */
     uint64_t n_instances;      /* host copy of *n_instances_dev, needed from htgs_create_instances on */
     void *keys[2];             /* [n_instances] of htgs_key_bytes() each, ping-pong, 16-byte aligned */
