@@ -187,11 +187,14 @@ constexpr uint32_t kLongListDefault = 8192;
 template <int K, bool FAST>
 __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
+    uint32_t *__restrict__ shortlist)
 {
     __shared__ TileStage<64> st[kLongWaves];
     __shared__ float s_merge[3 * K + 7][64];          // one wave's core, tail and least depth of a tie, lane-minor
     __shared__ uint32_t s_next;
+    __shared__ uint32_t s_redo[2];                    // the pixels (lanes) to walk again
+    __shared__ uint32_t s_short[kLongWaves];          // how many instances of each share reach one of them
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t n_long = long_tiles[0];
     for (;;) {
@@ -245,29 +248,57 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                 tie = other < tie ? other : tie;
             }
         }
-        if (wave == 0) {
-            if (kTies) {
-                // Equal depths matter where they can change the final core: a tie no deeper than its last entry (both
-                // fragments of a deeper tie end in the tail either way), or two equal depths next to each other in it.
-                bool redo = tie <= cd[K - 1];
+        if (kTies) {
+            // Equal depths matter where they can change the final core: a tie no deeper than its last entry (both
+            // fragments of a deeper tie end in the tail either way), or two equal depths next to each other in it.
+            // There the merged walk and the single walk can keep different fragments, or keep them in another order: the
+            // reference's insertion lets a displaced entry hop over a stored one of exactly equal depth.  Such pixels (a
+            // handful per frame of very long lists) are walked again in one piece by the first wave, over the instances
+            // that reach one of them; every wave picks those out of its share first (into the tile's own stretch of the
+            // shortlist, in list order), since the walk of one wave alone is bound by the latency of staging.
+            bool redo = false;
+            if (wave == 0) {
+                redo = tie <= cd[K - 1];
 #pragma unroll
                 for (int i = 0; i + 1 < K; ++i) redo = redo || (ca[i + 1] > 0.0f && cd[i] == cd[i + 1]);
-                const uint64_t redo_lanes = __ballot(redo);
-                if (redo_lanes != 0) {
-                    // The one case in which the merged walk and the single walk can keep different fragments, or keep them
-                    // in another order: the reference's insertion lets a displaced entry hop over a stored one of exactly
-                    // equal depth.  Such pixels (a handful per frame of very long lists) are walked again in one piece, by
-                    // this wave alone, over the instances that reach them; the others are finished first.
+                const uint64_t lanes = __ballot(redo);
+                if (lane == 0) { s_redo[0] = (uint32_t)lanes; s_redo[1] = (uint32_t)(lanes >> 32); }
+            }
+            __syncthreads();
+            const uint64_t redo_lanes = (uint64_t)s_redo[0] | (uint64_t)s_redo[1] << 32;
+            if (redo_lanes != 0) {
+                if (shortlist != nullptr) {
+                    uint32_t kept = 0;
+                    for (uint32_t base = seg_first; base < seg_last; base += 64) {
+                        const uint32_t fetch = base + lane;
+                        const bool reaches = tile_stage_load<HTGS_MODE_HYBRID_BLEND, 64, true, kCullPixels, true>(st[wave], prim, inst, fetch, seg_last, lane,
+                                                                                                               px.cx, px.cy, redo_lanes) != 0;
+                        const uint64_t keep = __ballot(reaches);
+                        if (reaches) shortlist[seg_first + kept + (uint32_t)__popcll(keep & ((1ull << lane) - 1ull))] = inst[fetch];
+                        kept += (uint32_t)__popcll(keep);
+                    }
+                    if (lane == 0) s_short[wave] = kept;
+                    __syncthreads();
+                }
+                if (wave == 0) {
                     if (px.inside && !redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
                     hybrid_tail_init(tail);
                     hybrid_core_init<K>(cd, ca, ci);
-                    hybrid_walk<K, FAST, false, false, true>(st[0], inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, nullptr, redo_lanes);
+                    if (shortlist != nullptr) {
+                        for (uint32_t s = 0; s < (uint32_t)kLongWaves; ++s) {
+                            const uint32_t from = first + 64u * (uint32_t)((uint64_t)n_batches * s / kLongWaves);
+                            hybrid_walk<K, FAST, false, false, true>(st[0], shortlist, prim, from, from + s_short[s], lane, px.pt, px.cx, px.cy, cd, ca, ci,
+                                                                     tail, nullptr, redo_lanes);
+                        }
+                    } else {
+                        hybrid_walk<K, FAST, false, false, true>(st[0], inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, nullptr, redo_lanes);
+                    }
                     if (px.inside && redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
-                    continue;
                 }
+                continue;
             }
-            if (px.inside) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
         }
+        if (wave == 0 && px.inside) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
     }
 }
 
@@ -499,7 +530,7 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
     if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
         hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
-                           (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+                           (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->vals[selector ^ 1]);
 }
 template <int K, bool FAST>
 static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)

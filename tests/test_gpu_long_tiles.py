@@ -1,0 +1,92 @@
+"""The second HYBRID inference kernel, which takes the tiles whose lists are longer than ``long_list_threshold``: a
+workgroup of waves splits the list, the K-buffers and tails are merged, and pixels at which fragments of exactly equal
+depth met are walked again in one piece.  The threshold is forced down so that small scenes go through it; the result
+must stay within the rasterizer's 1e-4 of the CPU oracle (whose walk is the reference's single one,
+R/include/hybrid_blend/kernels/inference.cuh:70-213) and close to this library's own single-wave kernel."""
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+from htgs_amd.synthetic import make_scene
+from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode
+from util import oracle_render
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4
+NEVER = 2 ** 31 - 1
+
+
+def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False):
+    fb = FrameBuffers(*scene_gpu.gaussians(), scene_gpu.settings(RasterizerMode.HYBRID_BLEND, K), to_chw, median, fast=fast,
+                      long_list_threshold=threshold)
+    fb.run()
+    torch.cuda.synchronize()
+    long_tiles, taken = (int(v) for v in fb.long_tiles[:2].cpu())
+    assert taken >= long_tiles                    # every listed tile was taken off the list
+    depth = None if fast else fb.depth.cpu().numpy()
+    return fb.image.cpu().numpy(), depth, long_tiles
+
+
+def with_coincident_copies(scene, copies):
+    """Every Gaussian ``copies`` times at the same place with the same shape (so every fragment meets fragments of
+    exactly its own depth at every pixel) but other colours and opacities."""
+    g = torch.Generator().manual_seed(11)
+    rep = lambda t: t.repeat(copies, *([1] * (t.dim() - 1))).contiguous()
+    n = scene.positions.shape[0] * copies
+    return dataclasses.replace(
+        scene, name=scene.name + "-coincident", positions=rep(scene.positions), scales=rep(scene.scales), rotations=rep(scene.rotations),
+        opacities=(rep(scene.opacities) + 0.5 * torch.randn(n, *scene.opacities.shape[1:], generator=g)).contiguous(),
+        sh_0=(rep(scene.sh_0) + 0.3 * torch.randn(n, *scene.sh_0.shape[1:], generator=g)).contiguous(), sh_rest=rep(scene.sh_rest))
+
+
+@pytest.mark.parametrize("config,n,K,threshold", [(0, 3000, 4, 64), (0, 3000, 1, 24), (1, 60_000, 16, 16), (2, 100_000, 32, 20),
+                                                    (3, 150_000, 16, 1000)])
+def test_long_tiles_against_oracle(cuda, config, n, K, threshold):
+    print(f"case config={config} n={n} K={K} threshold={threshold}", flush=True)
+    scene = make_scene(config, n)
+    ref = oracle_render(scene, 0, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, threshold)
+    single, single_depth, none = render(scene.to(cuda), K, NEVER)
+    assert long_tiles > 0 and none == 0
+    err = [float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max()),
+           float(np.abs(image - single).max()), float(np.abs(depth - single_depth).max())]
+    print(f"  long tiles {long_tiles}; against the oracle {err[0]:.3g} / {err[1]:.3g}, against the single walk {err[2]:.3g} / {err[3]:.3g}", flush=True)
+    assert max(err) <= TOL
+
+
+@pytest.mark.parametrize("to_chw,median", [(False, False), (True, True), (False, True)])
+def test_long_tiles_layout_and_median_depth(cuda, to_chw, median):
+    print(f"case to_chw={to_chw} median={median}", flush=True)
+    scene = make_scene(0, 3000)
+    ref = oracle_render(scene, 0, 4, to_chw=to_chw, median=median)
+    image, depth, long_tiles = render(scene.to(cuda), 4, 64, to_chw, median)
+    assert long_tiles > 0 and image.shape == ref["image"].shape
+    assert np.abs(image - ref["image"]).max() <= TOL
+    assert np.abs(depth - ref["depth"]).max() <= TOL
+
+
+@pytest.mark.parametrize("K", [4, 16])
+def test_long_tiles_with_fragments_of_equal_depth(cuda, K):
+    """Coincident Gaussians: which of two stored fragments of equal depth leaves the core depends on the order of arrival in
+    the reference's insertion, so the merged cores are not enough and the pixels are walked again in list order."""
+    print(f"case K={K} (coincident copies)", flush=True)
+    scene = with_coincident_copies(make_scene(0, 1500), 6)
+    ref = oracle_render(scene, 0, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, 64)
+    assert long_tiles > 0
+    err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
+    print(f"  long tiles {long_tiles}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
+    assert err_i <= TOL and err_d <= TOL
+
+
+def test_long_tiles_fast_variant(cuda):
+    """The variant without depth and with the hardware's reciprocal / exponential: same fragments, same sums up to their order."""
+    print("case fast", flush=True)
+    scene = make_scene(1, 60_000).to(cuda)
+    image, _, long_tiles = render(scene, 16, 16, fast=True)
+    single, _, none = render(scene, 16, NEVER, fast=True)
+    assert long_tiles > 0 and none == 0
+    assert np.abs(image - single).max() <= TOL
