@@ -300,6 +300,14 @@ def main():
         "launch_ms": round(blend_avg_ms, 4), "evals_per_launch": tile_px * n_inst,
     }
 
+    if args.mode == 2:
+        # GLOBAL_ORDERING stops a pixel once it is opaque, so the number of evaluations its blend kernel makes depends on
+        # the data and 256 per instance would overstate it; the stage priced here is the sort of the 64-bit keys
+        sort_gbs = algo_bytes["sort"] / 1e9 / (stages["sort"] / 1e3)
+        roofline = {"kernel": "sort (digit_histogram + digit_row_scan + digit_scatter, all passes)", "bound": "hbm", "achieved": round(sort_gbs, 1),
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(sort_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                    "launch_ms": round(stages["sort"], 4)}
+
     # ---- CPU baseline: the C oracle on this box's host cores, one whole frame of the same workload ----
     cpu_baseline = None
     if not args.no_cpu_baseline:

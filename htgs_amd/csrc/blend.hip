@@ -148,8 +148,9 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
+constexpr uint32_t kLongHeader = 4, kLongRounds = 3;
 // One wave per tile.  A tile whose list is longer than long_threshold is not walked here but put on the list of long tiles
-// (long_tiles[0] = their number and long_tiles[1] = a work counter, both zeroed with the ranges; long_tiles[2..] = the tiles) for blend_hybrid_long_kernel, if the
+// (long_tiles[0] = their number, long_tiles[1..3] = work counters, all zeroed with the ranges; long_tiles[4..] = the tiles) for blend_hybrid_long_kernel, if the
 // caller provided that list: one wave walks one tile at some 200 ns per instance once it has a SIMD to itself, so a single
 // list of 300 000 instances would otherwise hold the launch for 70 ms.
 template <int K, bool FAST>
@@ -163,7 +164,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (lane == 0) long_tiles[2 + atomicAdd(long_tiles, 1u)] = tile;
+        if (lane == 0) long_tiles[kLongHeader + atomicAdd(long_tiles, 1u)] = tile;
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -188,7 +189,7 @@ template <int K, bool FAST>
 __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
-    uint32_t *__restrict__ shortlist)
+    uint32_t *__restrict__ shortlist, uint32_t long_threshold)
 {
     __shared__ TileStage<64> st[kLongWaves];
     __shared__ float s_merge[3 * K + 7][64];          // one wave's core, tail and least depth of a tie, lane-minor
@@ -197,14 +198,27 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     __shared__ uint32_t s_short[kLongWaves];          // how many instances of each share reach one of them
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t n_long = long_tiles[0];
+    if (n_long == 0) return;                          // (the ordinary frame)
+    // The workgroups take the tiles off the list one by one, the longest first: the list is gone through kLongRounds times
+    // (a counter per round), and a round takes the tiles of its length class only -- more than 16, more than 4 and up to 4
+    // times the threshold.  The lists differ in length by orders of magnitude, and the launch ends when the workgroup with
+    // the longest one does.
+    uint32_t round = 0;
     for (;;) {
-        // the workgroups take the tiles off the list one by one (their lists differ in length by orders of magnitude)
         __syncthreads();
-        if (threadIdx.x == 0) s_next = atomicAdd(const_cast<uint32_t *>(long_tiles) + 1, 1u);
+        if (threadIdx.x == 0) s_next = atomicAdd(const_cast<uint32_t *>(long_tiles) + 1 + round, 1u);
         __syncthreads();
         const uint32_t j = s_next;
-        if (j >= n_long) break;
-        const uint32_t tile = long_tiles[2 + j];
+        if (j >= n_long) {
+            if (++round == kLongRounds) break;
+            continue;
+        }
+        const uint32_t tile = long_tiles[kLongHeader + j];
+        {
+            const uint32_t length = ranges[2 * tile + 1] - ranges[2 * tile];
+            const uint32_t length_class = length > 16u * long_threshold ? 0u : length > 4u * long_threshold ? 1u : 2u;
+            if (length_class != round) continue;
+        }
         const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
         const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
         const uint32_t n_batches = (last - first + 63u) / 64u;
@@ -530,7 +544,7 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
     if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
         hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
-                           (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->vals[selector ^ 1]);
+                           (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->vals[selector ^ 1], threshold);
 }
 template <int K, bool FAST>
 static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)

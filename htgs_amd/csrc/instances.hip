@@ -202,12 +202,12 @@ __global__ void __launch_bounds__(256) extract_ranges_kernel(const KeyT *__restr
     }
 }
 
-// zeroes p[0, n) and, if given, the two words at `also`
+// zeroes p[0, n) and, if given, the four words at `also`
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n, uint32_t *also)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = 0;
-    if (i < 2 && also) also[i] = 0;
+    if (i < 4 && also) also[i] = 0;
 }
 
 // Scratch of htgs_scan_offsets_static: the per-block sums of the scan, held in the library's own device image so

@@ -25,13 +25,18 @@ COUNTERS_FILE = os.path.join(ROOT, "profiles", "counters.json")
 CAL_KERNEL, CAL_BYTES = "copy_bytes_kernel", 1 << 30
 
 
+def short_name(kernel: str) -> str:
+    """the kernel's name without its argument list (a name may itself begin with a parenthesis: "(anonymous namespace)::")"""
+    return kernel.replace("(anonymous namespace)::", "").split("(")[0].replace("void ", "")
+
+
 def per_kernel_median(db_path: str, counter: str) -> dict:
     """kernel name (without its argument list) -> median over dispatches of the counter summed over its dimensions"""
     db = sqlite3.connect(db_path)
     rows = db.execute("select kernel_name, dispatch_id, value from counters_collection where counter_name = ?", (counter,)).fetchall()
     per_dispatch = collections.defaultdict(float)
     for name, dispatch, value in rows:
-        per_dispatch[(name.split("(")[0].replace("void ", ""), dispatch)] += value
+        per_dispatch[(short_name(name), dispatch)] += value
     per_kernel = collections.defaultdict(list)
     for (name, _), value in per_dispatch.items():
         per_kernel[name].append(value)

@@ -167,7 +167,7 @@ class FrameBuffers:
         self.n_instances_dev = self._scratch("n_instances_dev", 1, torch.int32)    # written by the scan
         self.ranges = self._scratch("ranges", 2 * self.n_tiles, torch.int32)[:2 * self.n_tiles].view(self.n_tiles, 2)
         # HYBRID_BLEND inference: the list of tiles with very long instance lists, which several waves walk together
-        self.long_tiles = self._scratch("long_tiles", self.n_tiles + 2, torch.int32) if mode == 0 and not train else None
+        self.long_tiles = self._scratch("long_tiles", self.n_tiles + 4, torch.int32) if mode == 0 and not train else None
         self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
                                  dtype=torch.float32, device=dev)
         # the image-only fast path (``fast_rasterize``) writes no depth map
