@@ -11,6 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libhtgs_amd.so")
 
 PRIM_FLOATS = 20
+PRIM_FLOATS_TRAIN = 32
 
 c_float_p = ctypes.c_void_p
 
@@ -41,6 +42,7 @@ class Frame(ctypes.Structure):
         ("offsets", ctypes.c_void_p),
         ("bounds", ctypes.c_void_p),
         ("prim", ctypes.c_void_p),
+        ("prim_floats", ctypes.c_int32),
         ("clamp_info", ctypes.c_void_p),
         ("scan_tmp", ctypes.c_void_p),
         ("n_instances_dev", ctypes.c_void_p),

@@ -606,6 +606,7 @@ extern "C" int htgs_blend(const htgs_frame *f, int selector)
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: null frame");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: bad argument");
+    if (frame_prim_floats(f) != HTGS_PRIM_FLOATS) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: the inference kernels read records of HTGS_PRIM_FLOATS floats (prim_floats)");
     if (!f->ranges || !f->image || (!f->depth && !f->fast_math) || (f->n_instances > 0 && (!f->vals[selector] || !f->prim)))
         return fail(HTGS_ERR_ARGUMENT, "htgs_blend: null pointer");
     const int tile = tile_size(f->mode);

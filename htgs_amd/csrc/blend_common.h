@@ -190,18 +190,19 @@ __device__ __forceinline__ void quadrant_pixel(uint32_t lane, uint32_t &local_x,
 enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2, kCullPixels = 3 };
 
 // With QUADRANTS the result has one bit per 4x4 quadrant of the tile (tile_quadrant_hits) instead of one for the tile.
-template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false>
+// REC4: 16-byte words per record of prim (five; eight in training frames).
+template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false, int REC4 = HTGS_PRIM_FLOATS / 4>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                     uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes = 0);
 
 // (PixelTerms is complete by the time the template is instantiated)
-template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS>
+template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS, int REC4>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                     uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes)
 {
     if (fetch >= last) return 0;
     const uint32_t g = inst[fetch];
-    const float4 *rec = prim + (size_t)g * (HTGS_PRIM_FLOATS / 4);
+    const float4 *rec = prim + (size_t)g * REC4;
     // (with CULL the record's colour row is fetched when it is needed, behind a compiler fence: it comes from a cache
     // line the other rows have just brought in, and four registers less at the peak keep the callers' K-buffers out
     // of scratch memory inside the batch loop)

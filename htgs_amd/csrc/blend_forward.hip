@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         quadrant_walk(hits, stage_base, [&](uint32_t addr) {
@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         float4 c = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (c3[i] > 0.0f) c = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS / 4) + 4];
+        if (c3[i] > 0.0f) c = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS_TRAIN / 4) + 4];
         c0[i] = c.x; c1[i] = c.y; c2[i] = c.z;
     }
 #pragma unroll
@@ -160,7 +160,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         quadrant_walk(hits, stage_base, [&](uint32_t addr) {
@@ -187,7 +187,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
         k0[i] = k1[i] = k2[i] = 0.0f;
         if (open) {
             const float bw = T * ca[i];
-            const float4 col = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS / 4) + 4];
+            const float4 col = prim[(size_t)ci[i] * (HTGS_PRIM_FLOATS_TRAIN / 4) + 4];
             k0[i] = col.x; k1[i] = col.y; k2[i] = col.z;
             r = __builtin_fmaf(bw, col.x, r);
             g = __builtin_fmaf(bw, col.y, g);
@@ -238,7 +238,7 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
         __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
+        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + lane, last, lane, cx, cy));
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
         quadrant_walk(hits, stage_base, [&](uint32_t addr) {
@@ -287,7 +287,7 @@ __global__ void __launch_bounds__(256) blend_global_forward_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        tile_stage_load<MODE, 256, false>(st, prim, inst, base + t, last, t, cx, cy);
+        tile_stage_load<MODE, 256, false, kCullNone, false, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const int nb = last - base < 256u ? (int)(last - base) : 256;
         uint32_t addr = stage_address(st);
@@ -334,6 +334,7 @@ extern "C" int htgs_blend_forward(const htgs_frame *f, int selector)
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: null frame");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: bad argument");
+    if (f->prim_floats != HTGS_PRIM_FLOATS_TRAIN) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: the training kernels read records of HTGS_PRIM_FLOATS_TRAIN floats (prim_floats)");
     const bool needs_core = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K;
     const bool needs_tail = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_OIT_BLEND;
     if (!f->ranges || !f->image || (f->n_instances > 0 && (!f->vals[selector] || !f->prim)) ||

@@ -38,6 +38,11 @@ template <int MODE> struct ModeCfg {
 
 inline int tile_size(int mode) { return mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING ? 16 : 8; }
 inline int div_up(int a, int b) { return (a + b - 1) / b; }
+// floats per record of f->prim; -1 for a value that no entry point takes
+inline int frame_prim_floats(const htgs_frame *f)
+{
+    return f->prim_floats == 0 || f->prim_floats == HTGS_PRIM_FLOATS ? HTGS_PRIM_FLOATS : f->prim_floats == HTGS_PRIM_FLOATS_TRAIN ? HTGS_PRIM_FLOATS_TRAIN : -1;
+}
 
 // host side error reporting (api.hip)
 int fail(int code, const char *fmt, ...);

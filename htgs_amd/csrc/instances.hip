@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(kScanBlock) scan_apply_kernel(const uint32_t *
 template <typename KeyT, bool DEPTH>
 __global__ void __launch_bounds__(256) create_instances_kernel(
     const uint32_t *__restrict__ n_touched, const uint32_t *__restrict__ offsets, const uint16_t *__restrict__ bounds,
-    const float *__restrict__ prim, KeyT *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t grid_w, int n, uint64_t capacity)
+    float *__restrict__ prim, KeyT *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t grid_w, int n, uint64_t capacity, int prim_floats)
 {
     __shared__ uint32_t s_end[256];     // inclusive offsets of the block's Gaussians
     __shared__ uint32_t s_x0[256], s_y0[256], s_w[256], s_depth[DEPTH ? 256 : 1];
@@ -132,7 +132,11 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
         if (n_touched[i] != 0) {
             const ushort4 b = *reinterpret_cast<const ushort4 *>(bounds + 4 * (size_t)i);
             x0 = b.x; y0 = b.z; w = (uint32_t)b.y - b.x;
-            if (DEPTH) depth = float_to_bits(prim[(size_t)HTGS_PRIM_FLOATS * i + 15]);   // MT3.w = camera-space z of the centre
+            if (DEPTH) depth = float_to_bits(prim[(size_t)prim_floats * i + 15]);   // MT3.w = camera-space z of the centre
+            // training records: where the Gaussian's instances start in this (unsorted) list and its rectangle, for the
+            // backward pass, which writes a gradient row at the slot of every instance
+            if (prim_floats == HTGS_PRIM_FLOATS_TRAIN)
+                *reinterpret_cast<uint4 *>(prim + (size_t)prim_floats * i + HTGS_PRIM_FLOATS) = make_uint4(end - n_touched[i], x0 | y0 << 16, w, 0u);
         }
     }
     s_end[threadIdx.x] = end;
@@ -304,15 +308,17 @@ extern "C" int htgs_create_instances(const htgs_frame *f)
     const uint32_t grid_w = div_up(f->width, tile);
     const dim3 grid(div_up(f->n_primitives, 256)), block(256);
     const int kb = htgs_key_bytes(f->mode, f->width, f->height);
+    const int prim_floats = frame_prim_floats(f);
+    if (prim_floats < 0) return fail(HTGS_ERR_ARGUMENT, "htgs_create_instances: prim_floats must be 0, %d or %d", HTGS_PRIM_FLOATS, HTGS_PRIM_FLOATS_TRAIN);
     if (kb == 8)
         hipLaunchKernelGGL((create_instances_kernel<uint64_t, true>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
-                           (uint64_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances);
+                           (uint64_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats);
     else if (kb == 4)
         hipLaunchKernelGGL((create_instances_kernel<uint32_t, false>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
-                           (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances);
+                           (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats);
     else
         hipLaunchKernelGGL((create_instances_kernel<uint16_t, false>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
-                           (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances);
+                           (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats);
     return check_launch("create_instances");
 }
 

@@ -178,6 +178,7 @@ extern "C" int htgs_max_weights_blend(const htgs_frame *f, int selector, float *
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: null frame");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: bad argument");
+    if (frame_prim_floats(f) != HTGS_PRIM_FLOATS) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: reads records of HTGS_PRIM_FLOATS floats (prim_floats)");
     if (f->n_instances == 0 || f->n_primitives == 0) return HTGS_OK;
     if (!f->ranges || !f->vals[selector] || !f->prim || !max_weights) return fail(HTGS_ERR_ARGUMENT, "htgs_max_weights_blend: null pointer");
     const int tile = tile_size(f->mode);

@@ -63,11 +63,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     uint32_t *__restrict__ n_touched, uint16_t *__restrict__ bounds, float *__restrict__ prim,
     uint8_t *__restrict__ clamp_info,
     int n, uint32_t grid_w, uint32_t grid_h, float tile, float min_alpha_rcp,
-    int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier)
+    int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier, int rec4)
 {
     // One LDS buffer, used twice: first the block's slice of sh_rest (contiguous in memory, loaded with coalesced
-    // 16-byte reads and then read back per Gaussian at a stride of 3 * total_sh words), then the block's 80-byte
-    // records, written back as one contiguous run of 16-byte stores.
+    // 16-byte reads and then read back per Gaussian at a stride of 3 * total_sh words), then the block's records
+    // (rec4 words of 16 bytes each: five, or eight in training frames, of which the last three are zeros here),
+    // written back as one contiguous run of 16-byte stores.
     extern __shared__ float4 lds4[];
     float *lds = reinterpret_cast<float *>(lds4);
     __shared__ uint8_t s_visible[256];
@@ -211,17 +212,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     __syncthreads();                                               // everyone is done reading the coefficients
 
     if (visible) {
-        float4 *rec = lds4 + (HTGS_PRIM_FLOATS / 4) * threadIdx.x;
+        float4 *rec = lds4 + rec4 * threadIdx.x;
         rec[0] = make_float4(V1.x, V1.y, V1.z, V1.w);
         rec[1] = make_float4(V2.x, V2.y, V2.z, V2.w);
         rec[2] = make_float4(V4.x, V4.y, V4.z, V4.w);
         rec[3] = make_float4(dot3(M3, u[0], u[1], u[2]), dot3(M3, v[0], v[1], v[2]), dot3(M3, w[0], w[1], w[2]), z);
         rec[4] = make_float4(clamp_pos(res[0]), clamp_pos(res[1]), clamp_pos(res[2]), opacity);
+        for (int k = HTGS_PRIM_FLOATS / 4; k < rec4; ++k) rec[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);   // (whole lines go out)
     }
     __syncthreads();
-    float4 *dst4 = reinterpret_cast<float4 *>(prim + (size_t)HTGS_PRIM_FLOATS * first);
-    for (int q = threadIdx.x; q < n_block * (HTGS_PRIM_FLOATS / 4); q += 256)
-        if (s_visible[q / (HTGS_PRIM_FLOATS / 4)]) dst4[q] = lds4[q];
+    float4 *dst4 = reinterpret_cast<float4 *>(prim) + (size_t)rec4 * first;
+    if (rec4 == HTGS_PRIM_FLOATS / 4) {
+        for (int q = threadIdx.x; q < n_block * (HTGS_PRIM_FLOATS / 4); q += 256)
+            if (s_visible[q / (HTGS_PRIM_FLOATS / 4)]) dst4[q] = lds4[q];
+    } else {
+        for (int q = threadIdx.x; q < n_block * (HTGS_PRIM_FLOATS_TRAIN / 4); q += 256)
+            if (s_visible[q / (HTGS_PRIM_FLOATS_TRAIN / 4)]) dst4[q] = lds4[q];
+    }
 }
 
 }  // namespace htgs
@@ -245,13 +252,15 @@ extern "C" int htgs_preprocess(const htgs_frame *f)
     const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
     if (grid_w > 65535u || grid_h > 65535u) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: image too large for 16-bit tile bounds");
     const float min_alpha_rcp = f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K ? 20.0f : 255.0f;
-    // dynamic LDS: the larger of the block's SH coefficients (256 x 3 x total_sh words) and its records (256 x 80 bytes)
+    // dynamic LDS: the larger of the block's SH coefficients (256 x 3 x total_sh words) and its records (256 x 80 or 128 bytes)
     const size_t sh_bytes = f->active_sh_bases > 1 ? (size_t)256 * 3 * f->total_sh_bases * sizeof(float) : 0;
-    const size_t lds_bytes = sh_bytes > 256 * HTGS_PRIM_FLOATS * sizeof(float) ? sh_bytes : 256 * HTGS_PRIM_FLOATS * sizeof(float);
+    const int prim_floats = frame_prim_floats(f);
+    if (prim_floats < 0) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: prim_floats must be 0, %d or %d", HTGS_PRIM_FLOATS, HTGS_PRIM_FLOATS_TRAIN);
+    const size_t lds_bytes = sh_bytes > 256 * prim_floats * sizeof(float) ? sh_bytes : 256 * prim_floats * sizeof(float);
     if (lds_bytes > 64 * 1024) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: sh_rest has more than 21 coefficients per Gaussian");
     hipLaunchKernelGGL(preprocess_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), lds_bytes, (hipStream_t)f->stream,
                        f->positions, f->scales, f->rotations, f->opacities, f->sh_0, f->sh_rest, f->M, f->VPM, f->cam_position,
                        f->n_touched, f->bounds, f->prim, f->clamp_info, f->n_primitives, grid_w, grid_h, (float)tile,
-                       min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier);
+                       min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier, prim_floats / 4);
     return check_launch("preprocess");
 }

@@ -161,7 +161,9 @@ class FrameBuffers:
         self.n_touched = self._scratch("n_touched", n, torch.int32)[:n]
         self.offsets = self._scratch("offsets", n, torch.int32)[:n]
         self.bounds = self._scratch("bounds", 4 * n, torch.int16)[:4 * n].view(n, 4)
-        self.prim = self._scratch("prim", _native.PRIM_FLOATS * n, torch.float32)[:_native.PRIM_FLOATS * n].view(n, _native.PRIM_FLOATS)
+        # (training frames use 128-byte records: the backward pass finds the slot of an instance's gradient row in them)
+        self.prim_floats = _native.PRIM_FLOATS_TRAIN if train else _native.PRIM_FLOATS
+        self.prim = self._scratch("prim", self.prim_floats * n, torch.float32)[:self.prim_floats * n].view(n, self.prim_floats)
         self.clamp_info = torch.empty((3, n), dtype=torch.uint8, device=dev) if train else None
         self.scan_tmp = self._scratch("scan_tmp", self.lib.htgs_scan_tmp_words(n), torch.int32)
         self.n_instances_dev = self._scratch("n_instances_dev", 1, torch.int32)    # written by the scan
@@ -190,6 +192,7 @@ class FrameBuffers:
         f.near_plane, f.far_plane = float(settings.near_plane), float(settings.far_plane)
         f.scale_modifier = float(settings.scale_modifier)
         f.n_touched, f.offsets, f.bounds, f.prim = _ptr(self.n_touched), _ptr(self.offsets), _ptr(self.bounds), _ptr(self.prim)
+        f.prim_floats = self.prim_floats
         f.clamp_info = _ptr(self.clamp_info)
         f.scan_tmp, f.n_instances_dev = _ptr(self.scan_tmp), _ptr(self.n_instances_dev)
         f.ranges = _ptr(self.ranges)

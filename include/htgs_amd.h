@@ -35,6 +35,10 @@ extern "C" {
 /* floats per Gaussian in the `prim` record written by the preprocess stage:
  * VPMT1.xyzw, VPMT2.xyzw, VPMT4.xyzw, MT3.xyzw, r, g, b, opacity */
 #define HTGS_PRIM_FLOATS 20
+/* the training entry points use records of 128 bytes (one cache line per gather): the twenty floats above, then four
+ * words written by htgs_create_instances for the backward pass -- the Gaussian's first slot in the unsorted instance
+ * list (offsets[g-1]), x_min | y_min << 16 and the width of its tile rectangle, 0 -- then padding */
+#define HTGS_PRIM_FLOATS_TRAIN 32
 
 /*
  * One frame: inputs, caller-owned scratch and outputs.  Mirrors the argument list of
@@ -64,7 +68,10 @@ typedef struct htgs_frame {
     uint32_t *n_touched;       /* [N] tiles covered, 0 = culled */
     uint32_t *offsets;         /* [N] inclusive prefix sum of n_touched */
     uint16_t *bounds;          /* [N,4] tile rectangle x_min,x_max,y_min,y_max (exclusive max) */
-    float *prim;               /* [N,HTGS_PRIM_FLOATS] */
+    float *prim;               /* [N,prim_floats] */
+    int32_t prim_floats;       /* 0 or HTGS_PRIM_FLOATS for the inference entry points and htgs_max_weights_*,
+                                  HTGS_PRIM_FLOATS_TRAIN for the training entry points (htgs_forward_*, htgs_blend_forward,
+                                  htgs_blend_backward); the stages they share honour either */
     uint8_t *clamp_info;       /* [3,N] sign flags of the unclamped colour, training only, else NULL */
     uint32_t *scan_tmp;        /* htgs_scan_tmp_words(N) words */
     uint32_t *n_instances_dev; /* [1] total number of instances, written by the scan */
