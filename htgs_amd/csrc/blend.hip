@@ -441,6 +441,9 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
 // ALPHA_BLEND_GLOBAL_ORDERING: instances arrive sorted by (tile, depth of the Gaussian centre);
 // classic front-to-back blending, a pixel stops at T < 1e-4, the workgroup stops when all have.
 // ---------------------------------------------------------------------------------------------
+// A wave holds one 8x8 sub-tile of the 16x16 tile, laid out for the quadrant walk; the 256 threads stage 256 instances
+// per batch, each with one bit per 4x4 quadrant of the tile it can reach, and every wave then walks the hits of its own
+// four quadrants, 64 staged slots at a time.
 template <bool FAST>
 __global__ void __launch_bounds__(256) blend_global_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
@@ -448,12 +451,17 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ TileStage<256> st;
+    __shared__ uint16_t s_reach[256];                  // per staged slot: the quadrants of the tile it can reach
     const uint32_t tile = blockIdx.x;
-    const uint32_t t = threadIdx.x;
+    const uint32_t t = threadIdx.x, wave = t >> 6, lane = t & 63;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
-    const uint32_t x = x0 + (t & 15), y = y0 + (t >> 4);
+    uint32_t local_x, local_y;
+    quadrant_pixel(lane, local_x, local_y);
+    local_x += 8 * (wave & 1);
+    local_y += 8 * (wave >> 1);
+    const uint32_t x = x0 + local_x, y = y0 + local_y;
     const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(t & 15, t >> 4, 16);
+    const PixelTerms pt = pixel_terms(local_x, local_y, 16);
     const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
     float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T = 1.0f;
     bool done = !inside;
@@ -461,26 +469,29 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        tile_stage_load<MODE, 256, false>(st, prim, inst, base + t, last, t, cx, cy);
+        s_reach[t] = (uint16_t)tile_stage_load<MODE, 256, false, kCullAlpha, true>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
-        const int nb = last - base < 256u ? (int)(last - base) : 256;
-        uint32_t addr = stage_address(st);
-        for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
-            TileFrag f;
-            if (!tile_frag_cutoff<256>(addr, pt, f)) continue;
-            f.den_rcp = frag_rcp<FAST>(f.den);
-            const float4 q4 = stage_row<256, 4>(addr);
-            if (!tile_frag_alpha<MODE, FAST>(q4.w, f)) continue;
-            const float4 col = stage_row<256, 5>(addr);
-            const float wgt = T * f.alpha;
-            r = __builtin_fmaf(wgt, col.x, r);
-            g = __builtin_fmaf(wgt, col.y, g);
-            b = __builtin_fmaf(wgt, col.z, b);
-            const float depth = q4.z;
-            if (median) depth_pixel = T > 0.5f ? depth : depth_pixel;
-            else depth_pixel = __builtin_fmaf(wgt, depth, depth_pixel);
-            T *= 1.0f - f.alpha;
-            if (T < kTransmittanceThreshold) done = true;
+        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+        for (uint32_t part = 0; part < 4 && base + 64 * part < last; ++part) {
+            if (__ballot(!done) == 0) break;            // (wave-uniform: every pixel of the sub-tile is opaque)
+            QuadrantHits hits = quadrant_ballot(((uint32_t)s_reach[64 * part + lane] >> (4 * wave)) & 0xfu);
+            quadrant_walk(hits, stage_base + 64u * 16u * part, [&](uint32_t addr) {
+                TileFrag f;
+                if (done || !tile_frag_cutoff<256>(addr, pt, f)) return;
+                f.den_rcp = frag_rcp<FAST>(f.den);
+                const float4 q4 = stage_row<256, 4>(addr);
+                if (!tile_frag_alpha<MODE, FAST>(q4.w, f)) return;
+                const float4 col = stage_row<256, 5>(addr);
+                const float wgt = T * f.alpha;
+                r = __builtin_fmaf(wgt, col.x, r);
+                g = __builtin_fmaf(wgt, col.y, g);
+                b = __builtin_fmaf(wgt, col.z, b);
+                const float depth = q4.z;
+                if (median) depth_pixel = T > 0.5f ? depth : depth_pixel;
+                else depth_pixel = __builtin_fmaf(wgt, depth, depth_pixel);
+                T *= 1.0f - f.alpha;
+                if (T < kTransmittanceThreshold) done = true;
+            });
         }
     }
     if (!inside) return;

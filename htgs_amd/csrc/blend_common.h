@@ -152,6 +152,52 @@ __device__ __forceinline__ uint32_t tile_quadrant_hits(const float (&n)[6], cons
     return bits;
 }
 
+// The 16x16 tile of ALPHA_BLEND_GLOBAL_ORDERING: sixteen 4x4 quadrants, four per 8x8 sub-tile.  Bit 4 s + q of the result
+// stands for quadrant q (numbered as above) of sub-tile s = 2 (row >= 8) + (column >= 8).  Four evaluations per pixel
+// row serve the row's four quadrants.
+template <int MODE>
+__device__ __forceinline__ uint32_t tile_quadrant_hits16(const float (&n)[6], const float (&d)[6], float opacity)
+{
+    static_assert(ModeCfg<MODE>::tile == 16, "16x16 tiles");
+    constexpr float h = 7.5f;
+    float r = __builtin_fmaf(__builtin_amdgcn_logf(opacity), -1.0f / ModeCfg<MODE>::exp2_scale, 1.0f);
+    r = r < 1.0f ? r : 1.0f;
+    r = r > -1.0f ? r : -1.0f;
+    r += 1e-5f;
+    float q[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) q[i] = __builtin_fmaf(-r, d[i], n[i]);
+    const float s0 = __builtin_fabsf(n[0]) + __builtin_fabsf(d[0]);
+    const float s1 = (__builtin_fabsf(n[1]) + __builtin_fabsf(d[1])) + (__builtin_fabsf(n[2]) + __builtin_fabsf(d[2]));
+    const float s2 = ((__builtin_fabsf(n[3]) + __builtin_fabsf(d[3])) + (__builtin_fabsf(n[4]) + __builtin_fabsf(d[4]))) +
+                     (__builtin_fabsf(n[5]) + __builtin_fabsf(d[5]));
+    const float margin = 1e-5f * __builtin_fmaf(h * h, s2, __builtin_fmaf(h, s1, s0));
+    if (!(q[3] > 0.0f)) return 0xffffu;              // (not convex along the rows, or not a number: kept everywhere)
+    const float to_vertex = -0.5f * __builtin_amdgcn_rcpf(q[3]);
+    uint32_t bits = 0;
+#pragma nounroll
+    for (int band = 0; band < 4; ++band) {           // four pixel rows: one row of quadrants
+        float least[4] = { __FLT_MAX__, __FLT_MAX__, __FLT_MAX__, __FLT_MAX__ };
+#pragma nounroll
+        for (int row = 0; row < 4; ++row) {
+            const float y = (float)(4 * band + row) - h;
+            const float b = __builtin_fmaf(q[4], y, q[1]);
+            const float c = __builtin_fmaf(y, __builtin_fmaf(q[5], y, q[2]), q[0]);
+            const float xv = __builtin_rintf(__builtin_fmaf(b, to_vertex, 0.5f)) - 0.5f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float lo = (float)(4 * k) - h;
+                const float xc = __builtin_fminf(__builtin_fmaxf(xv, lo), lo + 3.0f);
+                least[k] = __builtin_fminf(least[k], __builtin_fmaf(xc, __builtin_fmaf(q[3], xc, b), c));
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (!(least[k] > margin)) bits |= 1u << (4 * (2 * (band >> 1) + (k >> 1)) + 2 * (band & 1) + (k & 1));
+    }
+    return bits;
+}
+
 // Stages instance `fetch` of the sorted list in slot `slot` (the same arithmetic as tile_geometry / tile_quadratics,
 // written out so that every row is stored as soon as it is complete: the kernels that call this hold a K-buffer in
 // registers).  Returns whether the slot holds an instance that can reach a pixel of the tile: always true for a
@@ -264,6 +310,7 @@ __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const floa
         }
         return bits;
     }
+    else if constexpr (QUADRANTS && ModeCfg<MODE>::tile == 16) return tile_quadrant_hits16<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
     else if constexpr (QUADRANTS) return tile_quadrant_hits<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
     else return (uint32_t)!tile_misses<MODE>(n, d, CULL == kCullCutoff ? 1.0f : col.w);
 }
@@ -281,16 +328,6 @@ typedef __attribute__((address_space(3))) const float lds_float;
 template <int N>
 __device__ __forceinline__ uint32_t stage_address(const TileStage<N> &st) { return (uint32_t)(uintptr_t)(lds_float4 *)&st.q[0][0]; }
 __device__ __forceinline__ void stage_advance(uint32_t &addr) { asm volatile("v_add_u32 %0, 16, %0" : "+v"(addr)); }
-// the walk over the hits of a batch: takes the lowest set bit of the (wave-uniform) mask and returns the LDS address
-// of that slot's q[0] entry, again through an opaque move so that one VGPR serves every read of the iteration
-__device__ __forceinline__ uint32_t stage_next_hit(uint64_t &hits, uint32_t stage_base)
-{
-    const uint32_t at = stage_base + 16u * (uint32_t)__builtin_ctzll(hits);
-    hits &= hits - 1;
-    uint32_t addr;
-    asm volatile("v_mov_b32 %0, %1" : "=v"(addr) : "s"(at));
-    return addr;
-}
 // Quadrant walk.  Lanes 16 q .. 16 q + 15 hold the 4x4 pixels of quadrant q of the tile and walk the hits of that
 // quadrant, in list order, in lock step with the other three quadrants: a turn of the loop serves up to four instances,
 // one per quadrant, and a batch takes as many turns as its busiest quadrant has hits (an instance reaches 1.9 of the four
