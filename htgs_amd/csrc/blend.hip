@@ -456,9 +456,7 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
     const uint32_t t = threadIdx.x, wave = t >> 6, lane = t & 63;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
     uint32_t local_x, local_y;
-    quadrant_pixel(lane, local_x, local_y);
-    local_x += 8 * (wave & 1);
-    local_y += 8 * (wave >> 1);
+    subtile_pixel(t, local_x, local_y);
     const uint32_t x = x0 + local_x, y = y0 + local_y;
     const bool inside = x < width && y < height;
     const PixelTerms pt = pixel_terms(local_x, local_y, 16);
@@ -472,27 +470,25 @@ __global__ void __launch_bounds__(256) blend_global_kernel(
         s_reach[t] = (uint16_t)tile_stage_load<MODE, 256, false, kCullAlpha, true>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
         const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        for (uint32_t part = 0; part < 4 && base + 64 * part < last; ++part) {
-            if (__ballot(!done) == 0) break;            // (wave-uniform: every pixel of the sub-tile is opaque)
-            QuadrantHits hits = quadrant_ballot(((uint32_t)s_reach[64 * part + lane] >> (4 * wave)) & 0xfu);
-            quadrant_walk(hits, stage_base + 64u * 16u * part, [&](uint32_t addr) {
-                TileFrag f;
-                if (done || !tile_frag_cutoff<256>(addr, pt, f)) return;
-                f.den_rcp = frag_rcp<FAST>(f.den);
-                const float4 q4 = stage_row<256, 4>(addr);
-                if (!tile_frag_alpha<MODE, FAST>(q4.w, f)) return;
-                const float4 col = stage_row<256, 5>(addr);
-                const float wgt = T * f.alpha;
-                r = __builtin_fmaf(wgt, col.x, r);
-                g = __builtin_fmaf(wgt, col.y, g);
-                b = __builtin_fmaf(wgt, col.z, b);
-                const float depth = q4.z;
-                if (median) depth_pixel = T > 0.5f ? depth : depth_pixel;
-                else depth_pixel = __builtin_fmaf(wgt, depth, depth_pixel);
-                T *= 1.0f - f.alpha;
-                if (T < kTransmittanceThreshold) done = true;
-            });
-        }
+        subtile_walk(s_reach, stage_base, last - base < 256u ? last - base : 256u, wave, lane,
+                     [&]() { return __ballot(!done) == 0; },       // every pixel of the sub-tile is opaque
+                     [&](uint32_t addr) {
+            TileFrag f;
+            if (done || !tile_frag_cutoff<256>(addr, pt, f)) return;
+            f.den_rcp = frag_rcp<FAST>(f.den);
+            const float4 q4 = stage_row<256, 4>(addr);
+            if (!tile_frag_alpha<MODE, FAST>(q4.w, f)) return;
+            const float4 col = stage_row<256, 5>(addr);
+            const float wgt = T * f.alpha;
+            r = __builtin_fmaf(wgt, col.x, r);
+            g = __builtin_fmaf(wgt, col.y, g);
+            b = __builtin_fmaf(wgt, col.z, b);
+            const float depth = q4.z;
+            if (median) depth_pixel = T > 0.5f ? depth : depth_pixel;
+            else depth_pixel = __builtin_fmaf(wgt, depth, depth_pixel);
+            T *= 1.0f - f.alpha;
+            if (T < kTransmittanceThreshold) done = true;
+        });
     }
     if (!inside) return;
     if (!median) depth_pixel = T < 1.0f ? depth_pixel / (1.0f - T) : 0.0f;

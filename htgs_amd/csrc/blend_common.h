@@ -518,4 +518,25 @@ __device__ __forceinline__ TilePixel quadrant_tile_pixel(uint32_t tile, uint32_t
     return p;
 }
 
+// The 16x16 tile of ALPHA_BLEND_GLOBAL_ORDERING: 256 threads, wave w holds the 8x8 sub-tile 2 (row >= 8) + (column >= 8)
+// = w, laid out for the quadrant walk.
+__device__ __forceinline__ void subtile_pixel(uint32_t thread, uint32_t &local_x, uint32_t &local_y)
+{
+    quadrant_pixel(thread & 63u, local_x, local_y);
+    local_x += 8u * ((thread >> 6) & 1u);
+    local_y += 8u * (thread >> 7);
+}
+// One batch of 256 staged instances (reach[slot]: the sixteen quadrant bits tile_stage_load returned for it): the wave
+// walks the hits of its own four quadrants, 64 slots at a time, and stops early once all_done() says so (wave-uniform).
+template <typename Done, typename Turn>
+__device__ __forceinline__ void subtile_walk(const uint16_t *reach, uint32_t stage_base, uint32_t n_staged, uint32_t wave, uint32_t lane,
+                                             Done &&all_done, Turn &&turn)
+{
+    for (uint32_t part = 0; part < 4 && 64u * part < n_staged; ++part) {
+        if (all_done()) break;
+        QuadrantHits hits = quadrant_ballot(((uint32_t)reach[64u * part + lane] >> (4u * wave)) & 0xfu);
+        quadrant_walk(hits, stage_base + 64u * 16u * part, turn);
+    }
+}
+
 }  // namespace htgs
