@@ -422,8 +422,8 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
 // ALPHA_BLEND_GLOBAL_ORDERING: one lane per pixel walks the depth-sorted list front to back with the final
 // colour of the pixel (backward.cuh:97-249), evaluating every fragment with the forward pass's arithmetic.  Per
 // fragment a lane produces dL/drgb, dL/dopacity and the twelve moments of dL/dnum and dL/dden about the tile
-// centre (see the moments kernel above); the sixteen numbers are summed over the wave and parked in LDS, and
-// after a batch of 64 Gaussians one thread per Gaussian adds the four waves' sums, applies the chain to the VPMT
+// centre (see the moments kernel above); the sixteen numbers are summed over the lanes of a 4x4 quadrant and parked in
+// LDS, and after a batch of Gaussians one thread per Gaussian adds the quadrants' sums, applies the chain to the VPMT
 // rows once and writes the instance's row.
 // ---------------------------------------------------------------------------------------------
 // Sum over the 64 lanes with data-parallel-primitive moves (six v_add_f32 with a DPP operand): butterflies inside
@@ -445,11 +445,12 @@ __device__ __forceinline__ float wave_sum(float v)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
-// Sums of 16 values over the 64 lanes at once.  v_permlane32_swap exchanges the upper half of one register with the
-// lower half of another, so one swap and one add fold two values into one register whose halves hold the two half-way
-// sums; v_permlane16_swap does the same with the odd and even rows of 16 lanes.  After both folds register r holds, in
-// row q, a 16-lane partial sum of value r + 4 q, which four DPP adds complete: 40 vector instructions where 16
-// separate wave sums take 112.  On return every lane of row q holds the total of value r + 4 q in v[r], r < 4.
+// Sums of 16 values over the sixteen lanes of each quadrant at once, a quadrant being lanes 4 q .. 4 q + 3 of each of the
+// four rows of sixteen lanes.  v_permlane32_swap exchanges the upper half of one register with the lower half of another,
+// so one swap and one add fold two values into one register whose halves hold the two half-way sums; v_permlane16_swap
+// does the same with the odd and even rows.  After both folds register r holds, in row w, the sum over the four rows of
+// value r + 4 w, which two adds inside the group of four lanes complete: 32 vector instructions where sixteen separate
+// sums take 64.  On return the lanes of quadrant q in row w hold quadrant q's total of value r + 4 w in v[r], r < 4.
 __device__ __forceinline__ void fold_halves(float &a, float &b)
 {
     const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
@@ -460,7 +461,7 @@ __device__ __forceinline__ void fold_rows(float &a, float &b)
     const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
     a = __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
-__device__ __forceinline__ void wave_sum_16(float (&v)[16])
+__device__ __forceinline__ void quadrant_sum_16(float (&v)[16])
 {
 #pragma unroll
     for (int r = 0; r < 8; ++r) fold_halves(v[r], v[r + 8]);      // lower half: value r, upper half: value r + 8
@@ -469,16 +470,17 @@ __device__ __forceinline__ void wave_sum_16(float (&v)[16])
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         float t = v[r];
-        t += dpp_take<0xB1, 0xf>(t);
-        t += dpp_take<0x4E, 0xf>(t);
-        t += dpp_take<0x141, 0xf>(t);
-        t += dpp_take<0x140, 0xf>(t);
+        t += dpp_take<0xB1, 0xf>(t);        // quad_perm [1,0,3,2]
+        t += dpp_take<0x4E, 0xf>(t);        // quad_perm [2,3,0,1]
         v[r] = t;
     }
 }
 
-constexpr int kGlobalBatch = 64;              // Gaussians per staged batch: one bit each in a wave's 64-bit hit mask
-
+constexpr int kGlobalBatch = 32;              // Gaussians per staged batch (a bit each in a quadrant's hit mask); sized by the LDS the quadrants' sums take
+// A wave holds one 8x8 sub-tile of the 16x16 tile and walks the hits of its own four 4x4 quadrants (subtile_walk): a turn
+// serves up to four Gaussians, one per quadrant, whose sixteen sums are taken over the quadrant's sixteen lanes and parked
+// in LDS per (quadrant, Gaussian); the thread that finishes a Gaussian adds the parts of the quadrants it can reach, in
+// quadrant order.
 template <bool HELPER>
 __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
@@ -488,17 +490,22 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ TileStage<kGlobalBatch> st;
     __shared__ float4 s_rows[HELPER ? 3 : 1][kGlobalBatch];   // VPMT1, VPMT2, VPMT4 (third densification row only)
-    __shared__ float s_part[4][kGlobalBatch][17];             // per wave: the 16 sums of one Gaussian (padded row)
-    __shared__ float s_help[HELPER ? 4 : 1][kGlobalBatch];
-    __shared__ uint32_t s_hit[4][2];
+    __shared__ float4 s_part[16][kGlobalBatch][4];            // per quadrant of the tile: the 16 sums of one Gaussian
+    __shared__ float s_help[HELPER ? 16 : 1][kGlobalBatch];
+    __shared__ uint16_t s_reach[kGlobalBatch];                // per staged Gaussian: the quadrants it can reach
+    __shared__ uint32_t s_walked;                             // bit w: wave w walked this batch (its pixels were not all opaque)
     const uint32_t tile = blockIdx.x;
     const uint32_t t = threadIdx.x;
     const uint32_t lane = t & (kWave - 1), wave = t >> 6;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
-    const uint32_t x = x0 + (t & 15), y = y0 + (t >> 4);
+    uint32_t local_x, local_y;
+    banked_quadrant_pixel(lane, local_x, local_y);            // (a quadrant = one bank of four lanes in each row: quadrant_sum_16)
+    local_x += 8u * (wave & 1u);
+    local_y += 8u * (wave >> 1);
+    const uint32_t x = x0 + local_x, y = y0 + local_y;
     const bool inside = x < width && y < height;
     const float fx = (float)x, fy = (float)y;
-    const PixelTerms pt = pixel_terms(t & 15, t >> 4, 16);
+    const PixelTerms pt = pixel_terms(local_x, local_y, 16);
     const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
     const size_t np = (size_t)width * height, pix = inside ? (size_t)width * y + x : 0;
     float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f, e0 = 0.0f, e1 = 0.0f, e2 = 0.0f;
@@ -508,103 +515,117 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     }
     float n0 = 0.0f, n1 = 0.0f, n2 = 0.0f, T = 1.0f;
     bool done = !inside;
+    const uint32_t quadrant = 4u * wave + ((lane >> 2) & 3u); // of the tile
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     uint32_t base = first;
     for (; base < last; base += kGlobalBatch) {
         // (the barrier also separates the previous batch's reads of the staged records and sums from the writes below)
         if (__syncthreads_count(done) == 256) break;
-        if (wave == 0) tile_stage_load<MODE, kGlobalBatch, false, kCullNone, false, kTrainRec4>(st, prim, inst, base + lane, last, lane, cx, cy);
-        if (HELPER && wave >= 1 && base + lane < last)
+        if (wave == 0 && lane < (uint32_t)kGlobalBatch) {
+            s_reach[lane] = (uint16_t)tile_stage_load<MODE, kGlobalBatch, false, kCullAlpha, true, kTrainRec4>(st, prim, inst, base + lane, last, lane, cx, cy);
+            if (lane == 0) s_walked = 0u;
+        }
+        if (HELPER && wave >= 1 && lane < (uint32_t)kGlobalBatch && base + lane < last)
             s_rows[wave - 1][lane] = prim[(size_t)inst[base + lane] * kTrainRec4 + (wave - 1)];
         __syncthreads();
         const int nb = last - base < (uint32_t)kGlobalBatch ? (int)(last - base) : kGlobalBatch;
-        uint32_t hit_lo = 0u, hit_hi = 0u;                                       // wave-uniform
-        uint32_t addr = stage_address(st);
-        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
-            float acc[16];
+        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+        if (__ballot(!done) != 0) {                                              // wave-uniform
+            if (lane == 0) atomicOr(&s_walked, 1u << wave);
+            QuadrantHits hits = quadrant_ballot(lane < (uint32_t)kGlobalBatch ? ((uint32_t)s_reach[lane] >> (4u * wave)) & 0xfu : 0u);
+            quadrant_walk<true>(hits, stage_base, [&](uint32_t addr) {
+                const uint32_t j = (addr - stage_base) >> 4;                     // the staged slot, the same in the quadrant's lanes
+                float acc[16];
 #pragma unroll
-            for (int k = 0; k < 16; ++k) acc[k] = 0.0f;
-            float help = 0.0f;
-            bool hit = false;
-            TileFrag f;
-            // the forward pass's own arithmetic (blend_global_forward_kernel): same accept / reject decisions, same alpha
-            if (!done && tile_frag_cutoff<kGlobalBatch>(addr, pt, f)) {
-                f.den_rcp = rcp_exact(f.den);
-                const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * f.den_rcp);
-                const float4 col = stage_row<kGlobalBatch, 5>(addr);
-                const float opacity = stage_opacity<kGlobalBatch>(addr);
-                const float ag = opacity * G;
-                const float alpha = ag < kMaxFragmentAlpha ? ag : kMaxFragmentAlpha;
-                if (!(alpha < ModeCfg<MODE>::min_alpha)) {
-                    hit = true;
-                    const float bw = T * alpha;
-                    acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                        // :171-174
-                    n0 = __builtin_fmaf(bw, col.x, n0); n1 = __builtin_fmaf(bw, col.y, n1); n2 = __builtin_fmaf(bw, col.z, n2);   // :178
-                    const float oma = 1.0f - alpha;
-                    const float omar = rcp_refined(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);    // [1e-8, 1]: exact there
-                    const float dL_dalpha = (T * col.x - (e0 - n0) * omar) * g0 + (T * col.y - (e1 - n1) * omar) * g1
-                                          + (T * col.z - (e2 - n2) * omar) * g2;                // :181
-                    if (dL_dalpha != 0.0f) {
-                        acc[3] = dL_dalpha * G;                                                  // :262
-                        // rho^2 = num / (kc den) with num = kc |m|^2:  dL/dnum and dL/dden  (:263-266)
-                        const float dL_drho2 = dL_dalpha * opacity * -0.5f * G;
-                        const float wn = (dL_drho2 * ModeCfg<MODE>::cutoff_sq) * f.den_rcp;
-                        const float wd = -(wn * f.num) * f.den_rcp;
-                        const float wnx = wn * pt.X, wny = wn * pt.Y, wdx = wd * pt.X, wdy = wd * pt.Y;
-                        acc[4] = wn; acc[5] = wnx; acc[6] = wny; acc[7] = wnx * pt.X; acc[8] = wnx * pt.Y; acc[9] = wny * pt.Y;
-                        acc[10] = wd; acc[11] = wdx; acc[12] = wdy; acc[13] = wdx * pt.X; acc[14] = wdx * pt.Y; acc[15] = wdy * pt.Y;
-                        if (HELPER) {
-                            // fourth components of the fragment's dL/dVPMT rows (:260-289) -> |dL/dposition|_1 (:292-306)
-                            const float4 V1 = s_rows[0][j], V2 = s_rows[1][j], V4 = s_rows[2][j];
-                            const float px0 = __builtin_fmaf(-V4.x, fx, V1.x), px1 = __builtin_fmaf(-V4.y, fx, V1.y);
-                            const float px2 = __builtin_fmaf(-V4.z, fx, V1.z), px3 = __builtin_fmaf(-V4.w, fx, V1.w);
-                            const float py0 = __builtin_fmaf(-V4.x, fy, V2.x), py1 = __builtin_fmaf(-V4.y, fy, V2.y);
-                            const float py2 = __builtin_fmaf(-V4.z, fy, V2.z), py3 = __builtin_fmaf(-V4.w, fy, V2.w);
-                            const float w2 = 2.0f * (dL_drho2 * f.den_rcp);                       // 2 dL/d|m|^2
-                            const float dm0 = w2 * __builtin_fmaf(px3, py0, -(px0 * py3));
-                            const float dm1 = w2 * __builtin_fmaf(px3, py1, -(px1 * py3));
-                            const float dm2 = w2 * __builtin_fmaf(px3, py2, -(px2 * py3));
-                            const float dpx3 = py0 * dm0 + py1 * dm1 + py2 * dm2;
-                            const float dpy3 = -(px0 * dm0 + px1 * dm1 + px2 * dm2);
-                            const float dv3 = -fx * dpx3 - fy * dpy3;
+                for (int k = 0; k < 16; ++k) acc[k] = 0.0f;
+                float help = 0.0f;
+                bool hit = false;
+                TileFrag f;
+                // the forward pass's own arithmetic (blend_global_forward_kernel): same accept / reject decisions, same alpha
+                if (!done && tile_frag_cutoff<kGlobalBatch>(addr, pt, f)) {
+                    f.den_rcp = rcp_exact(f.den);
+                    const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * f.den_rcp);
+                    const float4 col = stage_row<kGlobalBatch, 5>(addr);
+                    const float opacity = stage_opacity<kGlobalBatch>(addr);
+                    const float ag = opacity * G;
+                    const float alpha = ag < kMaxFragmentAlpha ? ag : kMaxFragmentAlpha;
+                    if (!(alpha < ModeCfg<MODE>::min_alpha)) {
+                        hit = true;
+                        const float bw = T * alpha;
+                        acc[0] = bw * g0; acc[1] = bw * g1; acc[2] = bw * g2;                        // :171-174
+                        n0 = __builtin_fmaf(bw, col.x, n0); n1 = __builtin_fmaf(bw, col.y, n1); n2 = __builtin_fmaf(bw, col.z, n2);   // :178
+                        const float oma = 1.0f - alpha;
+                        const float omar = rcp_refined(oma > kOneMinusAlphaEps ? oma : kOneMinusAlphaEps);    // [1e-8, 1]: exact there
+                        const float dL_dalpha = (T * col.x - (e0 - n0) * omar) * g0 + (T * col.y - (e1 - n1) * omar) * g1
+                                              + (T * col.z - (e2 - n2) * omar) * g2;                // :181
+                        if (dL_dalpha != 0.0f) {
+                            acc[3] = dL_dalpha * G;                                                  // :262
+                            // rho^2 = num / (kc den) with num = kc |m|^2:  dL/dnum and dL/dden  (:263-266)
+                            const float dL_drho2 = dL_dalpha * opacity * -0.5f * G;
+                            const float wn = (dL_drho2 * ModeCfg<MODE>::cutoff_sq) * f.den_rcp;
+                            const float wd = -(wn * f.num) * f.den_rcp;
+                            const float wnx = wn * pt.X, wny = wn * pt.Y, wdx = wd * pt.X, wdy = wd * pt.Y;
+                            acc[4] = wn; acc[5] = wnx; acc[6] = wny; acc[7] = wnx * pt.X; acc[8] = wnx * pt.Y; acc[9] = wny * pt.Y;
+                            acc[10] = wd; acc[11] = wdx; acc[12] = wdy; acc[13] = wdx * pt.X; acc[14] = wdx * pt.Y; acc[15] = wdy * pt.Y;
+                            if (HELPER) {
+                                // fourth components of the fragment's dL/dVPMT rows (:260-289) -> |dL/dposition|_1 (:292-306)
+                                const float4 V1 = s_rows[0][j], V2 = s_rows[1][j], V4 = s_rows[2][j];
+                                const float px0 = __builtin_fmaf(-V4.x, fx, V1.x), px1 = __builtin_fmaf(-V4.y, fx, V1.y);
+                                const float px2 = __builtin_fmaf(-V4.z, fx, V1.z), px3 = __builtin_fmaf(-V4.w, fx, V1.w);
+                                const float py0 = __builtin_fmaf(-V4.x, fy, V2.x), py1 = __builtin_fmaf(-V4.y, fy, V2.y);
+                                const float py2 = __builtin_fmaf(-V4.z, fy, V2.z), py3 = __builtin_fmaf(-V4.w, fy, V2.w);
+                                const float w2 = 2.0f * (dL_drho2 * f.den_rcp);                       // 2 dL/d|m|^2
+                                const float dm0 = w2 * __builtin_fmaf(px3, py0, -(px0 * py3));
+                                const float dm1 = w2 * __builtin_fmaf(px3, py1, -(px1 * py3));
+                                const float dm2 = w2 * __builtin_fmaf(px3, py2, -(px2 * py3));
+                                const float dpx3 = py0 * dm0 + py1 * dm1 + py2 * dm2;
+                                const float dpy3 = -(px0 * dm0 + px1 * dm1 + px2 * dm2);
+                                const float dv3 = -fx * dpx3 - fy * dpy3;
 #pragma unroll
-                            for (int k = 0; k < 3; ++k) help += fabsf(VPM[k] * dpx3 + VPM[4 + k] * dpy3 + VPM[12 + k] * dv3);
+                                for (int k = 0; k < 3; ++k) help += fabsf(VPM[k] * dpx3 + VPM[4 + k] * dpy3 + VPM[12 + k] * dv3);
+                            }
                         }
+                        T *= oma;                                                                    // :245
+                        if (T < kTransmittanceThreshold) done = true;
                     }
-                    T *= oma;                                                                    // :245
-                    if (T < kTransmittanceThreshold) done = true;
                 }
-            }
-            if (__any(hit)) {                                                                    // wave-uniform
-                wave_sum_16(acc);
-                if ((lane & 15u) == 0u) {                                                        // one lane per row of 16 lanes
-                    float *dst = &s_part[wave][j][4 * (lane >> 4)];
-                    dst[0] = acc[0]; dst[1] = acc[1]; dst[2] = acc[2]; dst[3] = acc[3];
+                // the quadrant's sums (zeros where no pixel of it is touched: the part is written either way, the thread
+                // that finishes the Gaussian reads every part the staging lane promised)
+                const uint64_t hit_lanes = __ballot(hit);
+                if (hit_lanes & (0x000f000f000f000full << (lane & 12u))) {       // the same in the quadrant's lanes
+                    quadrant_sum_16(acc);
+                    if (HELPER) {
+                        help += dpp_take<0xB1, 0xf>(help);
+                        help += dpp_take<0x4E, 0xf>(help);
+                        help += __shfl_xor(help, 16, 64);
+                        help += __shfl_xor(help, 32, 64);
+                    }
                 }
-                if (HELPER) {
-                    const float s = wave_sum(help);
-                    if (lane == 0) s_help[wave][j] = s;
+                if ((lane & 3u) == 0u) {                                         // row r of the wave holds sums 4 r .. 4 r + 3
+                    s_part[quadrant][j][lane >> 4] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                    if (HELPER && lane < 16u) s_help[quadrant][j] = help;
                 }
-                if (j < 32) hit_lo |= 1u << j; else hit_hi |= 1u << (j - 32);
-            }
+            });
         }
-        if (lane == 0) { s_hit[wave][0] = hit_lo; s_hit[wave][1] = hit_hi; }
         __syncthreads();
-        // one thread per Gaussian of the batch: the four waves' sums in a fixed order, the chain to the VPMT rows, the row
+        // one thread per Gaussian of the batch: the quadrants' sums in a fixed order, the chain to the VPMT rows, the row
         if (t < (uint32_t)nb) {
             float m[16];
 #pragma unroll
             for (int k = 0; k < 16; ++k) m[k] = 0.0f;
             float help = 0.0f;
             bool any = false;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                if ((s_hit[w][t >> 5] >> (t & 31)) & 1u) {
+            const uint32_t reach = s_reach[t], walked = s_walked;
+            for (uint32_t qd = 0; qd < 16; ++qd) {
+                if (((reach >> qd) & 1u) && ((walked >> (qd >> 2)) & 1u)) {
                     any = true;
-#pragma unroll
-                    for (int k = 0; k < 16; ++k) m[k] += s_part[w][t][k];
-                    if (HELPER) help += s_help[w][t];
+                    const float4 p0 = s_part[qd][t][0], p1 = s_part[qd][t][1], p2 = s_part[qd][t][2], p3 = s_part[qd][t][3];
+                    m[0] += p0.x; m[1] += p0.y; m[2] += p0.z; m[3] += p0.w;
+                    m[4] += p1.x; m[5] += p1.y; m[6] += p1.z; m[7] += p1.w;
+                    m[8] += p2.x; m[9] += p2.y; m[10] += p2.z; m[11] += p2.w;
+                    m[12] += p3.x; m[13] += p3.y; m[14] += p3.z; m[15] += p3.w;
+                    if (HELPER) help += s_help[qd][t];
                 }
             }
             const uint32_t g = inst[base + t];

@@ -231,6 +231,14 @@ __device__ __forceinline__ void quadrant_pixel(uint32_t lane, uint32_t &local_x,
     local_y = (lane >> 5) * 4 + ((lane >> 2) & 3);
 }
 
+// the same for the banked layout (quadrant q = lanes 4 q .. 4 q + 3 of every row of sixteen lanes; the row is the pixel row)
+__device__ __forceinline__ void banked_quadrant_pixel(uint32_t lane, uint32_t &local_x, uint32_t &local_y)
+{
+    const uint32_t q = (lane >> 2) & 3u;
+    local_x = (q & 1u) * 4u + (lane & 3u);
+    local_y = (q >> 1) * 4u + (lane >> 4);
+}
+
 // kCullPixels: a slot counts for a quadrant when the instance passes the cut-off -- with the walk's own arithmetic -- at
 // one of the pixels named by pixel_lanes (a wave-uniform mask over the lanes of the quadrant walk) that lie in it.
 enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2, kCullPixels = 3 };
@@ -350,6 +358,9 @@ __device__ __forceinline__ bool quadrant_pending(const QuadrantHits &w) { return
 // clears that bit (bit 63 of an empty mask).  A quadrant is one row of sixteen lanes to the data-parallel primitives, so
 // its lanes take the slot by a move with that row's mask: no exec writes, and the scalar unit, which the four SIMDs of a
 // compute unit share, is left to the loop's branches.
+// BANKED: a quadrant is not a row of sixteen lanes but lanes 4 q .. 4 q + 3 of each of the four rows (bank q of the
+// data-parallel primitives), which is the layout in which sums over a quadrant's lanes fold across the rows.
+template <bool BANKED = false>
 __device__ __forceinline__ uint32_t quadrant_next_hit(QuadrantHits &w)
 {
     uint32_t a0, a1, a2, a3, addr, t;
@@ -358,19 +369,34 @@ __device__ __forceinline__ uint32_t quadrant_next_hit(QuadrantHits &w)
                  "s_bitset0_b64 %[h0], %[a0]\n\ts_bitset0_b64 %[h1], %[a1]\n\ts_bitset0_b64 %[h2], %[a2]\n\ts_bitset0_b64 %[h3], %[a3]"
                  : [a0] "=&s"(a0), [a1] "=&s"(a1), [a2] "=&s"(a2), [a3] "=&s"(a3),
                    [h0] "+s"(w.h[0]), [h1] "+s"(w.h[1]), [h2] "+s"(w.h[2]), [h3] "+s"(w.h[3]));
-    asm volatile("v_mov_b32 %[addr], %[a0]\n\t"
-                 "v_mov_b32 %[t], %[a1]\n\t"
-                 "s_nop 1\n\t"
-                 "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x2 bank_mask:0xf\n\t"
-                 "v_mov_b32 %[t], %[a2]\n\t"
-                 "s_nop 1\n\t"
-                 "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x4 bank_mask:0xf\n\t"
-                 "v_mov_b32 %[t], %[a3]\n\t"
-                 "s_nop 1\n\t"
-                 "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x8 bank_mask:0xf\n\t"
-                 "v_lshlrev_b32 %[addr], 4, %[addr]"
-                 : [addr] "=&v"(addr), [t] "=&v"(t)
-                 : [a0] "s"(a0), [a1] "s"(a1), [a2] "s"(a2), [a3] "s"(a3));
+    if constexpr (BANKED)
+        asm volatile("v_mov_b32 %[addr], %[a0]\n\t"
+                     "v_mov_b32 %[t], %[a1]\n\t"
+                     "s_nop 1\n\t"
+                     "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x2\n\t"
+                     "v_mov_b32 %[t], %[a2]\n\t"
+                     "s_nop 1\n\t"
+                     "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x4\n\t"
+                     "v_mov_b32 %[t], %[a3]\n\t"
+                     "s_nop 1\n\t"
+                     "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0xf bank_mask:0x8\n\t"
+                     "v_lshlrev_b32 %[addr], 4, %[addr]"
+                     : [addr] "=&v"(addr), [t] "=&v"(t)
+                     : [a0] "s"(a0), [a1] "s"(a1), [a2] "s"(a2), [a3] "s"(a3));
+    else
+        asm volatile("v_mov_b32 %[addr], %[a0]\n\t"
+                     "v_mov_b32 %[t], %[a1]\n\t"
+                     "s_nop 1\n\t"
+                     "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x2 bank_mask:0xf\n\t"
+                     "v_mov_b32 %[t], %[a2]\n\t"
+                     "s_nop 1\n\t"
+                     "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x4 bank_mask:0xf\n\t"
+                     "v_mov_b32 %[t], %[a3]\n\t"
+                     "s_nop 1\n\t"
+                     "v_mov_b32_dpp %[addr], %[t] quad_perm:[0,1,2,3] row_mask:0x8 bank_mask:0xf\n\t"
+                     "v_lshlrev_b32 %[addr], 4, %[addr]"
+                     : [addr] "=&v"(addr), [t] "=&v"(t)
+                     : [a0] "s"(a0), [a1] "s"(a1), [a2] "s"(a2), [a3] "s"(a3));
     return addr;
 }
 // orders one wave's LDS writes before its later LDS reads (the LDS serves a wave's instructions in order; this only keeps
@@ -382,13 +408,13 @@ __device__ __forceinline__ void wave_lds_sync()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 // The walk itself: turn(addr) is called, with the lanes of the quadrants that still have a hit, once per loop turn.
-template <typename Turn>
+template <bool BANKED = false, typename Turn>
 __device__ __forceinline__ void quadrant_walk(QuadrantHits &hits, uint32_t stage_base, Turn &&turn)
 {
     // (the exit is taken from the scalar masks, not from the lanes' addresses: an exit test that the optimizer can fold
     // into the per-lane test below makes the loop, and the masks it carries, divergent in the compiler's eyes)
     while (quadrant_pending(hits)) {
-        const uint32_t addr = quadrant_next_hit(hits);
+        const uint32_t addr = quadrant_next_hit<BANKED>(hits);
         if (addr != kNoHit) turn(addr + stage_base);
     }
 }
