@@ -105,32 +105,36 @@ __global__ void __launch_bounds__(256) max_weights_global_kernel(
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ TileStage<256> st;
+    __shared__ uint16_t s_reach[256];                  // per staged slot: the quadrants of the tile it can reach
     const uint32_t tile = blockIdx.x;
-    const uint32_t t = threadIdx.x;
+    const uint32_t t = threadIdx.x, wave = t >> 6, lane = t & 63;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
-    const uint32_t x = x0 + (t & 15), y = y0 + (t >> 4);
+    uint32_t local_x, local_y;
+    subtile_pixel(t, local_x, local_y);                // a wave = an 8x8 sub-tile, walked by quadrants
+    const uint32_t x = x0 + local_x, y = y0 + local_y;
     const bool inside = x < width && y < height;
-    const PixelTerms pt = pixel_terms(t & 15, t >> 4, 16);
+    const PixelTerms pt = pixel_terms(local_x, local_y, 16);
     const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
     float T = 1.0f;
     bool done = !inside;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 256) {
         if (__syncthreads_count(done) == 256) break;
-        tile_stage_load<MODE, 256, false>(st, prim, inst, base + t, last, t, cx, cy);
+        s_reach[t] = (uint16_t)tile_stage_load<MODE, 256, false, kCullAlpha, true>(st, prim, inst, base + t, last, t, cx, cy);
         __syncthreads();
-        const int nb = last - base < 256u ? (int)(last - base) : 256;
-        uint32_t addr = stage_address(st);
-        for (int j = 0; !done && j < nb; ++j, stage_advance(addr)) {
+        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
+        subtile_walk(s_reach, stage_base, last - base < 256u ? last - base : 256u, wave, lane,
+                     [&]() { return __ballot(!done) == 0; },
+                     [&](uint32_t addr) {
             TileFrag f;
-            if (!tile_frag_cutoff<256>(addr, pt, f)) continue;
+            if (done || !tile_frag_cutoff<256>(addr, pt, f)) return;
             f.den_rcp = rcp_exact(f.den);
-            if (!tile_frag_alpha<MODE>(stage_opacity<256>(addr), f)) continue;
+            if (!tile_frag_alpha<MODE>(stage_opacity<256>(addr), f)) return;
             const float w = T * f.alpha;
             T *= 1.0f - f.alpha;
             if (T < kTransmittanceThreshold) done = true;
             if (!(w < weight_threshold)) raise_max(max_weights, stage_index<256>(addr), w);
-        }
+        });
     }
 }
 
