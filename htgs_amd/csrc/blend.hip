@@ -541,6 +541,55 @@ __global__ void __launch_bounds__(64) check_tile_cull_kernel(
     }
 }
 
+// The same for the 16x16 tiles of ALPHA_BLEND_GLOBAL_ORDERING (sixteen quadrants per tile): every thread evaluates its
+// pixel for every staged instance, the waves note which quadrants are reached, and one thread per instance compares.
+__global__ void __launch_bounds__(256) check_tile_cull_16_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t grid_w,
+    unsigned long long *__restrict__ counts)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
+    __shared__ TileStage<256> st;
+    __shared__ uint32_t s_reach[256], s_reached[256];
+    const uint32_t tile = blockIdx.x, t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
+    uint32_t local_x, local_y;
+    subtile_pixel(t, local_x, local_y);
+    const PixelTerms pt = pixel_terms(local_x, local_y, 16);
+    const float cx = tile_centre(x0, 16), cy = tile_centre(y0, 16);
+    unsigned long long seen = 0, empty = 0, missed = 0, wrong = 0;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    for (uint32_t base = first; base < last; base += 256) {
+        __syncthreads();
+        s_reach[t] = tile_stage_load<MODE, 256, false, kCullAlpha, true>(st, prim, inst, base + t, last, t, cx, cy);
+        s_reached[t] = 0u;
+        __syncthreads();
+        const int nb = last - base < 256u ? (int)(last - base) : 256;
+        uint32_t addr = stage_address(st);
+        for (int j = 0; j < nb; ++j, stage_advance(addr)) {
+            TileFrag f;
+            bool pass = tile_frag_cutoff<256>(addr, pt, f);
+            if (pass) {
+                f.den_rcp = rcp_exact(f.den);
+                pass = tile_frag_alpha<MODE>(stage_opacity<256>(addr), f);
+            }
+            const uint64_t reached = __ballot(pass);
+            uint32_t bits = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) bits |= (((reached >> (16 * q)) & 0xffffu) != 0 ? 1u : 0u) << (4 * wave + q);
+            if (lane == 0 && bits) atomicOr(&s_reached[j], bits);
+        }
+        __syncthreads();
+        if (t < (uint32_t)nb) {
+            const uint32_t kept = s_reach[t], reached = s_reached[t];
+            ++seen; empty += reached == 0; missed += kept == 0; wrong += (unsigned)__builtin_popcount(reached & ~kept);
+        }
+    }
+    if (seen) {
+        atomicAdd(counts, seen); atomicAdd(counts + 1, empty); atomicAdd(counts + 2, missed);
+        if (wrong) atomicAdd(counts + 3, wrong);
+    }
+}
+
 template <int K, bool FAST>
 static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
@@ -628,13 +677,16 @@ extern "C" int htgs_check_tile_cull(const htgs_frame *f, int selector, unsigned 
 {
     if (!f || !counts) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: null pointer");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
-    if (f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING) return fail(HTGS_ERR_MODE, "htgs_check_tile_cull: the 16x16-tile mode does not cull");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: bad argument");
     if (!f->ranges || (f->n_instances > 0 && (!f->vals[selector] || !f->prim))) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: null pointer");
-    const uint32_t grid_w = div_up(f->width, 8), n_tiles = grid_w * div_up(f->height, 8);
+    if (frame_prim_floats(f) != HTGS_PRIM_FLOATS) return fail(HTGS_ERR_ARGUMENT, "htgs_check_tile_cull: reads records of HTGS_PRIM_FLOATS floats (prim_floats)");
+    const int tile = tile_size(f->mode);
+    const uint32_t grid_w = div_up(f->width, tile), n_tiles = grid_w * div_up(f->height, tile);
     hipStream_t s = (hipStream_t)f->stream;
     const float4 *prim = (const float4 *)f->prim;
-    if (f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K)
+    if (f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING)
+        hipLaunchKernelGGL(check_tile_cull_16_kernel, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector], prim, grid_w, counts);
+    else if (f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K)
         hipLaunchKernelGGL(check_tile_cull_kernel<HTGS_MODE_ALPHA_BLEND_FIRST_K>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], prim, grid_w, counts);
     else if (f->mode == HTGS_MODE_OIT_BLEND)
         hipLaunchKernelGGL(check_tile_cull_kernel<HTGS_MODE_OIT_BLEND>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], prim, grid_w, counts);

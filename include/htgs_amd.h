@@ -214,11 +214,12 @@ int htgs_update_3d_filter(const float *positions, const float *w2c, float *filte
  * compared (241 * 2^23) and the number that differ (0 on gfx950). */
 int htgs_check_reciprocal(unsigned long long *counts, void *stream);
 
-/* Self-check, no counterpart in the reference.  The 8x8-tile blend kernels leave out, batch by batch, the instances
- * whose Gaussian provably reaches no pixel of the tile (a bound on the least value of the cut-off / alpha quadratic
- * over the tile's pixels).  This call evaluates every instance of the frame's sorted list (after htgs_extract_ranges)
- * at all 64 pixels with the kernels' own tests and compares.  counts (device, four 64-bit words, zeroed by the
- * caller): instances looked at, instances that reach no pixel, instances left out, instances left out wrongly (0). */
+/* Self-check, no counterpart in the reference.  The blend kernels leave out, batch by batch and per 4x4 quadrant of the
+ * tile, the instances whose Gaussian provably reaches no pixel there (a bound on the least value of the cut-off / alpha
+ * quadratic over the quadrant's pixels).  This call evaluates every instance of the frame's sorted list (after
+ * htgs_extract_ranges) at every pixel of its tile with the kernels' own tests and compares.  counts (device, four
+ * 64-bit words, zeroed by the caller): instances looked at, instances that reach no pixel, instances left out of every
+ * quadrant, (instance, quadrant) pairs left out wrongly (0). */
 int htgs_check_tile_cull(const htgs_frame *f, int selector, unsigned long long *counts);
 
 #ifdef __cplusplus

@@ -1,5 +1,6 @@
-"""The 8x8-tile blend kernels leave out, batch by batch, the instances whose Gaussian provably reaches no pixel of the
-tile.  The library's self-check evaluates every instance at all 64 pixels with the kernels' own cut-off and alpha tests
+"""The blend kernels leave out, batch by batch and per 4x4 quadrant, the instances whose Gaussian provably reaches no pixel
+there (8x8 tiles: four quadrants; the 16x16 tiles of ALPHA_BLEND_GLOBAL_ORDERING: sixteen).  The library's self-check
+evaluates every instance at all pixels of its tile with the kernels' own cut-off and alpha tests
 and compares with the verdict of the staging lane: an instance that reaches a pixel must never be left out (then
 the walk over the kept instances gives the full walk's results bit for bit, which the parity tests confirm on the
 images), and nearly every instance that reaches none should be."""
@@ -52,17 +53,11 @@ def test_no_instance_that_reaches_a_pixel_is_left_out(cuda, config, n):
     base = make_scene(config, n)
     for name, scene in _variants(base):
         scene = scene.to(cuda)
-        for mode in (0, 1, 3):
+        for mode in (0, 1, 2, 3):
             print(f"case config={config} variant={name} mode={mode}", flush=True)
             seen, empty, left_out, wrong = _cull_counts(scene, mode)
             assert wrong == 0
             assert left_out <= empty
             if name == "plain" and config != 0:
                 assert seen > 10_000 and empty > 0
-                assert left_out >= 0.98 * empty
-
-
-def test_the_sixteen_pixel_tile_mode_is_refused(cuda):
-    scene = make_scene(0, 2000).to(cuda)
-    with pytest.raises(RuntimeError, match="does not cull"):
-        _cull_counts(scene, 2)
+                assert left_out >= (0.95 if mode == 2 else 0.98) * empty
