@@ -134,8 +134,11 @@ def test_self_check_entry_points_reject_bad_arguments():
     f.width = f.height = 64
     assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, None) == 2
     counts = (ctypes.c_ulonglong * 4)()
-    assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, counts) == 1               # the 16x16-tile mode does not cull
-    assert b"does not cull" in lib.htgs_last_error()
+    assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, counts) == 2               # no ranges
+    assert b"null pointer" in lib.htgs_last_error()
+    f.mode = 7
+    assert lib.htgs_check_tile_cull(ctypes.byref(f), 0, counts) == 1
+    assert b"unsupported rasterizer mode" in lib.htgs_last_error()
     assert lib.htgs_check_reciprocal(None, None) == 2
 
 
