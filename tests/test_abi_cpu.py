@@ -106,6 +106,27 @@ def test_entry_points_reject_bad_frames_without_touching_the_gpu():
     assert lib.htgs_preprocess(ctypes.byref(f)) == 2
 
 
+def test_record_size_is_checked_by_every_entry_point_that_reads_records():
+    """Inference entry points read 80-byte records, the training ones 128-byte records (htgs_frame.prim_floats); a frame
+    laid out for the other kind is refused before anything is launched."""
+    lib = _native.lib()
+    f = _native.Frame()
+    f.mode, f.width, f.height, f.n_primitives, f.n_instances = 0, 64, 64, 10, 10
+    assert _native.PRIM_FLOATS == 20 and _native.PRIM_FLOATS_TRAIN == 32
+    f.prim_floats = _native.PRIM_FLOATS_TRAIN
+    assert lib.htgs_blend(ctypes.byref(f), 0) == 2 and b"prim_floats" in lib.htgs_last_error()
+    assert lib.htgs_max_weights_blend(ctypes.byref(f), 0, None, ctypes.c_float(0.0)) == 2 and b"prim_floats" in lib.htgs_last_error()
+    counts = (ctypes.c_ulonglong * 4)()
+    for value in (0, _native.PRIM_FLOATS):
+        f.prim_floats = value
+        assert lib.htgs_blend_forward(ctypes.byref(f), 0) == 2 and b"prim_floats" in lib.htgs_last_error()
+        assert lib.htgs_blend_backward(ctypes.byref(f), 0) == 2 and b"prim_floats" in lib.htgs_last_error()
+        assert lib.htgs_blend(ctypes.byref(f), 0) == 2 and b"null pointer" in lib.htgs_last_error()
+    f.prim_floats = 24
+    assert lib.htgs_preprocess(ctypes.byref(f)) == 2
+    assert lib.htgs_create_instances(ctypes.byref(f)) == 2
+
+
 def test_instance_counts_beyond_32_bit_offsets_are_refused():
     """Offsets into the instance list are 32-bit, as in the reference; 0xffffffff is what the scan publishes when the
     tile counts do not fit.  The host refuses it, and so do the entry points that take the count."""
