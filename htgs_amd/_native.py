@@ -49,6 +49,7 @@ class Frame(ctypes.Structure):
         ("ranges", ctypes.c_void_p),
         ("long_tiles", ctypes.c_void_p),
         ("long_list_threshold", ctypes.c_int32),
+        ("tile_order", ctypes.c_void_p),
         ("n_instances", ctypes.c_uint64),
         ("keys", ctypes.c_void_p * 2),
         ("vals", ctypes.c_void_p * 2),
@@ -88,6 +89,7 @@ SYMBOLS = {
     "htgs_sort_passes": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "htgs_scan_tmp_words": (ctypes.c_size_t, [ctypes.c_int]),
     "htgs_sort_tmp_words": (ctypes.c_size_t, [ctypes.c_uint64]),
+    "htgs_tile_order_words": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "htgs_preprocess": (ctypes.c_int, [_FRAME_P]),
     "htgs_scan_offsets": (ctypes.c_int, [_FRAME_P]),
     "htgs_scan_offsets_static": (ctypes.c_int, [_FRAME_P]),

@@ -344,7 +344,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
     const float *__restrict__ grad_image, const float *__restrict__ VPM, float4 *__restrict__ grad_rows, float *__restrict__ helper_rows,
-    uint32_t width, uint32_t height, uint32_t grid_w)
+    uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order)
 {
     constexpr bool kHasTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = K > 0 ? K : 1;
@@ -355,7 +355,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
     __shared__ float s_tail_a[64 + 4];
     __shared__ float s_pos[HELPER ? 64 : 1][6];   // per pixel: (dL/dpx.w, dL/dpy.w) of a fragment -> its dL/dposition
     __shared__ uint8_t s_pairs[kBackwardWaves][256];   // per wave: the batch's (staging lane << 2 | quadrant) pairs, in list order
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
     const size_t np = (size_t)width * height;
@@ -488,7 +488,7 @@ template <bool HELPER>
 __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const float *__restrict__ image, const float *__restrict__ grad_image, const float *__restrict__ VPM,
-    float4 *__restrict__ grad_rows, float *__restrict__ helper_rows, uint32_t width, uint32_t height, uint32_t grid_w)
+    float4 *__restrict__ grad_rows, float *__restrict__ helper_rows, uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ TileStage<kGlobalBatch> st;
@@ -498,7 +498,7 @@ __global__ void __launch_bounds__(256) blend_global_backward_kernel(
     __shared__ float s_help[HELPER ? 16 : 1][kGlobalBatch];
     __shared__ uint16_t s_reach[kGlobalBatch];                // per staged Gaussian: the quadrants it can reach
     __shared__ uint32_t s_walked;                             // bit w: wave w walked this batch (its pixels were not all opaque)
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t t = threadIdx.x;
     const uint32_t lane = t & (kWave - 1), wave = t >> 6;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
@@ -933,11 +933,11 @@ static void launch_tail_backward(const htgs_frame *f, int sel, uint32_t grid_w, 
     if (f->dens_helper)
         hipLaunchKernelGGL((blend_tail_backward_moments_kernel<K, MODE, true>), dim3(n_tiles), dim3(64 * kBackwardWaves), 0, (hipStream_t)f->stream,
                            f->ranges, f->vals[sel], (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image,
-                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
     else
         hipLaunchKernelGGL((blend_tail_backward_moments_kernel<K, MODE, false>), dim3(n_tiles), dim3(64 * kBackwardWaves), 0, (hipStream_t)f->stream,
                            f->ranges, f->vals[sel], (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image,
-                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
 }
 
 }  // namespace htgs
@@ -992,11 +992,11 @@ extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
             if (f->dens_helper)
                 hipLaunchKernelGGL(blend_global_backward_kernel<true>, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
                                    (const float4 *)f->prim, f->image, f->grad_image, f->VPM, (float4 *)f->grad_rows,
-                                   f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+                                   f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
             else
                 hipLaunchKernelGGL(blend_global_backward_kernel<false>, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector],
                                    (const float4 *)f->prim, f->image, f->grad_image, f->VPM, (float4 *)f->grad_rows,
-                                   f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w);
+                                   f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
             break;
     }
     return check_launch("blend_backward");

@@ -157,10 +157,10 @@ template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
-    uint32_t *__restrict__ long_tiles, uint32_t long_threshold)
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, const uint32_t *__restrict__ tile_order)
 {
     __shared__ TileStage<64> st;
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
@@ -322,11 +322,11 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
 template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
     __shared__ TileStage<64> st;
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
     const uint32_t x = px.x, y = px.y;
@@ -390,11 +390,11 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 template <bool FAST>
 __global__ void __launch_bounds__(64) blend_oit_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw)
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_OIT_BLEND;
     __shared__ TileStage<64> st;
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
     const uint32_t x = px.x, y = px.y;
@@ -447,12 +447,12 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
 template <bool FAST>
 __global__ void __launch_bounds__(256) blend_global_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median)
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ TileStage<256> st;
     __shared__ uint16_t s_reach[256];                  // per staged slot: the quadrants of the tile it can reach
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t t = threadIdx.x, wave = t >> 6, lane = t & 63;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
     uint32_t local_x, local_y;
@@ -596,7 +596,7 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
     const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth, f->long_tiles, threshold);
+                       f->use_median_depth, f->long_tiles, threshold, f->tile_order);
     if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
         hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
@@ -607,7 +607,7 @@ static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, u
 {
     hipLaunchKernelGGL((blend_first_k_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth);
+                       f->use_median_depth, f->tile_order);
 }
 
 template <bool FAST>
@@ -639,11 +639,11 @@ static void launch_blend(const htgs_frame *f, int selector, uint32_t grid_w, uin
             break;
         case HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING:
             hipLaunchKernelGGL(blend_global_kernel<FAST>, dim3(n_tiles), dim3(256), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
-                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth);
+                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->tile_order);
             break;
         default:
             hipLaunchKernelGGL(blend_oit_kernel<FAST>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
-                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw);
+                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->tile_order);
             break;
     }
 }

@@ -418,6 +418,8 @@ __device__ __forceinline__ void quadrant_walk(QuadrantHits &hits, uint32_t stage
         if (addr != kNoHit) turn(addr + stage_base);
     }
 }
+// the tile a workgroup takes: the launch's blocks go through htgs_frame.tile_order (longest lists first) if there is one
+__device__ __forceinline__ uint32_t block_tile(const uint32_t *__restrict__ tile_order) { return tile_order ? tile_order[blockIdx.x] : blockIdx.x; }
 // pixel of a lane in an 8x8 tile that is walked by quadrants
 struct TilePixel {
     uint32_t x, y;

@@ -206,12 +206,62 @@ __global__ void __launch_bounds__(256) extract_ranges_kernel(const KeyT *__restr
     }
 }
 
-// zeroes p[0, n) and, if given, the four words at `also`
-__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n, uint32_t *also)
+// zeroes p[0, n) and, if given, the four words at `also` and the kOrderWords words at `also_order`
+constexpr uint32_t kOrderBuckets = 132;                   // (130 in use)
+constexpr uint32_t kOrderWords = 2 * kOrderBuckets;       // bin totals, bin cursors
+__global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n, uint32_t *also, uint32_t *also_order)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = 0;
     if (i < 4 && also) also[i] = 0;
+    if (i < kOrderWords && also_order) also_order[i] = 0;
+}
+
+// The order in which the blend kernels take the tiles: longest lists first.  One workgroup walks one tile, the hardware
+// hands out workgroups in index order, and lists differ in length by an order of magnitude; with the long ones at the
+// end of the launch a few compute units finish them while the rest of the device idles (blend of 3 M Gaussians at
+// 1080p: 1.43 ms in tile order, 1.30 ms longest first, 1.31 ms with the bins used here).  Tiles are binned by list
+// length, four bins per power of two, and laid out bin after bin (a counting sort; the order inside a bin is whatever
+// the atomics give, which no result depends on -- keeping it fixed costs 0.02 ms more and gains nothing).
+// order: [n_tiles] tiles, then kOrderBuckets bin totals and kOrderBuckets bin cursors, zeroed beforehand.
+__device__ __forceinline__ uint32_t order_bucket(uint32_t length)
+{
+    if (length == 0) return 129u;                          // empty lists last
+    const uint32_t p = 31u - (uint32_t)__builtin_clz(length);
+    const uint32_t sub = p >= 2u ? (length >> (p - 2u)) & 3u : (length << (2u - p)) & 3u;
+    return 128u - (4u * p + sub);                          // 1 .. 128, longer lists first
+}
+__global__ void __launch_bounds__(256) tile_order_count_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t n_tiles)
+{
+    __shared__ uint32_t count[kOrderBuckets];
+    if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t tile = blockIdx.x * 256 + threadIdx.x;
+    if (tile < n_tiles) atomicAdd(&count[order_bucket(ranges[2 * tile + 1] - ranges[2 * tile])], 1u);
+    __syncthreads();
+    if (threadIdx.x < kOrderBuckets && count[threadIdx.x]) atomicAdd(order + n_tiles + threadIdx.x, count[threadIdx.x]);
+}
+__global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t n_tiles)
+{
+    __shared__ uint32_t count[kOrderBuckets], base[kOrderBuckets];
+    if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t tile = blockIdx.x * 256 + threadIdx.x;
+    uint32_t bucket = 0, rank = 0;
+    if (tile < n_tiles) {
+        bucket = order_bucket(ranges[2 * tile + 1] - ranges[2 * tile]);
+        rank = atomicAdd(&count[bucket], 1u);
+    }
+    __syncthreads();
+    if (threadIdx.x < kOrderBuckets && count[threadIdx.x]) {
+        // where the bin starts (the totals of the bins before it) + what other workgroups have taken of it
+        const uint32_t *totals = order + n_tiles;
+        uint32_t start = 0;
+        for (uint32_t b = 0; b < threadIdx.x; ++b) start += totals[b];
+        base[threadIdx.x] = start + atomicAdd(order + n_tiles + kOrderBuckets + threadIdx.x, count[threadIdx.x]);
+    }
+    __syncthreads();
+    if (tile < n_tiles) order[base[bucket] + rank] = tile;
 }
 
 // Scratch of htgs_scan_offsets_static: the per-block sums of the scan, held in the library's own device image so
@@ -322,6 +372,14 @@ extern "C" int htgs_create_instances(const htgs_frame *f)
     return check_launch("create_instances");
 }
 
+extern "C" size_t htgs_tile_order_words(int mode, int width, int height)
+{
+    if (mode < 0 || mode > 3 || width <= 0 || height <= 0) return 0;
+    const int tile = tile_size(mode);
+    const size_t n_tiles = (size_t)div_up(width, tile) * div_up(height, tile);
+    return n_tiles + kOrderWords;
+}
+
 extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
 {
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: null frame");
@@ -330,7 +388,9 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
     hipStream_t s = (hipStream_t)f->stream;
     const int tile = tile_size(f->mode);
     const size_t n_tiles = (size_t)div_up(f->width, tile) * div_up(f->height, tile);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((2 * n_tiles + 255) / 256)), dim3(256), 0, s, f->ranges, 2 * n_tiles, f->long_tiles);
+    const size_t to_zero = 2 * n_tiles > kOrderWords ? 2 * n_tiles : kOrderWords;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((to_zero + 255) / 256)), dim3(256), 0, s, f->ranges, 2 * n_tiles, f->long_tiles,
+                       f->tile_order ? f->tile_order + n_tiles : nullptr);
     if (f->n_instances > 0) {
         if (!f->keys[selector]) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: null pointer");
         if ((uintptr_t)f->keys[selector] & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: keys must be 16-byte aligned");
@@ -343,6 +403,11 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
             hipLaunchKernelGGL((extract_ranges_kernel<uint32_t, 0>), grid, block, 0, s, (const uint32_t *)f->keys[selector], f->ranges, f->n_instances);
         else
             hipLaunchKernelGGL((extract_ranges_kernel<uint16_t, 0>), grid, block, 0, s, (const uint16_t *)f->keys[selector], f->ranges, f->n_instances);
+    }
+    if (f->tile_order) {
+        const dim3 grid((unsigned)((n_tiles + 255) / 256)), block(256);
+        hipLaunchKernelGGL(tile_order_count_kernel, grid, block, 0, s, f->ranges, f->tile_order, (uint32_t)n_tiles);
+        hipLaunchKernelGGL(tile_order_place_kernel, grid, block, 0, s, f->ranges, f->tile_order, (uint32_t)n_tiles);
     }
     return check_launch("extract_ranges");
 }

@@ -19,13 +19,13 @@ __device__ __forceinline__ void raise_max(uint32_t *__restrict__ max_weights, ui
 template <int K, int MODE>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) max_weights_tile_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold)
+    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold, const uint32_t *__restrict__ tile_order)
 {
     constexpr bool kCore = MODE != HTGS_MODE_OIT_BLEND;
     constexpr bool kTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = kCore ? K : 1;
     __shared__ TileStage<64> st;
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
     const bool inside = px.inside;
@@ -101,12 +101,12 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 
 __global__ void __launch_bounds__(256) max_weights_global_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold)
+    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING;
     __shared__ TileStage<256> st;
     __shared__ uint16_t s_reach[256];                  // per staged slot: the quadrants of the tile it can reach
-    const uint32_t tile = blockIdx.x;
+    const uint32_t tile = block_tile(tile_order);
     const uint32_t t = threadIdx.x, wave = t >> 6, lane = t & 63;
     const uint32_t x0 = (tile % grid_w) * 16, y0 = (tile / grid_w) * 16;
     uint32_t local_x, local_y;
@@ -142,7 +142,7 @@ template <int K, int MODE>
 static void launch_tile(const htgs_frame *f, int sel, uint32_t *max_weights, float thr, uint32_t grid_w, uint32_t n_tiles)
 {
     hipLaunchKernelGGL((max_weights_tile_kernel<K, MODE>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
-                       (const float4 *)f->prim, max_weights, (uint32_t)f->width, (uint32_t)f->height, grid_w, thr);
+                       (const float4 *)f->prim, max_weights, (uint32_t)f->width, (uint32_t)f->height, grid_w, thr, f->tile_order);
 }
 
 template <int MODE>
@@ -195,7 +195,7 @@ extern "C" int htgs_max_weights_blend(const htgs_frame *f, int selector, float *
         case HTGS_MODE_OIT_BLEND: launch_tile<1, HTGS_MODE_OIT_BLEND>(f, selector, mw, weight_threshold, grid_w, n_tiles); break;
         default:
             hipLaunchKernelGGL(max_weights_global_kernel, dim3(n_tiles), dim3(256), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
-                               (const float4 *)f->prim, mw, (uint32_t)f->width, (uint32_t)f->height, grid_w, weight_threshold);
+                               (const float4 *)f->prim, mw, (uint32_t)f->width, (uint32_t)f->height, grid_w, weight_threshold, f->tile_order);
             break;
     }
     return check_launch("max_weights");

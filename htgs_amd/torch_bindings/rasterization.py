@@ -120,7 +120,7 @@ class FrameBuffers:
 
     def __init__(self, positions, scales, rotations, opacities, sh_0, sh_rest, settings: RasterizerSettings,
                  to_chw: bool = True, use_median_depth: bool = False, train: bool = False,
-                 pool: Optional[ScratchPool] = None, fast: bool = False, long_list_threshold: int = 0):
+                 pool: Optional[ScratchPool] = None, fast: bool = False, long_list_threshold: int = 0, order_tiles: bool = True):
         mode = _mode_value(settings.mode)
         if mode not in (0, 1, 2, 3):
             raise RuntimeError("unsupported rasterizer mode")
@@ -170,6 +170,9 @@ class FrameBuffers:
         self.ranges = self._scratch("ranges", 2 * self.n_tiles, torch.int32)[:2 * self.n_tiles].view(self.n_tiles, 2)
         # HYBRID_BLEND inference: the list of tiles with very long instance lists, which several waves walk together
         self.long_tiles = self._scratch("long_tiles", self.n_tiles + 4, torch.int32) if mode == 0 and not train else None
+        # the tiles in the order the blend kernels take them (longest lists first), written with the ranges
+        self.tile_order = (self._scratch("tile_order", self.lib.htgs_tile_order_words(mode, self.width, self.height), torch.int32)
+                           if order_tiles else None)
         self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
                                  dtype=torch.float32, device=dev)
         # the image-only fast path (``fast_rasterize``) writes no depth map
@@ -197,6 +200,7 @@ class FrameBuffers:
         f.scan_tmp, f.n_instances_dev = _ptr(self.scan_tmp), _ptr(self.n_instances_dev)
         f.ranges = _ptr(self.ranges)
         f.long_tiles = _ptr(self.long_tiles)
+        f.tile_order = _ptr(self.tile_order)
         f.long_list_threshold = int(long_list_threshold)      # 0: the library's default
         f.image, f.depth = _ptr(self.image), _ptr(self.depth)
         f.to_chw, f.use_median_depth, f.fast_math = int(bool(to_chw)), int(bool(use_median_depth)), int(bool(fast))

@@ -84,6 +84,11 @@ typedef struct htgs_frame {
                                   NULL: every tile is walked by one wave (no counterpart in the reference, which
                                   does that) */
     int32_t long_list_threshold; /* 0 = the default (8192 instances) */
+    uint32_t *tile_order;      /* htgs_tile_order_words() words or NULL.  Written by htgs_extract_ranges: the n_tiles tiles,
+                                  longest lists first (binned by length, four bins per power of two), then scratch of
+                                  that stage.  Every kernel that walks tile lists takes its tiles in this order, so the long
+                                  lists are not left for the end of the launch; results do not depend on it.  NULL:
+                                  tile order (no counterpart in the reference) */
     /* ---- per-instance scratch (PerInstanceBuffers, buffer_utils.h:56-84) ---- */
     uint64_t n_instances;      /* host copy of *n_instances_dev, needed from htgs_create_instances on */
     void *keys[2];             /* [n_instances] of htgs_key_bytes() each, ping-pong, 16-byte aligned */
@@ -135,6 +140,8 @@ int htgs_key_bytes(int mode, int width, int height);
 int htgs_sort_passes(int mode, int width, int height);
 size_t htgs_scan_tmp_words(int n_primitives);
 size_t htgs_sort_tmp_words(uint64_t n_instances);
+/* size of htgs_frame.tile_order in 32-bit words (0 for an unsupported mode or an empty image) */
+size_t htgs_tile_order_words(int mode, int width, int height);
 
 /* preprocess_cu (R/include/<mode>/kernels/inference.cuh:10-76): cull, exact perspective bounds,
  * VPMT rows, MT3, SH colour.  Writes n_touched for every Gaussian, bounds and prim for visible ones. */

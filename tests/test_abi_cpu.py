@@ -85,6 +85,8 @@ def test_helper_functions():
             assert oracle.end_bit(fr) == lib.htgs_end_bit(mode, w, h)
     assert lib.htgs_scan_tmp_words(0) >= 1 and lib.htgs_scan_tmp_words(3_000_000) >= 3_000_000 // 2048
     assert lib.htgs_sort_tmp_words(0) >= 256 and lib.htgs_sort_tmp_words(20_000_000) >= 256 * (20_000_000 // 4096)
+    assert lib.htgs_tile_order_words(0, 1920, 1080) == 32400 + 264 and lib.htgs_tile_order_words(2, 1920, 1080) == 8160 + 264
+    assert lib.htgs_tile_order_words(0, 8, 8) == 1 + 264 and lib.htgs_tile_order_words(9, 8, 8) == 0
 
 
 def test_entry_points_reject_bad_frames_without_touching_the_gpu():
