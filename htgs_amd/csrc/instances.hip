@@ -56,38 +56,27 @@ __global__ void __launch_bounds__(kScanBlock) scan_reduce_kernel(const uint32_t 
     if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
 }
 
-// pass 2: one block turns the tile sums into exclusive tile offsets and publishes the grand total.  Offsets are
-// 32-bit as in the reference; a frame whose counts add up to more than 2^32 - 2 publishes 0xffffffff, which no valid
-// frame produces, so that the host can refuse it instead of sizing its buffers from a wrapped sum.
-__global__ void __launch_bounds__(kScanBlock) scan_tiles_kernel(uint32_t *__restrict__ tile_sums, int n_tiles, uint32_t *__restrict__ total_out)
+// pass 2: scan inside each tile and add the tile's offset, which every block sums up for itself from the tile sums
+// before it (a few hundred to a few thousand words from L2 -- cheaper than a launch in between that scans them once).
+// Thread t owns items [t*8, t*8+8) of the tile.  The last block publishes the grand total.  Offsets are 32-bit as in
+// the reference; a frame whose counts add up to more than 2^32 - 2 publishes 0xffffffff, which no valid frame
+// produces, so that the host can refuse it instead of sizing its buffers from a wrapped sum.
+__global__ void __launch_bounds__(kScanBlock) scan_apply_kernel(const uint32_t *__restrict__ in, const uint32_t *__restrict__ tile_sums,
+                                                               uint32_t *__restrict__ out, uint32_t *__restrict__ total_out, int n)
 {
     __shared__ uint32_t wave_sums[kScanBlock / kWave];
-    __shared__ unsigned long long s_wide[kScanBlock];
-    uint32_t carry = 0;
-    unsigned long long wide = 0;             // this thread's share of the same sum without wrap-around
-    for (int start = 0; start < n_tiles; start += kScanBlock) {
-        const int i = start + threadIdx.x;
-        const uint32_t v = i < n_tiles ? tile_sums[i] : 0u;
-        uint32_t total;
-        const uint32_t inc = block_inclusive_scan(v, wave_sums, &total);
-        if (i < n_tiles) tile_sums[i] = carry + inc - v;
-        carry += total;
-        wide += v;
-    }
-    s_wide[threadIdx.x] = wide;
+    __shared__ unsigned long long s_wide[kScanBlock / kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    unsigned long long before = 0;                         // without wrap-around, for the check of the total
+    for (uint32_t i = threadIdx.x; i < blockIdx.x; i += kScanBlock) before += tile_sums[i];
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) before += (unsigned long long)__shfl_xor((long long)before, d, kWave);
+    if (lane == 0) s_wide[wave] = before;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned long long sum = 0;
-        for (int t = 0; t < kScanBlock; ++t) sum += s_wide[t];
-        *total_out = sum > 0xfffffffeull ? 0xffffffffu : carry;
-    }
-}
+    before = 0;
+#pragma unroll
+    for (int w = 0; w < kScanBlock / kWave; ++w) before += s_wide[w];
 
-// pass 3: scan inside each tile, add the tile offset.  Thread t owns items [t*8, t*8+8) of the tile.
-__global__ void __launch_bounds__(kScanBlock) scan_apply_kernel(const uint32_t *__restrict__ in, const uint32_t *__restrict__ tile_offsets,
-                                                               uint32_t *__restrict__ out, int n)
-{
-    __shared__ uint32_t wave_sums[kScanBlock / kWave];
     const size_t base = (size_t)blockIdx.x * kScanTile + (size_t)threadIdx.x * kScanItems;
     uint32_t v[kScanItems];
     uint32_t s = 0;
@@ -98,11 +87,15 @@ __global__ void __launch_bounds__(kScanBlock) scan_apply_kernel(const uint32_t *
     }
     uint32_t total;
     const uint32_t inc = block_inclusive_scan(s, wave_sums, &total);
-    uint32_t run = tile_offsets[blockIdx.x] + inc - s;
+    uint32_t run = (uint32_t)before + inc - s;
 #pragma unroll
     for (int k = 0; k < kScanItems; ++k) {
         run += v[k];
         if (base + k < (size_t)n) out[base + k] = run;
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        const unsigned long long sum = before + total;
+        *total_out = sum > 0xfffffffeull ? 0xffffffffu : (uint32_t)sum;
     }
 }
 
@@ -243,8 +236,8 @@ __global__ void __launch_bounds__(256) tile_order_count_kernel(const uint32_t *_
 }
 __global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t n_tiles)
 {
-    __shared__ uint32_t count[kOrderBuckets], base[kOrderBuckets];
-    if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
+    __shared__ uint32_t count[kOrderBuckets], total[kOrderBuckets], base[kOrderBuckets];
+    if (threadIdx.x < kOrderBuckets) { count[threadIdx.x] = 0; total[threadIdx.x] = order[n_tiles + threadIdx.x]; }
     __syncthreads();
     const uint32_t tile = blockIdx.x * 256 + threadIdx.x;
     uint32_t bucket = 0, rank = 0;
@@ -255,9 +248,8 @@ __global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *_
     __syncthreads();
     if (threadIdx.x < kOrderBuckets && count[threadIdx.x]) {
         // where the bin starts (the totals of the bins before it) + what other workgroups have taken of it
-        const uint32_t *totals = order + n_tiles;
         uint32_t start = 0;
-        for (uint32_t b = 0; b < threadIdx.x; ++b) start += totals[b];
+        for (uint32_t b = 0; b < threadIdx.x; ++b) start += total[b];
         base[threadIdx.x] = start + atomicAdd(order + n_tiles + kOrderBuckets + threadIdx.x, count[threadIdx.x]);
     }
     __syncthreads();
@@ -306,9 +298,12 @@ static int launch_scan(const htgs_frame *f, uint32_t *tile_sums, const char *who
         return fail(HTGS_ERR_ARGUMENT, "%s: more than 2^20 tiles (images beyond 8192 x 8192 pixels are not supported)", who);
     const int tiles = n > 0 ? div_up(n, kScanTile) : 0;
     if (n > 0 && (!f->n_touched || !f->offsets)) return fail(HTGS_ERR_ARGUMENT, "%s: null pointer", who);
-    if (tiles > 0) hipLaunchKernelGGL(scan_reduce_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, n);
-    hipLaunchKernelGGL(scan_tiles_kernel, dim3(1), dim3(kScanBlock), 0, s, tile_sums, tiles, f->n_instances_dev);
-    if (tiles > 0) hipLaunchKernelGGL(scan_apply_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, f->offsets, n);
+    if (tiles > 0) {
+        hipLaunchKernelGGL(scan_reduce_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, n);
+        hipLaunchKernelGGL(scan_apply_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, f->offsets, f->n_instances_dev, n);
+    } else {
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(256), 0, s, f->n_instances_dev, (size_t)1, (uint32_t *)nullptr, (uint32_t *)nullptr);
+    }
     return check_launch("scan");
 }
 
