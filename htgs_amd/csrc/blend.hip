@@ -148,9 +148,10 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
-constexpr uint32_t kLongHeader = 4, kLongRounds = 3;
+constexpr uint32_t kLongHeader = 8, kLongRounds = 3;
 // One wave per tile.  A tile whose list is longer than long_threshold is not walked here but put on the list of long tiles
-// (long_tiles[0] = their number, long_tiles[1..3] = work counters, all zeroed with the ranges; long_tiles[4..] = the tiles) for blend_hybrid_long_kernel, if the
+// (long_tiles[0] = their number, [1..3] = work counters, [4] = workgroups done, all zeroed with the ranges and again by the
+// last workgroup of blend_hybrid_long_kernel; long_tiles[8..] = the tiles) for blend_hybrid_long_kernel, if the
 // caller provided that list: one wave walks one tile at some 200 ns per instance once it has a SIMD to itself, so a single
 // list of 300 000 instances would otherwise hold the launch for 70 ms.
 template <int K, bool FAST>
@@ -210,8 +211,18 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
         __syncthreads();
         const uint32_t j = s_next;
         if (j >= n_long) {
-            if (++round == kLongRounds) break;
-            continue;
+            if (++round < kLongRounds) continue;
+            // The last workgroup to get here clears the list's header, so that the list is empty again for the next
+            // launch of blend_hybrid_kernel on this frame (htgs_blend called again without htgs_extract_ranges).
+            if (threadIdx.x == 0) {
+                uint32_t *header = const_cast<uint32_t *>(long_tiles);
+                __threadfence();
+                if (atomicAdd(header + 4, 1u) == gridDim.x - 1) {
+#pragma unroll
+                    for (uint32_t k = 0; k < 5; ++k) header[k] = 0u;
+                }
+            }
+            break;
         }
         const uint32_t tile = long_tiles[kLongHeader + j];
         {

@@ -199,14 +199,14 @@ __global__ void __launch_bounds__(256) extract_ranges_kernel(const KeyT *__restr
     }
 }
 
-// zeroes p[0, n) and, if given, the four words at `also` and the kOrderWords words at `also_order`
+// zeroes p[0, n) and, if given, the eight words at `also` and the kOrderWords words at `also_order`
 constexpr uint32_t kOrderBuckets = 132;                   // (130 in use)
 constexpr uint32_t kOrderWords = 2 * kOrderBuckets;       // bin totals, bin cursors
 __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n, uint32_t *also, uint32_t *also_order)
 {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) p[i] = 0;
-    if (i < 4 && also) also[i] = 0;
+    if (i < 8 && also) also[i] = 0;
     if (i < kOrderWords && also_order) also_order[i] = 0;
 }
 

@@ -77,10 +77,11 @@ typedef struct htgs_frame {
     uint32_t *n_instances_dev; /* [1] total number of instances, written by the scan */
     /* ---- per-tile scratch (PerTileBuffers, buffer_utils.h:86-94) ---- */
     uint32_t *ranges;          /* [n_tiles,2] first,last+1 into the sorted instance list */
-    uint32_t *long_tiles;      /* [4 + n_tiles] or NULL.  HYBRID_BLEND inference: tiles whose list is longer than
-                                  long_list_threshold are collected here (word 0: their number, words 1-3: work
-                                  counters, all four zeroed by htgs_extract_ranges) and walked by several waves each,
-                                  the longest first; htgs_blend then also overwrites vals[1 - selector], see there.
+    uint32_t *long_tiles;      /* [8 + n_tiles] or NULL.  HYBRID_BLEND inference: tiles whose list is longer than
+                                  long_list_threshold are collected here (word 0: their number, words 1-4: work
+                                  counters; the eight header words are zeroed by htgs_extract_ranges, and again by
+                                  htgs_blend when it is done with the list) and walked by several waves each, the
+                                  longest first; htgs_blend then also overwrites vals[1 - selector], see there.
                                   NULL: every tile is walked by one wave (no counterpart in the reference, which
                                   does that) */
     int32_t long_list_threshold; /* 0 = the default (8192 instances) */

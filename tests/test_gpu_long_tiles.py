@@ -22,12 +22,22 @@ NEVER = 2 ** 31 - 1
 def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False):
     fb = FrameBuffers(*scene_gpu.gaussians(), scene_gpu.settings(RasterizerMode.HYBRID_BLEND, K), to_chw, median, fast=fast,
                       long_list_threshold=threshold)
-    fb.run()
+    fb.front()
+    fb.alloc_instances(fb.read_instance_count())
+    fb.create_instances()
+    fb.selector = fb.sort()
+    fb.extract_ranges()
+    ranges = fb.ranges.to(torch.int64)
+    long_tiles = int(((ranges[:, 1] - ranges[:, 0]) > (threshold if threshold else 8192)).sum())
+    fb.blend()
     torch.cuda.synchronize()
-    long_tiles, *taken = (int(v) for v in fb.long_tiles[:4].cpu())
-    assert min(taken) >= long_tiles               # every round went through the whole list
-    depth = None if fast else fb.depth.cpu().numpy()
-    return fb.image.cpu().numpy(), depth, long_tiles
+    assert not bool(fb.long_tiles[:8].any())      # the blend stage leaves the list empty for its next call
+    image, depth = fb.image.clone(), None if fast else fb.depth.clone()
+    fb.image.zero_()
+    fb.blend()                                    # again, without htgs_extract_ranges in between
+    torch.cuda.synchronize()
+    assert torch.equal(fb.image, image) and (fast or torch.equal(fb.depth, depth))
+    return image.cpu().numpy(), None if fast else depth.cpu().numpy(), long_tiles
 
 
 def with_coincident_copies(scene, copies):
