@@ -366,6 +366,7 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
         const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
         const bool inside = x < width && y < height;
         const size_t pix = inside ? (size_t)width * y + x : 0;
+        const size_t rp = record_pixel(tile, x, y), rnp = record_plane();     // (the forward pass's per-pixel records: tile by tile)
         const uint32_t ps = pixel_slot_of_lane(lane), pq = pixel_quadrant_of_lane(lane);
         float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f;
         if (inside) { g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix]; }
@@ -373,8 +374,8 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
             float4 tail = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             float tail_a = 0.0f;
             if (inside && kHasTail) {
-                const float r0 = tail_info[pix], r1 = tail_info[np + pix], r2 = tail_info[2 * np + pix];
-                const float asr = tail_info[3 * np + pix], T_tail = tail_info[4 * np + pix], T_core = tail_info[5 * np + pix];
+                const float r0 = tail_info[rp], r1 = tail_info[rnp + rp], r2 = tail_info[2 * rnp + rp];
+                const float asr = tail_info[3 * rnp + rp], T_tail = tail_info[4 * rnp + rp], T_core = tail_info[5 * rnp + rp];
                 const float w_tail = T_core * asr;                                   // backward.cuh:166
                 const float full = w_tail * (1.0f - T_tail);                         // :168
                 const float rdg = r0 * g0 + r1 * g1 + r2 * g2;
@@ -401,8 +402,8 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
                     uint32_t idx = 0xffffffffu;
                     float4 c = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
                     if (inside) {
-                        idx = core_idx[(size_t)i * np + pix];
-                        const float4 info = core_info[(size_t)i * np + pix];
+                        idx = core_idx[(size_t)i * rnp + rp];
+                        const float4 info = core_info[(size_t)i * rnp + rp];
                         c = make_float4(info.w * g0, info.w * g1, info.w * g2, info.x * g0 + info.y * g1 + info.z * g2);   // :154-155
                     }
                     s_idx[ps * KS + 4 * pq + i] = idx == 0xffffffffu ? idx : (idx << kSlotBits) | (uint32_t)i;

@@ -418,6 +418,11 @@ __device__ __forceinline__ void quadrant_walk(QuadrantHits &hits, uint32_t stage
         if (addr != kNoHit) turn(addr + stage_base);
     }
 }
+// The per-pixel records of the training pass are kept tile by tile: the 64 pixels of an 8x8 tile, row-major, are
+// contiguous, so a tile's workgroup writes and reads whole lines whatever order the tiles are taken in.  A record plane
+// has 64 entries per tile of the launch (gridDim.x tiles, the pixels beyond the image included).
+__device__ __forceinline__ size_t record_pixel(uint32_t tile, uint32_t x, uint32_t y) { return (size_t)tile * 64u + (y & 7u) * 8u + (x & 7u); }
+__device__ __forceinline__ size_t record_plane() { return (size_t)gridDim.x * 64u; }
 // the tile a workgroup takes: the launch's blocks go through htgs_frame.tile_order (longest lists first) if there is one
 __device__ __forceinline__ uint32_t block_tile(const uint32_t *__restrict__ tile_order) { return tile_order ? tile_order[blockIdx.x] : blockIdx.x; }
 // pixel of a lane in an 8x8 tile that is walked by quadrants

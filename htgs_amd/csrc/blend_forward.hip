@@ -71,6 +71,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     if (!inside) return;
 
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    const size_t rp = record_pixel(tile, x, y), rnp = record_plane();
     float c0[K], c1[K], c2[K];
 #pragma unroll
     for (int i = 0; i < K; ++i) {
@@ -105,15 +106,15 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
         w0 = s * tail0; w1 = s * tail1; w2 = s * tail2;
         t0 = tail0; t1 = tail1; t2 = tail2; t3 = asr; t4 = T_tail; t5 = T_core;
     }
-    tail_info[pix] = t0; tail_info[np + pix] = t1; tail_info[2 * np + pix] = t2;
-    tail_info[3 * np + pix] = t3; tail_info[4 * np + pix] = t4; tail_info[5 * np + pix] = t5;
+    tail_info[rp] = t0; tail_info[rnp + rp] = t1; tail_info[2 * rnp + rp] = t2;
+    tail_info[3 * rnp + rp] = t3; tail_info[4 * rnp + rp] = t4; tail_info[5 * rnp + rp] = t5;
 
     float n0 = 0.0f, n1 = 0.0f, n2 = 0.0f;
     T_core = 1.0f;
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         const bool skip = ci[i] == 0xffffffffu || T_core < kTransmittanceThreshold;
-        core_idx[(size_t)i * np + pix] = skip ? 0xffffffffu : ci[i];
+        core_idx[(size_t)i * rnp + rp] = skip ? 0xffffffffu : ci[i];
         float4 info = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if (!skip) {
             const float bw = T_core * c3[i];
@@ -128,7 +129,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             info.w = bw;
             T_core *= oma;
         }
-        core_info[(size_t)i * np + pix] = info;
+        core_info[(size_t)i * rnp + rp] = info;
     }
     image[pix] = r + w0; image[np + pix] = g + w1; image[2 * np + pix] = b + w2;
 }
@@ -178,6 +179,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     if (!inside) return;
 
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    const size_t rp = record_pixel(tile, x, y), rnp = record_plane();
     float r = 0.0f, g = 0.0f, b = 0.0f, T = 1.0f;
     float k0[K], k1[K], k2[K];
     bool open = true;
@@ -200,7 +202,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         const bool skip = ci[i] == 0xffffffffu || T < kTransmittanceThreshold;
-        core_idx[(size_t)i * np + pix] = skip ? 0xffffffffu : ci[i];
+        core_idx[(size_t)i * rnp + rp] = skip ? 0xffffffffu : ci[i];
         float4 info = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if (!skip) {
             const float bw = T * ca[i];
@@ -215,7 +217,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
             info.w = bw;
             T *= oma;
         }
-        core_info[(size_t)i * np + pix] = info;
+        core_info[(size_t)i * rnp + rp] = info;
     }
     image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
 }
@@ -256,6 +258,7 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     }
     if (!inside) return;
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
+    const size_t rp = record_pixel(tile, x, y), rnp = record_plane();
     float r = 0.0f, g = 0.0f, b = 0.0f, t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f, t4 = 0.0f, t5 = 0.0f;
     if (alpha_sum >= ModeCfg<MODE>::min_alpha) {
         const float asr = 1.0f / alpha_sum;
@@ -263,8 +266,8 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
         r = s * a0; g = s * a1; b = s * a2;
         t0 = a0; t1 = a1; t2 = a2; t3 = asr; t4 = T; t5 = 1.0f;   // row 5 plays the hybrid mode's T_core
     }
-    tail_info[pix] = t0; tail_info[np + pix] = t1; tail_info[2 * np + pix] = t2;
-    tail_info[3 * np + pix] = t3; tail_info[4 * np + pix] = t4; tail_info[5 * np + pix] = t5;
+    tail_info[rp] = t0; tail_info[rnp + rp] = t1; tail_info[2 * rnp + rp] = t2;
+    tail_info[3 * rnp + rp] = t3; tail_info[4 * rnp + rp] = t4; tail_info[5 * rnp + rp] = t5;
     image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
 }
 
@@ -314,22 +317,19 @@ __global__ void __launch_bounds__(256) blend_global_forward_kernel(
     image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
 }
 
-// (These two kernels take the tiles in tile order, not longest first: every tile, however short its list, ends with
-// 344 bytes of records per pixel, and with the short tiles bunched at the end of the launch those stores have no walks
-// to hide behind -- 0.72 instead of 0.67 ms for HYBRID at 1 M Gaussians / 1080p.)
 template <int K>
 static void launch_hybrid_forward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
 {
     hipLaunchKernelGGL((blend_hybrid_forward_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
                        (const float4 *)f->prim, f->image, f->core_idx, (float4 *)f->core_info, f->tail_info,
-                       (uint32_t)f->width, (uint32_t)f->height, grid_w, nullptr);
+                       (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
 }
 template <int K>
 static void launch_first_k_forward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
 {
     hipLaunchKernelGGL((blend_first_k_forward_kernel<K>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
                        (const float4 *)f->prim, f->image, f->core_idx, (float4 *)f->core_info,
-                       (uint32_t)f->width, (uint32_t)f->height, grid_w, nullptr);
+                       (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
 }
 
 }  // namespace htgs

@@ -271,8 +271,9 @@ class FrameBuffers:
 
     # ---- training ---------------------------------------------------------------------------
     def alloc_pixel_records(self):
-        """PerPixelBuffers of the reference (R/include/hybrid_blend/buffer_utils.h:96-108), pixel-minor."""
-        dev, P = self.device, self.width * self.height
+        """PerPixelBuffers of the reference (R/include/hybrid_blend/buffer_utils.h:96-108); here a plane holds the pixels
+        tile by tile (64 per 8x8 tile, row-major inside the tile), see ``records_in_image_order``."""
+        dev, P = self.device, 64 * self.n_tiles
         K = self.lib.htgs_effective_k(self.frame.K)
         if self.mode in (0, 1):
             self.core_idx = torch.empty((K, P), dtype=torch.int32, device=dev)
@@ -281,6 +282,14 @@ class FrameBuffers:
         if self.mode in (0, 3):
             self.tail_info = torch.empty((6, P), dtype=torch.float32, device=dev)
             self.frame.tail_info = _ptr(self.tail_info)
+
+    def records_in_image_order(self, records: torch.Tensor) -> torch.Tensor:
+        """``core_idx`` / ``tail_info`` (``[planes, 64 * n_tiles]``) or ``core_info`` (``[planes, 64 * n_tiles, 4]``) as
+        ``[planes, H * W(, 4)]``, the layout of the reference's per-pixel buffers."""
+        planes, tail = records.shape[0], records.shape[2:]
+        t = records.reshape(planes, self.grid_h, self.grid_w, 8, 8, *tail)
+        t = t.permute(0, 1, 3, 2, 4, *range(5, 5 + len(tail))).reshape(planes, 8 * self.grid_h, 8 * self.grid_w, *tail)
+        return t[:, :self.height, :self.width].reshape(planes, self.height * self.width, *tail)
 
     def forward_front(self):
         _native.check(self.lib.htgs_forward_front(self._ref))

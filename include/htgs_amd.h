@@ -103,10 +103,12 @@ typedef struct htgs_frame {
     int32_t fast_math;         /* htgs_blend only: image-only variant with the hardware's reciprocal and 2^x (one ulp each)
                                   instead of the exactly reproducible routines; depth is not written and may be NULL
                                   (the reference's fast_inference kernels, <mode>/kernels/fast_inference.cuh) */
-    /* ---- training: per-pixel records (PerPixelBuffers, buffer_utils.h:96-108), pixel-minor ---- */
-    uint32_t *core_idx;        /* [Keff,P] primitive of each blended core slot, 0xffffffff = none (modes 0, 1) */
-    float *core_info;          /* [Keff,P,4] (dC/dalpha of the slot, blending weight)        (modes 0, 1) */
-    float *tail_info;          /* [6,P] sum alpha*rgb (3), 1/sum alpha, T_tail, T_core       (modes 0, 3) */
+    /* ---- training: per-pixel records (PerPixelBuffers, buffer_utils.h:96-108).  Written by the forward blend, read by the
+     * backward blend, opaque to the caller.  R = 64 * n_tiles entries per plane, tile by tile: entry 64 * tile +
+     * 8 * (y & 7) + (x & 7) belongs to pixel (x, y), so that a tile's 64 pixels are contiguous ---- */
+    uint32_t *core_idx;        /* [Keff,R] primitive of each blended core slot, 0xffffffff = none (modes 0, 1) */
+    float *core_info;          /* [Keff,R,4] (dC/dalpha of the slot, blending weight)        (modes 0, 1) */
+    float *tail_info;          /* [6,R] sum alpha*rgb (3), 1/sum alpha, T_tail, T_core       (modes 0, 3) */
     /* ---- training: backward (backward_wrapper, rasterization_api.cu:178-363) ---- */
     const float *grad_image;   /* [3,H,W] upstream gradient */
     float *grad_rows;          /* [I,16] one row per instance, in creation order: dL/drgb (3), dL/dopacity,

@@ -51,11 +51,11 @@ def test_forward_records_and_gradients(cuda, config, n, mode, K):
     assert np.abs(image.cpu().numpy() - fwd["image"]).max() <= 1e-4
     Keff = oracle.effective_k(K)
     if mode in (0, 1):
-        np.testing.assert_array_equal(u32(fb.core_idx), fwd["core_idx"][:Keff])
-        np.testing.assert_allclose(fb.core_info.cpu().numpy(), fwd["core_info"][:Keff], rtol=1e-5, atol=1e-5)
+        np.testing.assert_array_equal(u32(fb.records_in_image_order(fb.core_idx)), fwd["core_idx"][:Keff])
+        np.testing.assert_allclose(fb.records_in_image_order(fb.core_info).cpu().numpy(), fwd["core_info"][:Keff], rtol=1e-5, atol=1e-5)
     if mode in (0, 3):
         rows = 6 if mode == 0 else 5
-        np.testing.assert_allclose(fb.tail_info.cpu().numpy()[:rows], fwd["tail_info"][:rows], rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(fb.records_in_image_order(fb.tail_info).cpu().numpy()[:rows], fwd["tail_info"][:rows], rtol=1e-5, atol=1e-6)
     for name, got in zip(NAMES, grads):
         assert_grad_close(name, got.cpu().numpy(), want[name])
 
