@@ -546,8 +546,9 @@ __device__ __forceinline__ TilePixel quadrant_tile_pixel(uint32_t tile, uint32_t
     p.y = y0 + local_y;
     p.inside = p.x < width && p.y < height;
     p.pt = pixel_terms(local_x, local_y, 8);
-    p.cx = tile_centre(x0, 8);
-    p.cy = tile_centre(y0, 8);
+    // (the same in every lane: held in scalar registers, two vector registers less in kernels that count them)
+    p.cx = bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(tile_centre(x0, 8))));
+    p.cy = bits_to_float((uint32_t)__builtin_amdgcn_readfirstlane((int)float_to_bits(tile_centre(y0, 8))));
     return p;
 }
 
