@@ -148,24 +148,46 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
-constexpr uint32_t kLongHeader = 8, kLongRounds = 3;
+constexpr uint32_t kLongHeader = 8, kLongRounds = 3, kLongParts = 32;
+// What a workgroup of blend_hybrid_long_kernel leaves of its part of a list: core, tail and the depth of a tie, per pixel.
+template <int K> constexpr uint32_t long_part_words() { return (3u * K + 7u) * 64u; }
+// The parts a list of this length is walked in by separate workgroups (1: by one).  A part is at least four times the
+// threshold long, and long enough that what the parts leave behind fits into the list's own stretch of the spare value buffer.
+template <int K>
+__device__ __forceinline__ uint32_t long_parts(uint32_t length, uint32_t long_threshold)
+{
+    const uint32_t least = 4u * long_threshold > long_part_words<K>() ? 4u * long_threshold : long_part_words<K>();
+    const uint32_t parts = length / least;
+    return parts < 1u ? 1u : parts > kLongParts ? kLongParts : parts;
+}
 // One wave per tile.  A tile whose list is longer than long_threshold is not walked here but put on the list of long tiles
-// (long_tiles[0] = their number, [1..3] = work counters, [4] = workgroups done, all zeroed with the ranges and again by the
-// last workgroup of blend_hybrid_long_kernel; long_tiles[8..] = the tiles) for blend_hybrid_long_kernel, if the
-// caller provided that list: one wave walks one tile at some 200 ns per instance once it has a SIMD to itself, so a single
-// list of 300 000 instances would otherwise hold the launch for 70 ms.
+// for blend_hybrid_long_kernel, if the caller provided that list: one wave walks one tile at some 200 ns per instance once it
+// has a SIMD to itself, so a single list of 300 000 instances would otherwise hold the launch for 70 ms.
+// long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = parts granted beyond one per
+// tile -- all zeroed with the ranges and again by the last workgroup of blend_hybrid_long_kernel; then 2 n_tiles words for
+// the entries (tile | part << 20 | (parts - 1) << 25: a tile is on the list once per part, and the parts beyond the first
+// of all tiles together are held to n_tiles, so the list cannot overflow) and n_tiles words that count a tile's finished parts.
 template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
-    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, const uint32_t *__restrict__ tile_order)
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, int in_parts, const uint32_t *__restrict__ tile_order)
 {
     __shared__ TileStage<64> st;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (lane == 0) long_tiles[kLongHeader + atomicAdd(long_tiles, 1u)] = tile;
+        if (lane == 0) {
+            const uint32_t n_tiles = gridDim.x;
+            uint32_t parts = in_parts ? long_parts<K>(last - first, long_threshold) : 1u;
+            if (parts > 1u) {
+                if (atomicAdd(long_tiles + 5, parts - 1u) + parts - 1u > n_tiles) parts = 1u;
+                else long_tiles[kLongHeader + 2u * n_tiles + tile] = 0u;
+            }
+            const uint32_t at = kLongHeader + atomicAdd(long_tiles, parts);
+            for (uint32_t part = 0; part < parts; ++part) long_tiles[at + part] = tile | part << 20 | (parts - 1u) << 25;
+        }
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -185,6 +207,32 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 // everything else in its tail, as in a single walk; what differs from the single walk is the order in which the tail's
 // sums are added (rounding) and which of two stored fragments of exactly equal depth is kept when a nearer one arrives.
 constexpr int kLongWaves = 16;
+// A core, a tail and a tie depth (3K + 7 rows of 64 lanes at from[]) join the running ones: they cover the stretch of the
+// list that follows.
+template <int K, bool FAST>
+__device__ __forceinline__ void hybrid_merge(const float *from, uint32_t lane, float (&cd)[K], float (&ca)[K], float (&ci)[K], HybridTail &tail,
+                                             float &tie)
+{
+    constexpr bool kTies = !FAST;
+    from += lane;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        float depth = from[(3 * i) * 64], alpha = from[(3 * i + 1) * 64], index = from[(3 * i + 2) * 64];
+        if (alpha > 0.0f) {                    // a filled slot
+            if (kTies && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
+            if (depth < cd[K - 1]) {
+                core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
+                if (kTies && alpha > 0.0f && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
+            }
+            hybrid_tail_add<FAST>(tail, depth, alpha);
+        }
+    }
+    tail.T *= from[(3 * K) * 64];
+    tail.c0 += from[(3 * K + 1) * 64]; tail.c1 += from[(3 * K + 2) * 64]; tail.c2 += from[(3 * K + 3) * 64];
+    tail.alpha += from[(3 * K + 4) * 64]; tail.depth += from[(3 * K + 5) * 64];
+    const float other = from[(3 * K + 6) * 64];
+    tie = other < tie ? other : tie;
+}
 constexpr uint32_t kLongListDefault = 8192;
 template <int K, bool FAST>
 __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
@@ -197,6 +245,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     __shared__ uint32_t s_next;
     __shared__ uint32_t s_redo[2];                    // the pixels (lanes) to walk again
     __shared__ uint32_t s_short[kLongWaves];          // how many instances of each share reach one of them
+    __shared__ uint32_t s_whole;                      // this workgroup finished the last part of its tile
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t n_long = long_tiles[0];
     if (n_long == 0) return;                          // (the ordinary frame)
@@ -219,21 +268,27 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                 __threadfence();
                 if (atomicAdd(header + 4, 1u) == gridDim.x - 1) {
 #pragma unroll
-                    for (uint32_t k = 0; k < 5; ++k) header[k] = 0u;
+                    for (uint32_t k = 0; k < 6; ++k) header[k] = 0u;
                 }
             }
             break;
         }
-        const uint32_t tile = long_tiles[kLongHeader + j];
+        const uint32_t entry = long_tiles[kLongHeader + j];
+        const uint32_t tile = entry & 0xfffffu, part = entry >> 20 & 31u, parts = (entry >> 25) + 1u;
+        // (the tile's list, and this entry's part of it: whole batches of 64)
+        const uint32_t tile_first = ranges[2 * tile], tile_last = ranges[2 * tile + 1];
+        const uint32_t tile_batches = (tile_last - tile_first + 63u) / 64u;
+        uint32_t first = tile_first + 64u * (uint32_t)((uint64_t)tile_batches * part / parts);
+        uint32_t last = tile_first + 64u * (uint32_t)((uint64_t)tile_batches * (part + 1u) / parts);
+        last = last < tile_last ? last : tile_last;
         {
-            const uint32_t length = ranges[2 * tile + 1] - ranges[2 * tile];
+            const uint32_t length = last - first;
             const uint32_t length_class = length > 16u * long_threshold ? 0u : length > 4u * long_threshold ? 1u : 2u;
             if (length_class != round) continue;
         }
-        const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
         const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
-        const uint32_t n_batches = (last - first + 63u) / 64u;
-        const uint32_t seg_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
+        uint32_t n_batches = (last - first + 63u) / 64u;
+        uint32_t seg_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
         uint32_t seg_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
         seg_last = seg_last < last ? seg_last : last;
         constexpr bool kTies = !FAST;
@@ -253,25 +308,41 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                 s_merge[3 * K + 6][lane] = tie;
             }
             __syncthreads();
+            if (wave == 0) hybrid_merge<K, FAST>(&s_merge[0][0], lane, cd, ca, ci, tail, tie);
+        }
+        if (parts > 1u) {
+            // One of several parts: what it came to goes to the tile's stretch of the spare value buffer (which is as long as the
+            // list and unused until pixels are walked again), and the workgroup that finds the other parts there already
+            // merges them all, in list order, and goes on with the whole tile.
+            float *const left = reinterpret_cast<float *>(shortlist + tile_first);
             if (wave == 0) {
+                float *mine = left + (size_t)part * long_part_words<K>() + lane;
 #pragma unroll
-                for (int i = 0; i < K; ++i) {
-                    float depth = s_merge[3 * i][lane], alpha = s_merge[3 * i + 1][lane], index = s_merge[3 * i + 2][lane];
-                    if (alpha > 0.0f) {                    // a filled slot
-                        if (kTies && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
-                        if (depth < cd[K - 1]) {
-                            core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
-                            if (kTies && alpha > 0.0f && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
-                        }
-                        hybrid_tail_add<FAST>(tail, depth, alpha);
-                    }
+                for (int i = 0; i < K; ++i) { mine[(3 * i) * 64] = cd[i]; mine[(3 * i + 1) * 64] = ca[i]; mine[(3 * i + 2) * 64] = ci[i]; }
+                mine[(3 * K) * 64] = tail.T; mine[(3 * K + 1) * 64] = tail.c0; mine[(3 * K + 2) * 64] = tail.c1;
+                mine[(3 * K + 3) * 64] = tail.c2; mine[(3 * K + 4) * 64] = tail.alpha; mine[(3 * K + 5) * 64] = tail.depth;
+                mine[(3 * K + 6) * 64] = tie;
+                __threadfence();
+                if (lane == 0) {
+                    uint32_t *finished = const_cast<uint32_t *>(long_tiles) + kLongHeader + 2u * grid_w * ((height + 7u) / 8u) + tile;
+                    s_whole = atomicAdd(finished, 1u) == parts - 1u;
                 }
-                tail.T *= s_merge[3 * K][lane];
-                tail.c0 += s_merge[3 * K + 1][lane]; tail.c1 += s_merge[3 * K + 2][lane]; tail.c2 += s_merge[3 * K + 3][lane];
-                tail.alpha += s_merge[3 * K + 4][lane]; tail.depth += s_merge[3 * K + 5][lane];
-                const float other = s_merge[3 * K + 6][lane];
-                tie = other < tie ? other : tie;
             }
+            __syncthreads();
+            if (!s_whole) continue;
+            if (wave == 0) {
+                __threadfence();
+                hybrid_tail_init(tail);
+                hybrid_core_init<K>(cd, ca, ci);
+                tie = __FLT_MAX__;
+                for (uint32_t other = 0; other < parts; ++other)
+                    hybrid_merge<K, FAST>(left + (size_t)other * long_part_words<K>(), lane, cd, ca, ci, tail, tie);
+            }
+            first = tile_first; last = tile_last; n_batches = tile_batches;
+            seg_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
+            seg_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
+            seg_last = seg_last < last ? seg_last : last;
+            __syncthreads();                               // (the parts are read before the shortlist overwrites them)
         }
         if (kTies) {
             // Equal depths matter where they can change the final core: a tie no deeper than its last entry (both
@@ -607,7 +678,7 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
     const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth, f->long_tiles, threshold, f->tile_order);
+                       f->use_median_depth, f->long_tiles, threshold, f->vals[selector ^ 1] != nullptr, f->tile_order);
     if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
         hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,

@@ -77,11 +77,13 @@ typedef struct htgs_frame {
     uint32_t *n_instances_dev; /* [1] total number of instances, written by the scan */
     /* ---- per-tile scratch (PerTileBuffers, buffer_utils.h:86-94) ---- */
     uint32_t *ranges;          /* [n_tiles,2] first,last+1 into the sorted instance list */
-    uint32_t *long_tiles;      /* [8 + n_tiles] or NULL.  HYBRID_BLEND inference: tiles whose list is longer than
-                                  long_list_threshold are collected here (word 0: their number, words 1-4: work
+    uint32_t *long_tiles;      /* [8 + 3 n_tiles] or NULL.  HYBRID_BLEND inference: tiles whose list is longer than
+                                  long_list_threshold are collected here (word 0: entries on the list, words 1-5: work
                                   counters; the eight header words are zeroed by htgs_extract_ranges, and again by
-                                  htgs_blend when it is done with the list) and walked by several waves each, the
-                                  longest first; htgs_blend then also overwrites vals[1 - selector], see there.
+                                  htgs_blend when it is done with the list; then 2 n_tiles words of entries -- a list
+                                  of several times the threshold is entered in up to 32 parts -- and a counter per
+                                  tile) and walked by several waves each, the longest first; htgs_blend then also
+                                  overwrites vals[1 - selector], see there.
                                   NULL: every tile is walked by one wave (no counterpart in the reference, which
                                   does that) */
     int32_t long_list_threshold; /* 0 = the default (8192 instances) */
@@ -168,10 +170,11 @@ int htgs_sort_instances(const htgs_frame *f, int *selector);
 int htgs_extract_ranges(const htgs_frame *f, int selector);
 /* blend_cu of the frame's mode (R/include/<mode>/kernels/inference.cuh:78-216).
  * HYBRID_BLEND with f->long_tiles: a second launch walks the tiles whose lists exceed long_list_threshold with sixteen
- * waves each and merges their K-buffers and tail sums; a pixel's result is that of the single walk up to the rounding
- * of the tail's sums (pixels at which fragments of exactly equal depth met are walked again in one piece).  That
- * launch uses the spare value buffer vals[1 - selector] as scratch (its content is lost; NULL: a slower path without
- * it).  Without long_tiles the stage reads vals[selector] only. */
+ * waves each (the longest in parts, by several such workgroups) and merges their K-buffers and tail sums; a pixel's
+ * result is that of the single walk up to the rounding of the tail's sums (pixels at which fragments of exactly equal
+ * depth met are walked again in one piece).  That launch uses the spare value buffer vals[1 - selector] as scratch
+ * (its content is lost; NULL: a slower path without it, one workgroup per tile).  Without long_tiles the stage reads
+ * vals[selector] only. */
 int htgs_blend(const htgs_frame *f, int selector);
 
 /* <mode>::inference split at its one host/device synchronisation point (inference.cu:118-119):

@@ -19,7 +19,7 @@ TOL = 1e-4
 NEVER = 2 ** 31 - 1
 
 
-def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False):
+def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False, in_parts=None):
     fb = FrameBuffers(*scene_gpu.gaussians(), scene_gpu.settings(RasterizerMode.HYBRID_BLEND, K), to_chw, median, fast=fast,
                       long_list_threshold=threshold)
     fb.front()
@@ -28,9 +28,13 @@ def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False):
     fb.selector = fb.sort()
     fb.extract_ranges()
     ranges = fb.ranges.to(torch.int64)
-    long_tiles = int(((ranges[:, 1] - ranges[:, 0]) > (threshold if threshold else 8192)).sum())
+    lengths = ranges[:, 1] - ranges[:, 0]
+    long_tiles = int((lengths > (threshold if threshold else 8192)).sum())
     fb.blend()
     torch.cuda.synchronize()
+    if in_parts is not None:                      # lists long enough to be walked in parts by several workgroups
+        part = max(4 * threshold, (3 * K + 7) * 64)
+        assert (int((lengths >= 2 * part).sum()) > 0) == in_parts, f"longest list {int(lengths.max())}, a part {part}"
     assert not bool(fb.long_tiles[:8].any())      # the blend stage leaves the list empty for its next call
     image, depth = fb.image.clone(), None if fast else fb.depth.clone()
     fb.image.zero_()
@@ -90,6 +94,25 @@ def test_long_tiles_with_fragments_of_equal_depth(cuda, K):
     err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
     print(f"  long tiles {long_tiles}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
     assert err_i <= TOL and err_d <= TOL
+
+
+@pytest.mark.parametrize("n,K,threshold,copies", [(150_000, 4, 200, 1), (150_000, 1, 64, 1), (300_000, 16, 500, 1), (30_000, 4, 200, 5)])
+def test_long_tiles_walked_in_parts(cuda, n, K, threshold, copies):
+    """Lists of many times the threshold are entered in parts, each walked by a workgroup of its own; the one that
+    finishes last merges what the parts left (in the tile's stretch of the spare value buffer) and ends the tile."""
+    print(f"case n={n} K={K} threshold={threshold} copies={copies} (parts)", flush=True)
+    scene = make_scene(3, n)
+    if copies > 1:
+        scene = with_coincident_copies(scene, copies)
+    ref = oracle_render(scene, 0, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, threshold, in_parts=True)
+    err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
+    print(f"  long tiles {long_tiles}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
+    assert err_i <= TOL and err_d <= TOL
+    if copies == 1:                               # (the fast variant does not walk pixels with equal depths again)
+        fast, _, _ = render(scene.to(cuda), K, threshold, fast=True)
+        single, _, _ = render(scene.to(cuda), K, NEVER, fast=True)
+        assert np.abs(fast - single).max() <= TOL
 
 
 def test_long_tiles_fast_variant(cuda):
