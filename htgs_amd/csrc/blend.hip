@@ -164,7 +164,9 @@ __device__ __forceinline__ uint32_t long_parts(uint32_t length, uint32_t long_th
 // for blend_hybrid_long_kernel, if the caller provided that list: one wave walks one tile at some 200 ns per instance once it
 // has a SIMD to itself, so a single list of 300 000 instances would otherwise hold the launch for 70 ms.
 // long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = parts granted beyond one per
-// tile -- all zeroed with the ranges and again by the last workgroup of blend_hybrid_long_kernel; then 2 n_tiles words for
+// tile -- all zeroed with the ranges and again by the last workgroup of blend_hybrid_long_kernel; [6], [7] = tiles with
+// pixels settled by a second look / walked again in one piece (upper half: of these, after a second look that ran out of
+// room) since the ranges were made (for the tests); then 2 n_tiles words for
 // the entries (tile | part << 20 | (parts - 1) << 25: a tile is on the list once per part, and the parts beyond the first
 // of all tiles together are held to n_tiles, so the list cannot overflow) and n_tiles words that count a tile's finished parts.
 template <int K, bool FAST>
@@ -198,6 +200,99 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     hybrid_walk<K, FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
     if (!px.inside) return;
     hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+}
+
+__device__ __forceinline__ float wave_total(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ float wave_product(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v *= __shfl_xor(v, o);
+    return v;
+}
+constexpr int kAgainPixels = 2;       // pixels a pass of hybrid_pixels_again takes at once
+constexpr int kAgainMost = 8;         // pixels of a tile beyond which they are walked again in one piece instead
+
+// The second look at the pixels of pixel_lanes, whose cores the merge could not settle: lanes = instances.  Every wave
+// goes through its share [first, last) of the tile's list once per kAgainPixels pixels and evaluates each instance at these
+// pixels with the walk's own arithmetic.  A fragment that cannot be in the pixel's final core -- farther than the merged
+// core's last entry (last_depth[pixel]: which depths the K nearest have is certain, which fragments of equal depth they
+// are is not), or too faint for the core -- joins the pixel's tail in sums[][j] (this wave's sums and product, to be combined
+// over the waves; the colour sums take every fragment); the others, the few that decide the core, are put down in list
+// order at `out` as (pixel, depth, alpha, index) for the walk's insertion to be replayed on them alone.  Returns their
+// number, or ~0u when `room` entries were not enough.  pass_done(pixels) is called, by the whole workgroup, after each pass.
+template <int K, typename PassDone>
+__device__ __forceinline__ uint32_t hybrid_pixels_again(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
+                                                        uint32_t last, uint32_t lane, float cx, float cy, uint64_t pixel_lanes,
+                                                        const float *last_depth, float (*sums)[6], uint32_t *__restrict__ out, uint32_t room,
+                                                        PassDone pass_done)
+{
+    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    uint32_t n_out = 0;
+    bool fits = true;
+    for (uint64_t todo = pixel_lanes; todo != 0;) {
+        uint32_t pixel[kAgainPixels];
+        PixelTerms pt[kAgainPixels];
+        float farthest[kAgainPixels];
+        HybridTail acc[kAgainPixels];
+#pragma unroll
+        for (int j = 0; j < kAgainPixels; ++j) {
+            pixel[j] = todo != 0 ? (uint32_t)__builtin_ctzll(todo) : 64u;
+            todo &= todo - 1;                                       // (0 stays 0)
+            uint32_t local_x, local_y;
+            quadrant_pixel(pixel[j] & 63u, local_x, local_y);
+            pt[j] = pixel_terms(local_x, local_y, 8);
+            farthest[j] = last_depth[pixel[j] & 63u];
+            hybrid_tail_init(acc[j]);
+        }
+        for (uint32_t base = first; base < last; base += 64) {
+            wave_lds_sync();
+            tile_stage_load<MODE, 64, true, kCullNone, true>(st, prim, inst, base + lane, last, lane, cx, cy);
+            wave_lds_sync();
+            const bool loaded = base + lane < last;
+            const uint32_t addr = stage_address(st) + 16u * lane;
+#pragma unroll
+            for (int j = 0; j < kAgainPixels; ++j) {
+                if (pixel[j] >= 64u) continue;                      // (wave-uniform)
+                TileFrag f;
+                const bool in_reach = tile_frag_cutoff<64>(addr, pt[j], f);
+                f.den_rcp = frag_rcp<false>(f.den);
+                const float4 col = stage_row<64, 5>(addr);
+                const bool fragment = tile_frag_alpha<MODE, false>(stage_opacity<64>(addr), f) && in_reach && loaded;
+                const float depth = tile_frag_depth<64>(addr, pt[j], f);
+                bool decides = false;
+                if (fragment) {
+                    acc[j].c0 = __builtin_fmaf(f.alpha, col.x, acc[j].c0);
+                    acc[j].c1 = __builtin_fmaf(f.alpha, col.y, acc[j].c1);
+                    acc[j].c2 = __builtin_fmaf(f.alpha, col.z, acc[j].c2);
+                    decides = depth <= farthest[j] && f.alpha >= kMinAlphaCore;
+                    if (!decides) hybrid_tail_add<false>(acc[j], depth, f.alpha);
+                }
+                const uint64_t deciding = __ballot(decides);
+                if (deciding != 0) {
+                    const uint32_t at = n_out + (uint32_t)__popcll(deciding & ((1ull << lane) - 1ull));
+                    n_out += (uint32_t)__popcll(deciding);
+                    fits = fits && n_out <= room;
+                    if (decides && fits) {
+                        out[4 * at] = pixel[j]; out[4 * at + 1] = float_to_bits(depth); out[4 * at + 2] = float_to_bits(f.alpha);
+                        out[4 * at + 3] = float_to_bits(col.w);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kAgainPixels; ++j) {
+            const float T = wave_product(acc[j].T), c0 = wave_total(acc[j].c0), c1 = wave_total(acc[j].c1), c2 = wave_total(acc[j].c2),
+                        alpha = wave_total(acc[j].alpha), depth = wave_total(acc[j].depth);
+            if (lane == 0) { sums[j][0] = T; sums[j][1] = c0; sums[j][2] = c1; sums[j][3] = c2; sums[j][4] = alpha; sums[j][5] = depth; }
+        }
+        pass_done(pixel);
+    }
+    return fits ? n_out : ~0u;
 }
 
 // The long tiles: a workgroup of kLongWaves waves takes a tile, every wave walks a contiguous share of the list (whole
@@ -246,6 +341,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     __shared__ uint32_t s_redo[2];                    // the pixels (lanes) to walk again
     __shared__ uint32_t s_short[kLongWaves];          // how many instances of each share reach one of them
     __shared__ uint32_t s_whole;                      // this workgroup finished the last part of its tile
+    __shared__ float s_last_depth[64];                // depth of the merged core's last entry
+    __shared__ float s_sums[kLongWaves][kAgainPixels][6], s_tails[64][6];   // tails of the pixels looked at again: per wave, whole
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t n_long = long_tiles[0];
     if (n_long == 0) return;                          // (the ordinary frame)
@@ -363,6 +460,69 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
             __syncthreads();
             const uint64_t redo_lanes = (uint64_t)s_redo[0] | (uint64_t)s_redo[1] << 32;
             if (redo_lanes != 0) {
+                bool others_done = false;                       // the pixels that need no second look are composited
+                if (shortlist != nullptr && __popcll(redo_lanes) <= kAgainMost) {
+                    // All waves look at these pixels again, lanes = instances (hybrid_pixels_again), into the tile's stretch of
+                    // the shortlist, four words per fragment that decides a core: a wave has a quarter as many entries as
+                    // its share has instances, which is ample unless depths coincide by the hundred -- then, and when the
+                    // pixels are many (a pass over the list serves kAgainPixels of them), the other way below is taken.
+                    others_done = true;
+                    if (wave == 0) {
+                        s_last_depth[lane] = cd[K - 1];
+                        if (px.inside && !redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+                    }
+                    __syncthreads();
+                    const uint32_t listed = hybrid_pixels_again<K>(
+                        st[wave], inst, prim, seg_first, seg_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, s_sums[wave], shortlist + seg_first,
+                        (seg_last - seg_first) / 4u, [&](const uint32_t (&pixel)[kAgainPixels]) {
+                            __syncthreads();
+                            if (wave == 0 && lane < (uint32_t)kAgainPixels) {      // the waves' sums of a pixel, in list order
+                                uint32_t mine = pixel[0];
+#pragma unroll
+                                for (int j = 1; j < kAgainPixels; ++j) mine = lane == (uint32_t)j ? pixel[j] : mine;
+                                if (mine < 64u) {
+                                    float T = 1.0f, sum[5] = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f };
+                                    for (int w = 0; w < kLongWaves; ++w) {
+                                        T *= s_sums[w][lane][0];
+#pragma unroll
+                                        for (int k = 0; k < 5; ++k) sum[k] += s_sums[w][lane][1 + k];
+                                    }
+                                    s_tails[mine][0] = T;
+#pragma unroll
+                                    for (int k = 0; k < 5; ++k) s_tails[mine][1 + k] = sum[k];
+                                }
+                            }
+                            __syncthreads();
+                        });
+                    if (lane == 0) s_short[wave] = listed;
+                    __syncthreads();
+                    bool settled = true;
+                    for (int w = 0; w < kLongWaves; ++w) settled = settled && s_short[w] != ~0u;
+                    __syncthreads();                            // (s_short is written again below)
+                    if (settled) {
+                        if (wave == 0) {
+                            // The walk's insertion, on the fragments that decide the cores alone, in list order; every pixel's lane
+                            // takes its own.
+                            hybrid_core_init<K>(cd, ca, ci);
+                            tail.T = s_tails[lane][0]; tail.c0 = s_tails[lane][1]; tail.c1 = s_tails[lane][2]; tail.c2 = s_tails[lane][3];
+                            tail.alpha = s_tails[lane][4]; tail.depth = s_tails[lane][5];
+                            for (uint32_t w = 0; w < (uint32_t)kLongWaves; ++w) {
+                                const uint32_t *entry = shortlist + first + 64u * (uint32_t)((uint64_t)n_batches * w / kLongWaves);
+                                for (uint32_t left = s_short[w]; left != 0; --left, entry += 4) {
+                                    float depth = bits_to_float(entry[1]), alpha = bits_to_float(entry[2]), index = bits_to_float(entry[3]);
+                                    if (lane == entry[0]) {
+                                        if (depth < cd[K - 1]) core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
+                                        hybrid_tail_add<false>(tail, depth, alpha);
+                                    }
+                                }
+                            }
+                            if (px.inside && redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+                        }
+                        if (threadIdx.x == 0) atomicAdd(const_cast<uint32_t *>(long_tiles) + 6, 1u);
+                        continue;
+                    }
+                }
+                if (threadIdx.x == 0) atomicAdd(const_cast<uint32_t *>(long_tiles) + 7, others_done ? 0x10001u : 1u);
                 if (shortlist != nullptr) {
                     uint32_t kept = 0;
                     for (uint32_t base = seg_first; base < seg_last; base += 64) {
@@ -377,7 +537,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                     __syncthreads();
                 }
                 if (wave == 0) {
-                    if (px.inside && !redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
+                    if (!others_done && px.inside && !redo)
+                        hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
                     hybrid_tail_init(tail);
                     hybrid_core_init<K>(cd, ca, ci);
                     if (shortlist != nullptr) {

@@ -17,6 +17,7 @@ pytestmark = pytest.mark.gpu
 
 TOL = 1e-4
 NEVER = 2 ** 31 - 1
+SECOND_LOOKS = []
 
 
 def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False, in_parts=None):
@@ -35,7 +36,10 @@ def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False, in_pa
     if in_parts is not None:                      # lists long enough to be walked in parts by several workgroups
         part = max(4 * threshold, (3 * K + 7) * 64)
         assert (int((lengths >= 2 * part).sum()) > 0) == in_parts, f"longest list {int(lengths.max())}, a part {part}"
-    assert not bool(fb.long_tiles[:8].any())      # the blend stage leaves the list empty for its next call
+    assert not bool(fb.long_tiles[:6].any())      # the blend stage leaves the list empty for its next call
+    # tiles with pixels at which depths coincided: settled by a second look at those pixels / walked again in one piece
+    # (of the latter, third number: after a second look for which the room did not do)
+    SECOND_LOOKS.append((int(fb.long_tiles[6]), int(fb.long_tiles[7]) & 0xffff, int(fb.long_tiles[7]) >> 16))
     image, depth = fb.image.clone(), None if fast else fb.depth.clone()
     fb.image.zero_()
     fb.blend()                                    # again, without htgs_extract_ranges in between
@@ -82,6 +86,34 @@ def test_long_tiles_layout_and_median_depth(cuda, to_chw, median):
     assert np.abs(depth - ref["depth"]).max() <= TOL
 
 
+def with_some_twins(scene, n_twins):
+    """``n_twins`` of the Gaussians once more at the same place with the same shape but other colours and opacities: a few
+    pixels per tile get two fragments of exactly equal depth."""
+    g = torch.Generator().manual_seed(12)
+    pick = torch.randperm(scene.positions.shape[0], generator=g)[:n_twins]
+    both = lambda t: torch.cat([t, t[pick]]).contiguous()
+    opacities, sh_0 = both(scene.opacities), both(scene.sh_0)
+    opacities[-n_twins:] = (opacities[-n_twins:] * 0.7 + 0.1)
+    sh_0[-n_twins:] += 0.3 * torch.randn(sh_0[-n_twins:].shape, generator=g)
+    return dataclasses.replace(scene, name=scene.name + "-twins", positions=both(scene.positions), scales=both(scene.scales),
+                               rotations=both(scene.rotations), opacities=opacities, sh_0=sh_0, sh_rest=both(scene.sh_rest))
+
+
+@pytest.mark.parametrize("config,n,K,threshold,twins", [(0, 3000, 4, 24, 150), (3, 150_000, 16, 1000, 300), (3, 150_000, 4, 200, 300)])
+def test_long_tiles_second_look_at_a_few_pixels(cuda, config, n, K, threshold, twins):
+    """Few pixels of a tile with fragments of equal depth: every wave looks at them again, lanes = instances, and the
+    insertion is replayed on the fragments that decide their cores."""
+    print(f"case config={config} n={n} K={K} threshold={threshold} twins={twins}", flush=True)
+    scene = with_some_twins(make_scene(config, n), twins)
+    ref = oracle_render(scene, 0, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, threshold)
+    second_looks, walked_again, _ = SECOND_LOOKS[-1]
+    err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
+    print(f"  long tiles {long_tiles}, second looks {second_looks}, walked again {walked_again}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
+    assert second_looks > 0
+    assert err_i <= TOL and err_d <= TOL
+
+
 @pytest.mark.parametrize("K", [4, 16])
 def test_long_tiles_with_fragments_of_equal_depth(cuda, K):
     """Coincident Gaussians: which of two stored fragments of equal depth leaves the core depends on the order of arrival in
@@ -90,7 +122,7 @@ def test_long_tiles_with_fragments_of_equal_depth(cuda, K):
     scene = with_coincident_copies(make_scene(0, 1500), 6)
     ref = oracle_render(scene, 0, K)
     image, depth, long_tiles = render(scene.to(cuda), K, 64)
-    assert long_tiles > 0
+    assert long_tiles > 0 and SECOND_LOOKS[-1][1] > 0
     err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
     print(f"  long tiles {long_tiles}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
     assert err_i <= TOL and err_d <= TOL
@@ -113,6 +145,28 @@ def test_long_tiles_walked_in_parts(cuda, n, K, threshold, copies):
         fast, _, _ = render(scene.to(cuda), K, threshold, fast=True)
         single, _, _ = render(scene.to(cuda), K, NEVER, fast=True)
         assert np.abs(fast - single).max() <= TOL
+
+
+def test_long_tiles_with_depths_that_coincide_by_the_hundred(cuda):
+    """A few pixels with so many fragments as deep as their core's last entry that these do not fit the room the second
+    look has for them: the pixels are then walked again in one piece."""
+    print("case a few tiny Gaussians 400 times each", flush=True)
+    scene = make_scene(0, 3000)
+    g = torch.Generator().manual_seed(13)
+    pick = torch.randperm(3000, generator=g)[:6]
+    often = lambda t: torch.cat([t, t[pick].repeat(400, *([1] * (t.dim() - 1)))]).contiguous()
+    scales, sh_0 = often(scene.scales), often(scene.sh_0)
+    scales[3000:] = 2e-4                                    # a pixel or two each
+    sh_0[3000:] += 0.3 * torch.randn(sh_0[3000:].shape, generator=g)
+    scene = dataclasses.replace(scene, name=scene.name + "-heaps", positions=often(scene.positions), scales=scales, rotations=often(scene.rotations),
+                                opacities=often(scene.opacities), sh_0=sh_0, sh_rest=often(scene.sh_rest))
+    ref = oracle_render(scene, 0, 4)
+    image, depth, long_tiles = render(scene.to(cuda), 4, 64)
+    print(f"  second looks {SECOND_LOOKS[-1][0]}, walked again {SECOND_LOOKS[-1][1]}, of these for want of room {SECOND_LOOKS[-1][2]}", flush=True)
+    assert long_tiles > 0 and SECOND_LOOKS[-1][2] > 0
+    err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
+    print(f"  long tiles {long_tiles}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
+    assert err_i <= TOL and err_d <= TOL
 
 
 def test_long_tiles_fast_variant(cuda):
