@@ -148,27 +148,107 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Tiles with very long lists (HYBRID_BLEND, ALPHA_BLEND_FIRST_K and OIT_BLEND, which walk all of a list): the kernel
+// with one wave per tile puts a tile whose list is longer than long_threshold on a list instead of walking it, if the
+// caller provided that list, and a second launch of workgroups of kLongWaves waves takes those: one wave walks one tile at some
+// 200 ns per instance once it has a SIMD to itself, so a single list of 300 000 instances would otherwise hold the
+// launch for 70 ms.
+// long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = parts granted beyond one per
+// tile -- all zeroed with the ranges and again by the last workgroup of the second launch; [6], [7] = HYBRID's tiles with
+// pixels settled by a second look / walked again in one piece (upper half: of these, after a second look that ran out of
+// room) since the ranges were made (for the tests); then 2 n_tiles words for the entries (tile | part << 20 |
+// (parts - 1) << 25: a tile is on the list once per part, and the parts beyond the first of all tiles together are held
+// to n_tiles, so the list cannot overflow) and n_tiles words that count a tile's finished parts.
+// ---------------------------------------------------------------------------------------------
 constexpr uint32_t kLongHeader = 8, kLongRounds = 3, kLongParts = 32;
-// What a workgroup of blend_hybrid_long_kernel leaves of its part of a list: core, tail and the depth of a tie, per pixel.
+constexpr int kLongWaves = 16;
+constexpr uint32_t kLongListDefault = 8192;
+// What a workgroup leaves of its part of a list, in 64-lane rows: HYBRID's core, tail and the depth of a tie.
 template <int K> constexpr uint32_t long_part_words() { return (3u * K + 7u) * 64u; }
 // The parts a list of this length is walked in by separate workgroups (1: by one).  A part is at least four times the
-// threshold long, and long enough that what the parts leave behind fits into the list's own stretch of the spare value buffer.
-template <int K>
-__device__ __forceinline__ uint32_t long_parts(uint32_t length, uint32_t long_threshold)
+// threshold long, and long enough that what the parts leave behind (part_words each) fits into the list's own stretch of
+// the spare value buffer.
+__device__ __forceinline__ uint32_t long_parts(uint32_t length, uint32_t long_threshold, uint32_t part_words)
 {
-    const uint32_t least = 4u * long_threshold > long_part_words<K>() ? 4u * long_threshold : long_part_words<K>();
+    const uint32_t least = 4u * long_threshold > part_words ? 4u * long_threshold : part_words;
     const uint32_t parts = length / least;
     return parts < 1u ? 1u : parts > kLongParts ? kLongParts : parts;
 }
-// One wave per tile.  A tile whose list is longer than long_threshold is not walked here but put on the list of long tiles
-// for blend_hybrid_long_kernel, if the caller provided that list: one wave walks one tile at some 200 ns per instance once it
-// has a SIMD to itself, so a single list of 300 000 instances would otherwise hold the launch for 70 ms.
-// long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = parts granted beyond one per
-// tile -- all zeroed with the ranges and again by the last workgroup of blend_hybrid_long_kernel; [6], [7] = tiles with
-// pixels settled by a second look / walked again in one piece (upper half: of these, after a second look that ran out of
-// room) since the ranges were made (for the tests); then 2 n_tiles words for
-// the entries (tile | part << 20 | (parts - 1) << 25: a tile is on the list once per part, and the parts beyond the first
-// of all tiles together are held to n_tiles, so the list cannot overflow) and n_tiles words that count a tile's finished parts.
+// (one lane of the tile's wave) enters the tile
+__device__ __forceinline__ void long_tile_enter(uint32_t *__restrict__ long_tiles, uint32_t tile, uint32_t n_tiles, uint32_t length,
+                                                uint32_t long_threshold, uint32_t part_words, bool in_parts)
+{
+    uint32_t parts = in_parts ? long_parts(length, long_threshold, part_words) : 1u;
+    if (parts > 1u) {
+        if (atomicAdd(long_tiles + 5, parts - 1u) + parts - 1u > n_tiles) parts = 1u;
+        else long_tiles[kLongHeader + 2u * n_tiles + tile] = 0u;
+    }
+    const uint32_t at = kLongHeader + atomicAdd(long_tiles, parts);
+    for (uint32_t part = 0; part < parts; ++part) long_tiles[at + part] = tile | part << 20 | (parts - 1u) << 25;
+}
+// An entry of the list: part `part` of `parts` of the tile's list [tile_first, tile_last) is [first, last), whole batches of 64.
+struct LongEntry {
+    uint32_t tile, part, parts, tile_first, tile_last, first, last;
+};
+// The workgroups take the entries off the list one by one, the longest first: the list is gone through kLongRounds times
+// (a counter per round, `round` starts at 0), and a round takes the entries of its length class only -- more than 16, more
+// than 4 and up to 4 times the threshold.  The lists differ in length by orders of magnitude, and the launch ends when the
+// workgroup with the longest one does.  Called by all threads of the workgroup (barriers inside); false: the list is
+// through.  The last workgroup to find that clears the list's header, so that the list is empty again for the next blend of
+// this frame (htgs_blend called again without htgs_extract_ranges).
+__device__ __forceinline__ bool long_tile_take(const uint32_t *long_tiles, const uint32_t *__restrict__ ranges, uint32_t long_threshold,
+                                               uint32_t &round, uint32_t *s_next, LongEntry &e)
+{
+    const uint32_t n_long = long_tiles[0];
+    for (;;) {
+        __syncthreads();
+        if (threadIdx.x == 0) *s_next = atomicAdd(const_cast<uint32_t *>(long_tiles) + 1 + round, 1u);
+        __syncthreads();
+        const uint32_t j = *s_next;
+        if (j >= n_long) {
+            if (++round < kLongRounds) continue;
+            if (threadIdx.x == 0) {
+                uint32_t *header = const_cast<uint32_t *>(long_tiles);
+                __threadfence();
+                if (atomicAdd(header + 4, 1u) == gridDim.x - 1) {
+#pragma unroll
+                    for (uint32_t k = 0; k < 6; ++k) header[k] = 0u;
+                }
+            }
+            return false;
+        }
+        const uint32_t entry = long_tiles[kLongHeader + j];
+        e.tile = entry & 0xfffffu; e.part = entry >> 20 & 31u; e.parts = (entry >> 25) + 1u;
+        e.tile_first = ranges[2 * e.tile]; e.tile_last = ranges[2 * e.tile + 1];
+        const uint32_t tile_batches = (e.tile_last - e.tile_first + 63u) / 64u;
+        e.first = e.tile_first + 64u * (uint32_t)((uint64_t)tile_batches * e.part / e.parts);
+        e.last = e.tile_first + 64u * (uint32_t)((uint64_t)tile_batches * (e.part + 1u) / e.parts);
+        e.last = e.last < e.tile_last ? e.last : e.tile_last;
+        const uint32_t length = e.last - e.first;
+        const uint32_t length_class = length > 16u * long_threshold ? 0u : length > 4u * long_threshold ? 1u : 2u;
+        if (length_class == round) return true;
+    }
+}
+// share of wave `wave` of [first, last): whole batches of 64
+__device__ __forceinline__ void long_wave_share(uint32_t first, uint32_t last, uint32_t wave, uint32_t &share_first, uint32_t &share_last)
+{
+    const uint32_t n_batches = (last - first + 63u) / 64u;
+    share_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
+    share_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
+    share_last = share_last < last ? share_last : last;
+}
+// One of several parts is done and the first wave has written what it left (and called __threadfence()): whether the
+// other parts are there already, so that this workgroup ends the tile.  Called by all threads; the first wave calls
+// __threadfence() again before it reads the other parts.
+__device__ __forceinline__ bool long_part_done(const uint32_t *long_tiles, uint32_t n_tiles, const LongEntry &e, uint32_t *s_whole)
+{
+    if (threadIdx.x == 0) *s_whole = atomicAdd(const_cast<uint32_t *>(long_tiles) + kLongHeader + 2u * n_tiles + e.tile, 1u) == e.parts - 1u;
+    __syncthreads();
+    return *s_whole != 0;
+}
+
+// One wave per tile; the tiles with very long lists are left to blend_hybrid_long_kernel.
 template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
@@ -180,16 +260,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (lane == 0) {
-            const uint32_t n_tiles = gridDim.x;
-            uint32_t parts = in_parts ? long_parts<K>(last - first, long_threshold) : 1u;
-            if (parts > 1u) {
-                if (atomicAdd(long_tiles + 5, parts - 1u) + parts - 1u > n_tiles) parts = 1u;
-                else long_tiles[kLongHeader + 2u * n_tiles + tile] = 0u;
-            }
-            const uint32_t at = kLongHeader + atomicAdd(long_tiles, parts);
-            for (uint32_t part = 0; part < parts; ++part) long_tiles[at + part] = tile | part << 20 | (parts - 1u) << 25;
-        }
+        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, long_part_words<K>(), in_parts);
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -295,13 +366,6 @@ __device__ __forceinline__ uint32_t hybrid_pixels_again(TileStage<64> &st, const
     return fits ? n_out : ~0u;
 }
 
-// The long tiles: a workgroup of kLongWaves waves takes a tile, every wave walks a contiguous share of the list (whole
-// batches of 64) into a core and a tail of its own, and the shares are then merged into the first wave's, in list
-// order, through LDS: the entries of the incoming core enter the running core like fragments (what does not stay in
-// the core, of either, joins the tail), the tails add up.  The pixel gets the K nearest fragments of the whole list and
-// everything else in its tail, as in a single walk; what differs from the single walk is the order in which the tail's
-// sums are added (rounding) and which of two stored fragments of exactly equal depth is kept when a nearer one arrives.
-constexpr int kLongWaves = 16;
 // A core, a tail and a tie depth (3K + 7 rows of 64 lanes at from[]) join the running ones: they cover the stretch of the
 // list that follows.
 template <int K, bool FAST>
@@ -328,7 +392,12 @@ __device__ __forceinline__ void hybrid_merge(const float *from, uint32_t lane, f
     const float other = from[(3 * K + 6) * 64];
     tie = other < tie ? other : tie;
 }
-constexpr uint32_t kLongListDefault = 8192;
+// The long tiles: a workgroup of kLongWaves waves takes a tile, every wave walks a contiguous share of the list (whole
+// batches of 64) into a core and a tail of its own, and the shares are then merged into the first wave's, in list
+// order, through LDS: the entries of the incoming core enter the running core like fragments (what does not stay in
+// the core, of either, joins the tail), the tails add up.  The pixel gets the K nearest fragments of the whole list and
+// everything else in its tail, as in a single walk; what differs from the single walk is the order in which the tail's
+// sums are added (rounding) and which of two stored fragments of exactly equal depth is kept when a nearer one arrives.
 template <int K, bool FAST>
 __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
@@ -344,50 +413,17 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
     __shared__ float s_last_depth[64];                // depth of the merged core's last entry
     __shared__ float s_sums[kLongWaves][kAgainPixels][6], s_tails[64][6];   // tails of the pixels looked at again: per wave, whole
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const uint32_t n_long = long_tiles[0];
-    if (n_long == 0) return;                          // (the ordinary frame)
-    // The workgroups take the tiles off the list one by one, the longest first: the list is gone through kLongRounds times
-    // (a counter per round), and a round takes the tiles of its length class only -- more than 16, more than 4 and up to 4
-    // times the threshold.  The lists differ in length by orders of magnitude, and the launch ends when the workgroup with
-    // the longest one does.
+    if (long_tiles[0] == 0) return;                   // (the ordinary frame)
+    const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
     uint32_t round = 0;
-    for (;;) {
-        __syncthreads();
-        if (threadIdx.x == 0) s_next = atomicAdd(const_cast<uint32_t *>(long_tiles) + 1 + round, 1u);
-        __syncthreads();
-        const uint32_t j = s_next;
-        if (j >= n_long) {
-            if (++round < kLongRounds) continue;
-            // The last workgroup to get here clears the list's header, so that the list is empty again for the next
-            // launch of blend_hybrid_kernel on this frame (htgs_blend called again without htgs_extract_ranges).
-            if (threadIdx.x == 0) {
-                uint32_t *header = const_cast<uint32_t *>(long_tiles);
-                __threadfence();
-                if (atomicAdd(header + 4, 1u) == gridDim.x - 1) {
-#pragma unroll
-                    for (uint32_t k = 0; k < 6; ++k) header[k] = 0u;
-                }
-            }
-            break;
-        }
-        const uint32_t entry = long_tiles[kLongHeader + j];
-        const uint32_t tile = entry & 0xfffffu, part = entry >> 20 & 31u, parts = (entry >> 25) + 1u;
-        // (the tile's list, and this entry's part of it: whole batches of 64)
-        const uint32_t tile_first = ranges[2 * tile], tile_last = ranges[2 * tile + 1];
-        const uint32_t tile_batches = (tile_last - tile_first + 63u) / 64u;
-        uint32_t first = tile_first + 64u * (uint32_t)((uint64_t)tile_batches * part / parts);
-        uint32_t last = tile_first + 64u * (uint32_t)((uint64_t)tile_batches * (part + 1u) / parts);
-        last = last < tile_last ? last : tile_last;
-        {
-            const uint32_t length = last - first;
-            const uint32_t length_class = length > 16u * long_threshold ? 0u : length > 4u * long_threshold ? 1u : 2u;
-            if (length_class != round) continue;
-        }
+    LongEntry entry;
+    while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, entry)) {
+        const uint32_t tile = entry.tile, part = entry.part, parts = entry.parts, tile_first = entry.tile_first, tile_last = entry.tile_last;
+        uint32_t first = entry.first, last = entry.last;
         const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
         uint32_t n_batches = (last - first + 63u) / 64u;
-        uint32_t seg_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
-        uint32_t seg_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
-        seg_last = seg_last < last ? seg_last : last;
+        uint32_t seg_first, seg_last;
+        long_wave_share(first, last, wave, seg_first, seg_last);
         constexpr bool kTies = !FAST;
         HybridTail tail;
         hybrid_tail_init(tail);
@@ -420,13 +456,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                 mine[(3 * K + 3) * 64] = tail.c2; mine[(3 * K + 4) * 64] = tail.alpha; mine[(3 * K + 5) * 64] = tail.depth;
                 mine[(3 * K + 6) * 64] = tie;
                 __threadfence();
-                if (lane == 0) {
-                    uint32_t *finished = const_cast<uint32_t *>(long_tiles) + kLongHeader + 2u * grid_w * ((height + 7u) / 8u) + tile;
-                    s_whole = atomicAdd(finished, 1u) == parts - 1u;
-                }
             }
-            __syncthreads();
-            if (!s_whole) continue;
+            if (!long_part_done(long_tiles, n_tiles, entry, &s_whole)) continue;
             if (wave == 0) {
                 __threadfence();
                 hybrid_tail_init(tail);
@@ -435,10 +466,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                 for (uint32_t other = 0; other < parts; ++other)
                     hybrid_merge<K, FAST>(left + (size_t)other * long_part_words<K>(), lane, cd, ca, ci, tail, tie);
             }
-            first = tile_first; last = tile_last; n_batches = tile_batches;
-            seg_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
-            seg_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
-            seg_last = seg_last < last ? seg_last : last;
+            first = tile_first; last = tile_last; n_batches = (last - first + 63u) / 64u;
+            long_wave_share(first, last, wave, seg_first, seg_last);
             __syncthreads();                               // (the parts are read before the shortlist overwrites them)
         }
         if (kTies) {
@@ -630,27 +659,20 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
 // ---------------------------------------------------------------------------------------------
 // OIT_BLEND: weighted-sum order-independent transparency over all fragments.
 // ---------------------------------------------------------------------------------------------
-template <bool FAST>
-__global__ void __launch_bounds__(64) blend_oit_kernel(
-    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, const uint32_t *__restrict__ tile_order)
+// what a pixel has summed up: alpha * (colour, depth), alpha, and the transmittance
+struct OitSums {
+    float a0, a1, a2, a3, alpha, T;
+};
+// The walk over instances [first, last) of a tile's list by one wave (SOLO: the wave is the whole workgroup).
+template <bool FAST, bool SOLO>
+__device__ __forceinline__ void oit_walk(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first, uint32_t last,
+                                         uint32_t lane, const PixelTerms &pt, float cx, float cy, OitSums &sum)
 {
     constexpr int MODE = HTGS_MODE_OIT_BLEND;
-    __shared__ TileStage<64> st;
-    const uint32_t tile = block_tile(tile_order);
-    const uint32_t lane = threadIdx.x;
-    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
-    const uint32_t x = px.x, y = px.y;
-    const bool inside = px.inside;
-    const PixelTerms pt = px.pt;
-    const float cx = px.cx, cy = px.cy;
-    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
-
-    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
+        if (SOLO) __syncthreads(); else wave_lds_sync();
         QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
+        if (SOLO) __syncthreads(); else wave_lds_sync();
         {
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
             quadrant_walk(hits, stage_base, [&](uint32_t addr) {
@@ -660,24 +682,102 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
                 const float4 col = stage_row<64, 5>(addr);
                 if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach)) return;
                 const float depth = FAST ? 0.0f : tile_frag_depth<64>(addr, pt, f);
-                a0 = __builtin_fmaf(f.alpha, col.x, a0);
-                a1 = __builtin_fmaf(f.alpha, col.y, a1);
-                a2 = __builtin_fmaf(f.alpha, col.z, a2);
-                if (!FAST) a3 = __builtin_fmaf(f.alpha, depth, a3);
-                alpha_sum += f.alpha;
-                T *= 1.0f - f.alpha;
+                sum.a0 = __builtin_fmaf(f.alpha, col.x, sum.a0);
+                sum.a1 = __builtin_fmaf(f.alpha, col.y, sum.a1);
+                sum.a2 = __builtin_fmaf(f.alpha, col.z, sum.a2);
+                if (!FAST) sum.a3 = __builtin_fmaf(f.alpha, depth, sum.a3);
+                sum.alpha += f.alpha;
+                sum.T *= 1.0f - f.alpha;
             });
         }
     }
-    if (!inside) return;
+}
+__device__ __forceinline__ void oit_composite(const OitSums &sum, float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height,
+                                              uint32_t x, uint32_t y, int chw)
+{
     float r = 0.0f, g = 0.0f, b = 0.0f, d = 0.0f;
-    if (alpha_sum >= ModeCfg<MODE>::min_alpha) {
-        const float alpha = 1.0f - T;
-        const float s = alpha * (1.0f / alpha_sum);
-        r = s * a0; g = s * a1; b = s * a2;
-        d = (s * a3) / alpha;
+    if (sum.alpha >= ModeCfg<HTGS_MODE_OIT_BLEND>::min_alpha) {
+        const float alpha = 1.0f - sum.T;
+        const float s = alpha * (1.0f / sum.alpha);
+        r = s * sum.a0; g = s * sum.a1; b = s * sum.a2;
+        d = (s * sum.a3) / alpha;
     }
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, d);
+}
+constexpr uint32_t kOitPartWords = 6u * 64u;
+template <bool FAST>
+__global__ void __launch_bounds__(64) blend_oit_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw,
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, int in_parts, const uint32_t *__restrict__ tile_order)
+{
+    __shared__ TileStage<64> st;
+    const uint32_t tile = block_tile(tile_order);
+    const uint32_t lane = threadIdx.x;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    if (long_tiles != nullptr && last - first > long_threshold) {
+        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, kOitPartWords, in_parts);
+        return;
+    }
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    OitSums sum = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f };
+    oit_walk<FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, sum);
+    if (!px.inside) return;
+    oit_composite(sum, image, depths, width, height, px.x, px.y, chw);
+}
+
+// The tiles with very long lists: every wave of the workgroup walks a share of the list, the sums add up in the order of
+// the shares (the transmittances multiply), and so do those of the parts of a list that several workgroups walked
+// (`left`: the spare value buffer, where the parts of a tile leave their sums in the tile's own stretch).  The pixel's
+// result is that of the single walk up to the order of its sums.
+template <bool FAST>
+__global__ void __launch_bounds__(64 * kLongWaves) blend_oit_long_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw,
+    uint32_t *__restrict__ left, uint32_t long_threshold)
+{
+    __shared__ TileStage<64> st[kLongWaves];
+    __shared__ float s_sums[kLongWaves][6][64];
+    __shared__ uint32_t s_next, s_whole;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (long_tiles[0] == 0) return;                   // (the ordinary frame)
+    const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
+    uint32_t round = 0;
+    LongEntry entry;
+    while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, entry)) {
+        const TilePixel px = quadrant_tile_pixel(entry.tile, grid_w, lane, width, height);
+        uint32_t share_first, share_last;
+        long_wave_share(entry.first, entry.last, wave, share_first, share_last);
+        OitSums sum = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f };
+        oit_walk<FAST, false>(st[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, sum);
+        s_sums[wave][0][lane] = sum.a0; s_sums[wave][1][lane] = sum.a1; s_sums[wave][2][lane] = sum.a2; s_sums[wave][3][lane] = sum.a3;
+        s_sums[wave][4][lane] = sum.alpha; s_sums[wave][5][lane] = sum.T;
+        __syncthreads();
+        if (wave == 0) {
+            for (int w = 1; w < kLongWaves; ++w) {
+                sum.a0 += s_sums[w][0][lane]; sum.a1 += s_sums[w][1][lane]; sum.a2 += s_sums[w][2][lane]; sum.a3 += s_sums[w][3][lane];
+                sum.alpha += s_sums[w][4][lane]; sum.T *= s_sums[w][5][lane];
+            }
+        }
+        if (entry.parts > 1u) {
+            float *const parts = reinterpret_cast<float *>(left + entry.tile_first);
+            if (wave == 0) {
+                float *mine = parts + (size_t)entry.part * kOitPartWords + lane;
+                mine[0] = sum.a0; mine[64] = sum.a1; mine[128] = sum.a2; mine[192] = sum.a3; mine[256] = sum.alpha; mine[320] = sum.T;
+                __threadfence();
+            }
+            if (!long_part_done(long_tiles, n_tiles, entry, &s_whole)) continue;
+            if (wave == 0) {
+                __threadfence();
+                sum = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f };
+                for (uint32_t part = 0; part < entry.parts; ++part) {
+                    const float *its = parts + (size_t)part * kOitPartWords + lane;
+                    sum.a0 += its[0]; sum.a1 += its[64]; sum.a2 += its[128]; sum.a3 += its[192]; sum.alpha += its[256]; sum.T *= its[320];
+                }
+            }
+        }
+        if (wave == 0 && px.inside) oit_composite(sum, image, depths, width, height, px.x, px.y, chw);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -885,9 +985,17 @@ static void launch_blend(const htgs_frame *f, int selector, uint32_t grid_w, uin
                                f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->tile_order);
             break;
         default:
+        {
+            const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
             hipLaunchKernelGGL(blend_oit_kernel<FAST>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
-                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->tile_order);
+                               f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->long_tiles, threshold,
+                               f->vals[selector ^ 1] != nullptr, f->tile_order);
+            if (f->long_tiles)
+                hipLaunchKernelGGL(blend_oit_long_kernel<FAST>, dim3(256), dim3(64 * kLongWaves), 0, s, f->ranges, f->vals[selector],
+                                   (const float4 *)f->prim, f->long_tiles, f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w,
+                                   f->to_chw, f->vals[selector ^ 1], threshold);
             break;
+        }
     }
 }
 

@@ -20,9 +20,8 @@ NEVER = 2 ** 31 - 1
 SECOND_LOOKS = []
 
 
-def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False, in_parts=None):
-    fb = FrameBuffers(*scene_gpu.gaussians(), scene_gpu.settings(RasterizerMode.HYBRID_BLEND, K), to_chw, median, fast=fast,
-                      long_list_threshold=threshold)
+def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False, in_parts=None, mode=RasterizerMode.HYBRID_BLEND, part_rows=None):
+    fb = FrameBuffers(*scene_gpu.gaussians(), scene_gpu.settings(mode, K), to_chw, median, fast=fast, long_list_threshold=threshold)
     fb.front()
     fb.alloc_instances(fb.read_instance_count())
     fb.create_instances()
@@ -34,7 +33,7 @@ def render(scene_gpu, K, threshold, to_chw=True, median=False, fast=False, in_pa
     fb.blend()
     torch.cuda.synchronize()
     if in_parts is not None:                      # lists long enough to be walked in parts by several workgroups
-        part = max(4 * threshold, (3 * K + 7) * 64)
+        part = max(4 * threshold, (part_rows or 3 * K + 7) * 64)
         assert (int((lengths >= 2 * part).sum()) > 0) == in_parts, f"longest list {int(lengths.max())}, a part {part}"
     assert not bool(fb.long_tiles[:6].any())      # the blend stage leaves the list empty for its next call
     # tiles with pixels at which depths coincided: settled by a second look at those pixels / walked again in one piece
@@ -177,3 +176,23 @@ def test_long_tiles_fast_variant(cuda):
     single, _, none = render(scene, 16, NEVER, fast=True)
     assert long_tiles > 0 and none == 0
     assert np.abs(image - single).max() <= TOL
+
+
+@pytest.mark.parametrize("config,n,threshold,in_parts,to_chw", [(0, 3000, 24, False, True), (1, 60_000, 16, False, False), (3, 150_000, 500, True, True),
+                                                                 (3, 150_000, 100, True, False)])
+def test_long_tiles_oit(cuda, config, n, threshold, in_parts, to_chw):
+    """OIT_BLEND: the sums of the waves' shares, and of the parts of a list, add up in list order."""
+    print(f"case OIT config={config} n={n} threshold={threshold}", flush=True)
+    oit = RasterizerMode.OIT_BLEND
+    scene = make_scene(config, n)
+    ref = oracle_render(scene, 3, 16, to_chw=to_chw)
+    image, depth, long_tiles = render(scene.to(cuda), 16, threshold, to_chw=to_chw, in_parts=in_parts, mode=oit, part_rows=6)
+    single, single_depth, none = render(scene.to(cuda), 16, NEVER, to_chw=to_chw, mode=oit)
+    assert long_tiles > 0 and none == 0
+    err = [float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max()),
+           float(np.abs(image - single).max()), float(np.abs(depth - single_depth).max())]
+    print(f"  long tiles {long_tiles}; against the oracle {err[0]:.3g} / {err[1]:.3g}, against the single walk {err[2]:.3g} / {err[3]:.3g}", flush=True)
+    assert max(err) <= TOL
+    fast, _, _ = render(scene.to(cuda), 16, threshold, to_chw=to_chw, fast=True, mode=oit)
+    single_fast, _, _ = render(scene.to(cuda), 16, NEVER, to_chw=to_chw, fast=True, mode=oit)
+    assert np.abs(fast - single_fast).max() <= TOL
