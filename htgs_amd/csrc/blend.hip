@@ -155,7 +155,7 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
 // 200 ns per instance once it has a SIMD to itself, so a single list of 300 000 instances would otherwise hold the
 // launch for 70 ms.
 // long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = parts granted beyond one per
-// tile -- all zeroed with the ranges and again by the last workgroup of the second launch; [6], [7] = HYBRID's tiles with
+// tile -- all zeroed with the ranges and again by the last workgroup of the second launch; [6], [7] = tiles with
 // pixels settled by a second look / walked again in one piece (upper half: of these, after a second look that ran out of
 // room) since the ranges were made (for the tests); then 2 n_tiles words for the entries (tile | part << 20 |
 // (parts - 1) << 25: a tile is on the list once per part, and the parts beyond the first of all tiles together are held
@@ -285,7 +285,7 @@ __device__ __forceinline__ float wave_product(float v)
     for (int o = 32; o > 0; o >>= 1) v *= __shfl_xor(v, o);
     return v;
 }
-constexpr int kAgainPixels = 2;       // pixels a pass of hybrid_pixels_again takes at once
+constexpr int kAgainPixels = 2;       // pixels a pass of pixels_again takes at once
 constexpr int kAgainMost = 8;         // pixels of a tile beyond which they are walked again in one piece instead
 
 // The second look at the pixels of pixel_lanes, whose cores the merge could not settle: lanes = instances.  Every wave
@@ -296,13 +296,14 @@ constexpr int kAgainMost = 8;         // pixels of a tile beyond which they are 
 // over the waves; the colour sums take every fragment); the others, the few that decide the core, are put down in list
 // order at `out` as (pixel, depth, alpha, index) for the walk's insertion to be replayed on them alone.  Returns their
 // number, or ~0u when `room` entries were not enough.  pass_done(pixels) is called, by the whole workgroup, after each pass.
-template <int K, typename PassDone>
-__device__ __forceinline__ uint32_t hybrid_pixels_again(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
+// ALPHA_BLEND_FIRST_K has no tail: its fragments that are not farther than the core's last entry are put down, no sums.
+template <int MODE, bool FAST, typename PassDone>
+__device__ __forceinline__ uint32_t pixels_again(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
                                                         uint32_t last, uint32_t lane, float cx, float cy, uint64_t pixel_lanes,
                                                         const float *last_depth, float (*sums)[6], uint32_t *__restrict__ out, uint32_t room,
                                                         PassDone pass_done)
 {
-    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    constexpr bool kTail = MODE == HTGS_MODE_HYBRID_BLEND;
     uint32_t n_out = 0;
     bool fits = true;
     for (uint64_t todo = pixel_lanes; todo != 0;) {
@@ -331,17 +332,19 @@ __device__ __forceinline__ uint32_t hybrid_pixels_again(TileStage<64> &st, const
                 if (pixel[j] >= 64u) continue;                      // (wave-uniform)
                 TileFrag f;
                 const bool in_reach = tile_frag_cutoff<64>(addr, pt[j], f);
-                f.den_rcp = frag_rcp<false>(f.den);
+                f.den_rcp = frag_rcp<FAST>(f.den);
                 const float4 col = stage_row<64, 5>(addr);
-                const bool fragment = tile_frag_alpha<MODE, false>(stage_opacity<64>(addr), f) && in_reach && loaded;
+                const bool fragment = tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach && loaded;
                 const float depth = tile_frag_depth<64>(addr, pt[j], f);
                 bool decides = false;
                 if (fragment) {
-                    acc[j].c0 = __builtin_fmaf(f.alpha, col.x, acc[j].c0);
-                    acc[j].c1 = __builtin_fmaf(f.alpha, col.y, acc[j].c1);
-                    acc[j].c2 = __builtin_fmaf(f.alpha, col.z, acc[j].c2);
-                    decides = depth <= farthest[j] && f.alpha >= kMinAlphaCore;
-                    if (!decides) hybrid_tail_add<false>(acc[j], depth, f.alpha);
+                    if (kTail) {
+                        acc[j].c0 = __builtin_fmaf(f.alpha, col.x, acc[j].c0);
+                        acc[j].c1 = __builtin_fmaf(f.alpha, col.y, acc[j].c1);
+                        acc[j].c2 = __builtin_fmaf(f.alpha, col.z, acc[j].c2);
+                    }
+                    decides = depth <= farthest[j] && (!kTail || f.alpha >= kMinAlphaCore);
+                    if (kTail && !decides) hybrid_tail_add<false>(acc[j], depth, f.alpha);
                 }
                 const uint64_t deciding = __ballot(decides);
                 if (deciding != 0) {
@@ -356,7 +359,7 @@ __device__ __forceinline__ uint32_t hybrid_pixels_again(TileStage<64> &st, const
             }
         }
 #pragma unroll
-        for (int j = 0; j < kAgainPixels; ++j) {
+        for (int j = 0; kTail && j < kAgainPixels; ++j) {
             const float T = wave_product(acc[j].T), c0 = wave_total(acc[j].c0), c1 = wave_total(acc[j].c1), c2 = wave_total(acc[j].c2),
                         alpha = wave_total(acc[j].alpha), depth = wave_total(acc[j].depth);
             if (lane == 0) { sums[j][0] = T; sums[j][1] = c0; sums[j][2] = c1; sums[j][3] = c2; sums[j][4] = alpha; sums[j][5] = depth; }
@@ -491,7 +494,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
             if (redo_lanes != 0) {
                 bool others_done = false;                       // the pixels that need no second look are composited
                 if (shortlist != nullptr && __popcll(redo_lanes) <= kAgainMost) {
-                    // All waves look at these pixels again, lanes = instances (hybrid_pixels_again), into the tile's stretch of
+                    // All waves look at these pixels again, lanes = instances (pixels_again), into the tile's stretch of
                     // the shortlist, four words per fragment that decides a core: a wave has a quarter as many entries as
                     // its share has instances, which is ample unless depths coincide by the hundred -- then, and when the
                     // pixels are many (a pass over the list serves kAgainPixels of them), the other way below is taken.
@@ -501,7 +504,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                         if (px.inside && !redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
                     }
                     __syncthreads();
-                    const uint32_t listed = hybrid_pixels_again<K>(
+                    const uint32_t listed = pixels_again<HTGS_MODE_HYBRID_BLEND, false>(
                         st[wave], inst, prim, seg_first, seg_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, s_sums[wave], shortlist + seg_first,
                         (seg_last - seg_first) / 4u, [&](const uint32_t (&pixel)[kAgainPixels]) {
                             __syncthreads();
@@ -591,34 +594,28 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
 // ---------------------------------------------------------------------------------------------
 // ALPHA_BLEND_FIRST_K: the K nearest fragments with alpha >= 1/20, alpha-blended; no tail.
 // ---------------------------------------------------------------------------------------------
-template <int K, bool FAST>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
-    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median, const uint32_t *__restrict__ tile_order)
+template <int K>
+__device__ __forceinline__ void first_k_core_init(float (&cd)[K], float (&ca)[K], uint32_t (&ci)[K])
 {
-    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
-    __shared__ TileStage<64> st;
-    const uint32_t tile = block_tile(tile_order);
-    const uint32_t lane = threadIdx.x;
-    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
-    const uint32_t x = px.x, y = px.y;
-    const bool inside = px.inside;
-    const PixelTerms pt = px.pt;
-    const float cx = px.cx, cy = px.cy;
-
-    float ca[K], cd[K];
-    uint32_t ci[K];
 #pragma unroll
     for (int i = 0; i < K; ++i) {
         ca[i] = 0.0f; cd[i] = __FLT_MAX__; ci[i] = 0xffffffffu;
         asm volatile("" : "+v"(cd[i]), "+v"(ca[i]), "+v"(ci[i]));      // one register per slot
     }
-
-    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+}
+// The walk over instances [first, last) of a tile's list by one wave (SOLO: the wave is the whole workgroup).  TIES (the
+// walks of blend_first_k_long_kernel): `tie` receives the least depth at which an entry was pushed out of the core that is
+// exactly as deep as the entry that is now last.
+template <int K, bool FAST, bool SOLO, bool TIES = false>
+__device__ __forceinline__ void first_k_walk(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
+                                             uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K], float (&ca)[K],
+                                             uint32_t (&ci)[K], float *tie = nullptr)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
     for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
+        if (SOLO) __syncthreads(); else wave_lds_sync();
         QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
+        if (SOLO) __syncthreads(); else wave_lds_sync();
         {
             const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
             quadrant_walk(hits, stage_base, [&](uint32_t addr) {
@@ -631,11 +628,16 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
                 float alpha = f.alpha;
                 uint32_t idx = stage_index<64>(addr);
                 core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
+                if (TIES && alpha > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
             });
         }
     }
-    if (!inside) return;
-
+}
+template <int K>
+__device__ __forceinline__ void first_k_composite(const float4 *__restrict__ prim, const float (&cd)[K], const float (&ca)[K], const uint32_t (&ci)[K],
+                                                  float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t x,
+                                                  uint32_t y, int chw, int median)
+{
     float r = 0.0f, g = 0.0f, b = 0.0f, depth_pixel = 0.0f, T = 1.0f;
     bool open = true;
 #pragma unroll
@@ -654,6 +656,166 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     }
     if (!median) depth_pixel = T < 1.0f ? depth_pixel / (1.0f - T) : 0.0f;
     store_pixel(image, depths, width, height, x, y, chw, r, g, b, depth_pixel);
+}
+// what a workgroup leaves of its part of a list: the core and the depth of a tie
+template <int K> constexpr uint32_t first_k_part_words() { return (3u * K + 1u) * 64u; }
+template <int K, bool FAST>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, int in_parts, const uint32_t *__restrict__ tile_order)
+{
+    __shared__ TileStage<64> st;
+    const uint32_t tile = block_tile(tile_order);
+    const uint32_t lane = threadIdx.x;
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    if (long_tiles != nullptr && last - first > long_threshold) {
+        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, first_k_part_words<K>(), in_parts);
+        return;
+    }
+    const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
+    float ca[K], cd[K];
+    uint32_t ci[K];
+    first_k_core_init<K>(cd, ca, ci);
+    first_k_walk<K, FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
+    if (!px.inside) return;
+    first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+}
+
+// A core and a tie depth (3K + 1 rows of 64 lanes at from[]) join the running ones: they cover the stretch of the list
+// that follows.
+template <int K, bool FAST>
+__device__ __forceinline__ void first_k_merge(const float *from, uint32_t lane, float (&cd)[K], float (&ca)[K], uint32_t (&ci)[K], float &tie)
+{
+    constexpr bool kTies = true;
+    from += lane;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        float depth = from[(3 * i) * 64], alpha = from[(3 * i + 1) * 64];
+        uint32_t index = float_to_bits(from[(3 * i + 2) * 64]);
+        if (alpha > 0.0f) {                    // a filled slot
+            if (kTies && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
+            if (depth < cd[K - 1]) {
+                core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
+                if (kTies && alpha > 0.0f && depth == cd[K - 1]) tie = depth < tie ? depth : tie;
+            }
+        }
+    }
+    const float other = from[(3 * K) * 64];
+    tie = other < tie ? other : tie;
+}
+template <int K>
+__device__ __forceinline__ void first_k_put(float *to, uint32_t lane, const float (&cd)[K], const float (&ca)[K], const uint32_t (&ci)[K], float tie)
+{
+    to += lane;
+#pragma unroll
+    for (int i = 0; i < K; ++i) { to[(3 * i) * 64] = cd[i]; to[(3 * i + 1) * 64] = ca[i]; to[(3 * i + 2) * 64] = bits_to_float(ci[i]); }
+    to[(3 * K) * 64] = tie;
+}
+
+// The tiles with very long lists, as in blend_hybrid_long_kernel: every wave of the workgroup walks a share of the list
+// into a core of its own, the cores are merged in list order (and so are those of the parts of a list that several
+// workgroups walked, through the tile's stretch of the spare value buffer `spare`), and the pixels at which fragments of
+// exactly equal depth met where they can change the final core get a second look (pixels_again) with the insertion
+// replayed on the fragments that are not farther than the merged core's last entry -- or, when they are many or the room
+// for those fragments does not do, the first wave walks the whole list again for them.
+template <int K, bool FAST>
+__global__ void __launch_bounds__(64 * kLongWaves) blend_first_k_long_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
+    float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
+    uint32_t *__restrict__ spare, uint32_t long_threshold)
+{
+    __shared__ TileStage<64> st[kLongWaves];
+    __shared__ float s_merge[3 * K + 1][64];
+    __shared__ uint32_t s_next, s_whole, s_redo[2], s_listed[kLongWaves];
+    __shared__ float s_last_depth[64];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (long_tiles[0] == 0) return;                   // (the ordinary frame)
+    const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
+    constexpr bool kTies = true;                      // (the fast variant too: a tie decides which fragment a pixel shows)
+    uint32_t round = 0;
+    LongEntry entry;
+    while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, entry)) {
+        const TilePixel px = quadrant_tile_pixel(entry.tile, grid_w, lane, width, height);
+        uint32_t share_first, share_last;
+        long_wave_share(entry.first, entry.last, wave, share_first, share_last);
+        float ca[K], cd[K];
+        uint32_t ci[K];
+        first_k_core_init<K>(cd, ca, ci);
+        float tie = __FLT_MAX__;
+        first_k_walk<K, FAST, false, kTies>(st[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, &tie);
+        for (uint32_t s = 1; s < (uint32_t)kLongWaves; ++s) {
+            __syncthreads();                               // the buffer is free
+            if (wave == s) first_k_put<K>(&s_merge[0][0], lane, cd, ca, ci, tie);
+            __syncthreads();
+            if (wave == 0) first_k_merge<K, FAST>(&s_merge[0][0], lane, cd, ca, ci, tie);
+        }
+        if (entry.parts > 1u) {
+            float *const left = reinterpret_cast<float *>(spare + entry.tile_first);
+            if (wave == 0) {
+                first_k_put<K>(left + (size_t)entry.part * first_k_part_words<K>(), lane, cd, ca, ci, tie);
+                __threadfence();
+            }
+            if (!long_part_done(long_tiles, n_tiles, entry, &s_whole)) continue;
+            if (wave == 0) {
+                __threadfence();
+                first_k_core_init<K>(cd, ca, ci);
+                tie = __FLT_MAX__;
+                for (uint32_t other = 0; other < entry.parts; ++other)
+                    first_k_merge<K, FAST>(left + (size_t)other * first_k_part_words<K>(), lane, cd, ca, ci, tie);
+            }
+            long_wave_share(entry.tile_first, entry.tile_last, wave, share_first, share_last);
+            __syncthreads();                               // (the parts are read before the second look overwrites them)
+        }
+        if (kTies) {
+            bool redo = false;
+            if (wave == 0) {
+                redo = tie <= cd[K - 1];
+#pragma unroll
+                for (int i = 0; i + 1 < K; ++i) redo = redo || (ca[i + 1] > 0.0f && cd[i] == cd[i + 1]);
+                const uint64_t lanes = __ballot(redo);
+                if (lane == 0) { s_redo[0] = (uint32_t)lanes; s_redo[1] = (uint32_t)(lanes >> 32); }
+                s_last_depth[lane] = cd[K - 1];
+                if (lanes != 0 && px.inside && !redo) first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+            }
+            __syncthreads();
+            const uint64_t redo_lanes = (uint64_t)s_redo[0] | (uint64_t)s_redo[1] << 32;
+            if (redo_lanes != 0) {
+                bool settled = false, looked = false;
+                if (spare != nullptr && __popcll(redo_lanes) <= kAgainMost) {
+                    looked = true;
+                    const uint32_t listed = pixels_again<HTGS_MODE_ALPHA_BLEND_FIRST_K, FAST>(
+                        st[wave], inst, prim, share_first, share_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, nullptr, spare + share_first,
+                        (share_last - share_first) / 4u, [](const uint32_t (&)[kAgainPixels]) {});
+                    if (lane == 0) s_listed[wave] = listed;
+                    __syncthreads();
+                    settled = true;
+                    for (int w = 0; w < kLongWaves; ++w) settled = settled && s_listed[w] != ~0u;
+                }
+                if (threadIdx.x == 0) atomicAdd(const_cast<uint32_t *>(long_tiles) + (settled ? 6 : 7), settled || !looked ? 1u : 0x10001u);
+                if (wave == 0) {
+                    first_k_core_init<K>(cd, ca, ci);
+                    if (settled) {
+                        for (uint32_t w = 0; w < (uint32_t)kLongWaves; ++w) {
+                            uint32_t from, to;
+                            long_wave_share(entry.tile_first, entry.tile_last, w, from, to);
+                            const uint32_t *candidate = spare + from;
+                            for (uint32_t todo = s_listed[w]; todo != 0; --todo, candidate += 4) {
+                                float depth = bits_to_float(candidate[1]), alpha = bits_to_float(candidate[2]);
+                                uint32_t index = candidate[3];
+                                if (lane == candidate[0] && depth < cd[K - 1]) core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
+                            }
+                        }
+                    } else {
+                        first_k_walk<K, FAST, false>(st[0], inst, prim, entry.tile_first, entry.tile_last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
+                    }
+                    if (px.inside && redo) first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+                }
+                continue;
+            }
+        }
+        if (wave == 0 && px.inside) first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -948,9 +1110,14 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
 template <int K, bool FAST>
 static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
+    const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     hipLaunchKernelGGL((blend_first_k_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth, f->tile_order);
+                       f->use_median_depth, f->long_tiles, threshold, f->vals[selector ^ 1] != nullptr, f->tile_order);
+    if (f->long_tiles)
+        hipLaunchKernelGGL((blend_first_k_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
+                           f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
+                           (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->vals[selector ^ 1], threshold);
 }
 
 template <bool FAST>

@@ -196,3 +196,43 @@ def test_long_tiles_oit(cuda, config, n, threshold, in_parts, to_chw):
     fast, _, _ = render(scene.to(cuda), 16, threshold, to_chw=to_chw, fast=True, mode=oit)
     single_fast, _, _ = render(scene.to(cuda), 16, NEVER, to_chw=to_chw, fast=True, mode=oit)
     assert np.abs(fast - single_fast).max() <= TOL
+
+
+FIRST_K = RasterizerMode.ALPHA_BLEND_FIRST_K
+
+
+@pytest.mark.parametrize("config,n,K,threshold,in_parts,median", [(0, 3000, 4, 24, None, False), (0, 3000, 1, 24, None, True), (1, 60_000, 16, 16, None, False),
+                                                                   (2, 100_000, 32, 20, None, True), (3, 150_000, 4, 200, True, False),
+                                                                   (3, 300_000, 16, 500, True, False)])
+def test_long_tiles_first_k(cuda, config, n, K, threshold, in_parts, median):
+    """ALPHA_BLEND_FIRST_K: the cores of the waves' shares, and of the parts of a list, merged in list order."""
+    print(f"case FIRST_K config={config} n={n} K={K} threshold={threshold}", flush=True)
+    scene = make_scene(config, n)
+    ref = oracle_render(scene, 1, K, median=median)
+    image, depth, long_tiles = render(scene.to(cuda), K, threshold, median=median, in_parts=in_parts, mode=FIRST_K, part_rows=3 * K + 1)
+    single, single_depth, none = render(scene.to(cuda), K, NEVER, median=median, mode=FIRST_K)
+    assert long_tiles > 0 and none == 0
+    err = [float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max()),
+           float(np.abs(image - single).max()), float(np.abs(depth - single_depth).max())]
+    print(f"  long tiles {long_tiles}; against the oracle {err[0]:.3g} / {err[1]:.3g}, against the single walk {err[2]:.3g} / {err[3]:.3g}", flush=True)
+    assert max(err) <= TOL
+    fast, _, _ = render(scene.to(cuda), K, threshold, fast=True, mode=FIRST_K)
+    single_fast, _, _ = render(scene.to(cuda), K, NEVER, fast=True, mode=FIRST_K)
+    assert np.abs(fast - single_fast).max() <= TOL
+
+
+@pytest.mark.parametrize("config,n,K,threshold,twins,copies", [(0, 3000, 4, 24, 150, 1), (3, 150_000, 16, 1000, 300, 1), (0, 1500, 4, 64, 0, 6),
+                                                                (0, 1500, 16, 64, 0, 6)])
+def test_long_tiles_first_k_with_fragments_of_equal_depth(cuda, config, n, K, threshold, twins, copies):
+    """A few twins: the pixels get a second look and the insertion is replayed; coincident copies of everything: the first
+    wave walks the list again."""
+    print(f"case FIRST_K config={config} n={n} K={K} threshold={threshold} twins={twins} copies={copies}", flush=True)
+    scene = make_scene(config, n)
+    scene = with_some_twins(scene, twins) if twins else with_coincident_copies(scene, copies)
+    ref = oracle_render(scene, 1, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, threshold, mode=FIRST_K)
+    second_looks, walked_again, _ = SECOND_LOOKS[-1]
+    err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
+    print(f"  long tiles {long_tiles}, second looks {second_looks}, walked again {walked_again}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
+    assert long_tiles > 0 and (second_looks > 0 if twins else walked_again > 0)
+    assert err_i <= TOL and err_d <= TOL
