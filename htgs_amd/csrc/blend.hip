@@ -1186,6 +1186,8 @@ extern "C" int htgs_blend(const htgs_frame *f, int selector)
     const int tile = tile_size(f->mode);
     const uint32_t grid_w = div_up(f->width, tile), grid_h = div_up(f->height, tile);
     const uint32_t n_tiles = grid_w * grid_h;
+    // (an entry of the list of long tiles holds the tile in 20 bits; htgs_scan_offsets refuses larger grids as well)
+    if ((uint64_t)grid_w * grid_h > (1ull << 20)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend: more than 2^20 tiles");
     if (f->fast_math) launch_blend<true>(f, selector, grid_w, n_tiles);
     else launch_blend<false>(f, selector, grid_w, n_tiles);
     return check_launch("blend");

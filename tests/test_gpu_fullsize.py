@@ -1,7 +1,7 @@
 """Full-size runs of the benchmark configurations on the GPU.
 
-cfg1 (1 M, 720p), cfg2 (3 M, 1080p, all four modes) and cfg3 (6 M stress scene, 8e7 instances, the mode it is
-specified for) are small enough for the C oracle, so they are compared with it outright.  cfg3 is also checked
+cfg1 (1 M, 720p), cfg2 (3 M, 1080p, all four modes) and cfg3 (6 M stress scene, 8e7 instances, the three modes that
+walk all of its very long lists) are small enough for the C oracle, so they are compared with it outright.  cfg3 is also checked
 through size-independent properties:
 tile counts against the oracle's per-Gaussian stage, conservation of instances through duplication and sort,
 sortedness and stability of the sorted list, ranges partitioning it, and a repeat of the frame giving identical
@@ -18,7 +18,7 @@ from util import gpu_stages, oracle_frame, oracle_render, u32
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("config,mode", [(1, 0), (2, 0), (2, 1), (2, 2), (2, 3), (3, 0)])
+@pytest.mark.parametrize("config,mode", [(1, 0), (2, 0), (2, 1), (2, 2), (2, 3), (3, 0), (3, 1), (3, 3)])
 def test_full_size_against_oracle(cuda, config, mode):
     print(f"case config={config} mode={mode} (full size)", flush=True)
     scene = make_scene(config)
@@ -107,8 +107,12 @@ def test_full_size_training_step_against_oracle(cuda, mode):
             np.testing.assert_allclose(got_info[r], info_ref[r], rtol=2e-3, atol=2e-4 * float(np.abs(info_ref[r]).max()))
 
 
-def test_frames_are_reproducible_bit_for_bit(cuda):
-    scene = make_scene(1, 300_000).to(cuda)
+@pytest.mark.parametrize("config,n", [(1, 300_000), (3, 1_000_000)])
+def test_frames_are_reproducible_bit_for_bit(cuda, config, n):
+    """(the stress scene has tiles that several workgroups walk in parts: whichever finishes last, the parts are merged in
+    list order)"""
+    print(f"case config={config} n={n} (twice)", flush=True)
+    scene = make_scene(config, n).to(cuda)
     for mode in range(4):
         s = scene.settings(RasterizerMode(mode), 16)
         a = rasterize(*scene.gaussians(), s, True, False)
