@@ -279,7 +279,9 @@ def main():
     blend_avg_ms = sum(samples["blend"]) / len(samples["blend"])
     algo_bytes = {
         "preprocess": N * (56 + 12 * (B - 1) * (B > 1)) + 4 * N + 88 * n_vis,   # 80 B record + 8 B bounds per visible Gaussian
-        "scan": 8 * N,
+        # (GLOBAL_ORDERING with the Gaussians sorted by depth first: four passes over N (key, index) pairs, each moving the
+        # pairs once each way and reading the keys once more for the histograms, and the gather of rectangles and counts)
+        "scan": 8 * N + (fb.depth_order is not None) * (4 * (2 * 8 + 4) * N + 8 * N + 16 * n_vis),
         "create_instances": 16 * n_vis + (kb + 4) * n_inst,
         "sort": passes * 2 * (kb + 4) * n_inst + kb * n_inst,            # every pass moves the pairs once each way; the keys are read once more for the histograms
         "extract_ranges": kb * n_inst + 8 * T,
@@ -302,11 +304,11 @@ def main():
 
     if args.mode == 2:
         # GLOBAL_ORDERING stops a pixel once it is opaque, so the number of evaluations its blend kernel makes depends on
-        # the data and 256 per instance would overstate it; the stage priced here is the sort of the 64-bit keys
-        sort_gbs = algo_bytes["sort"] / 1e9 / (stages["sort"] / 1e3)
-        roofline = {"kernel": "sort (digit_histogram + digit_row_scan + digit_scatter, all passes)", "bound": "hbm", "achieved": round(sort_gbs, 1),
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(sort_gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                    "launch_ms": round(stages["sort"], 4)}
+        # the data and 256 per instance would overstate it; the kernel priced here is the next one by time, the per-Gaussian
+        # stage, which is bound by its HBM traffic
+        pre_gbs = algo_bytes["preprocess"] / 1e9 / (stages["preprocess"] / 1e3)
+        roofline = {"kernel": "preprocess", "bound": "hbm", "achieved": round(pre_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(pre_gbs / HBM_PEAK_GBS, 4), "traffic": None, "launch_ms": round(stages["preprocess"], 4)}
 
     # ---- CPU baseline: the C oracle on this box's host cores, one whole frame of the same workload ----
     cpu_baseline = None

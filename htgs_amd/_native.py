@@ -50,6 +50,7 @@ class Frame(ctypes.Structure):
         ("long_tiles", ctypes.c_void_p),
         ("long_list_threshold", ctypes.c_int32),
         ("tile_order", ctypes.c_void_p),
+        ("depth_order", ctypes.c_void_p),
         ("n_instances", ctypes.c_uint64),
         ("keys", ctypes.c_void_p * 2),
         ("vals", ctypes.c_void_p * 2),
@@ -87,6 +88,10 @@ SYMBOLS = {
     "htgs_end_bit": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "htgs_key_bytes": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "htgs_sort_passes": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "htgs_frame_end_bit": (ctypes.c_int, [_FRAME_P]),
+    "htgs_frame_key_bytes": (ctypes.c_int, [_FRAME_P]),
+    "htgs_frame_sort_passes": (ctypes.c_int, [_FRAME_P]),
+    "htgs_depth_order_words": (ctypes.c_size_t, [ctypes.c_int]),
     "htgs_scan_tmp_words": (ctypes.c_size_t, [ctypes.c_int]),
     "htgs_sort_tmp_words": (ctypes.c_size_t, [ctypes.c_uint64]),
     "htgs_tile_order_words": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),

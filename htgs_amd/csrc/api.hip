@@ -78,6 +78,26 @@ extern "C" int htgs_key_bytes(int mode, int width, int height)
     return htgs_end_bit(mode, width, height) <= 16 ? 2 : 4;
 }
 
+extern "C" int htgs_frame_end_bit(const htgs_frame *f)
+{
+    if (!f) return 0;
+    return htgs_end_bit(f->mode, f->width, f->height) - (frame_depth_ordered(f) ? 32 : 0);
+}
+
+extern "C" int htgs_frame_key_bytes(const htgs_frame *f)
+{
+    if (!f) return 0;
+    if (frame_depth_ordered(f)) return htgs_frame_end_bit(f) <= 16 ? 2 : 4;
+    return htgs_key_bytes(f->mode, f->width, f->height);
+}
+
+extern "C" int htgs_frame_sort_passes(const htgs_frame *f)
+{
+    if (!f) return 0;
+    const int bits = htgs_frame_key_bytes(f) == 8 ? 9 : 8;
+    return (htgs_frame_end_bit(f) + bits - 1) / bits;
+}
+
 extern "C" int htgs_sort_passes(int mode, int width, int height)
 {
     // 8 bits per pass, 9 for the 8-byte tile|depth keys (radix_sort.hip)

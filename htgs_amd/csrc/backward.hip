@@ -1010,6 +1010,8 @@ extern "C" int htgs_preprocess_backward(const htgs_frame *f)
     if (f->n_primitives == 0) return HTGS_OK;
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (!f->offsets || (f->n_instances > 0 && !f->grad_rows)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: null pointer");
+    // (a Gaussian's gradient rows are found through offsets[], which must be in index order)
+    if (frame_depth_ordered(f)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: depth_order is for the inference entry points");
     if (!f->positions || !f->scales || !f->rotations || !f->n_touched || !f->clamp_info || !f->M || !f->VPM ||
         !f->cam_position || !f->grad_positions || !f->grad_scales || !f->grad_rotations || !f->grad_opacities || !f->grad_sh_0 ||
         (f->total_sh_bases > 0 && (!f->sh_rest || !f->grad_sh_rest)))

@@ -44,6 +44,28 @@ inline int frame_prim_floats(const htgs_frame *f)
     return f->prim_floats == 0 || f->prim_floats == HTGS_PRIM_FLOATS ? HTGS_PRIM_FLOATS : f->prim_floats == HTGS_PRIM_FLOATS_TRAIN ? HTGS_PRIM_FLOATS_TRAIN : -1;
 }
 
+// ALPHA_BLEND_GLOBAL_ORDERING with the Gaussians sorted by depth before the instances are made (htgs_frame.depth_order)
+inline bool frame_depth_ordered(const htgs_frame *f) { return f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING && f->depth_order != nullptr; }
+// the parts of depth_order, n4 = N rounded up to a multiple of four words each: depth keys and Gaussian indices (two
+// buffers each for the sort, which leaves its result in the first ones after four passes; htgs_preprocess writes the
+// pairs), the counts and the tile rectangles in depth order, scratch of the sort
+struct DepthOrder {
+    uint32_t *keys[2], *vals[2], *counts;
+    uint16_t *bounds;
+    uint32_t *sort_tmp;
+};
+inline DepthOrder depth_order_parts(const htgs_frame *f)
+{
+    const size_t n4 = ((size_t)(f->n_primitives > 0 ? f->n_primitives : 0) + 3) & ~(size_t)3;
+    DepthOrder d;
+    d.keys[0] = f->depth_order; d.keys[1] = f->depth_order + n4;
+    d.vals[0] = f->depth_order + 2 * n4; d.vals[1] = f->depth_order + 3 * n4;
+    d.counts = f->depth_order + 4 * n4; d.bounds = reinterpret_cast<uint16_t *>(f->depth_order + 5 * n4); d.sort_tmp = f->depth_order + 7 * n4;
+    return d;
+}
+// stable sort of n (32-bit key, value) pairs by all 32 key bits (radix_sort.hip); the result is in keys[0] / vals[0]
+int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n);
+
 // host side error reporting (api.hip)
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);

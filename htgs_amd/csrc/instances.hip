@@ -106,32 +106,37 @@ __global__ void __launch_bounds__(kScanBlock) scan_apply_kernel(const uint32_t *
 // gives the tile.  Stores are fully coalesced and a Gaussian covering thousands of tiles costs no more per
 // instance than one covering a single tile.  The emitted order is the reference's: ascending primitive, then
 // row-major tiles.
-template <typename KeyT, bool DEPTH>
+// ORDERED: position i of the walk is Gaussian order[i] (the Gaussians by depth; counts and offsets are in that order).
+template <typename KeyT, bool DEPTH, bool ORDERED = false>
 __global__ void __launch_bounds__(256) create_instances_kernel(
     const uint32_t *__restrict__ n_touched, const uint32_t *__restrict__ offsets, const uint16_t *__restrict__ bounds,
-    float *__restrict__ prim, KeyT *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t grid_w, int n, uint64_t capacity, int prim_floats)
+    float *__restrict__ prim, KeyT *__restrict__ keys, uint32_t *__restrict__ vals, uint32_t grid_w, int n, uint64_t capacity, int prim_floats,
+    const uint32_t *__restrict__ order)
 {
+    static_assert(!(DEPTH && ORDERED), "keys of the tile alone");
     __shared__ uint32_t s_end[256];     // inclusive offsets of the block's Gaussians
-    __shared__ uint32_t s_x0[256], s_y0[256], s_w[256], s_depth[DEPTH ? 256 : 1];
+    __shared__ uint32_t s_x0[256], s_y0[256], s_w[256], s_depth[DEPTH ? 256 : 1], s_gaussian[ORDERED ? 256 : 1];
     __shared__ float s_rw[256];         // 1 / width of the rectangle
     const int first = blockIdx.x * 256;
     const int i = first + threadIdx.x;
     const uint32_t block_start = first == 0 ? 0u : offsets[first - 1];
     const int last_in_block = (first + 255 < n ? first + 255 : n - 1);
     const uint32_t block_end = offsets[last_in_block];
-    uint32_t end = block_end, x0 = 0, y0 = 0, w = 1, depth = 0;
+    uint32_t end = block_end, x0 = 0, y0 = 0, w = 1, depth = 0, gaussian = 0;
     if (i < n) {
         end = offsets[i];
+        gaussian = ORDERED ? order[i] : (uint32_t)i;
         if (n_touched[i] != 0) {
-            const ushort4 b = *reinterpret_cast<const ushort4 *>(bounds + 4 * (size_t)i);
+            const ushort4 b = *reinterpret_cast<const ushort4 *>(bounds + 4 * (size_t)(ORDERED ? (uint32_t)i : gaussian));   // (ORDERED: in that order too)
             x0 = b.x; y0 = b.z; w = (uint32_t)b.y - b.x;
-            if (DEPTH) depth = float_to_bits(prim[(size_t)prim_floats * i + 15]);   // MT3.w = camera-space z of the centre
+            if (DEPTH) depth = float_to_bits(prim[(size_t)prim_floats * gaussian + 15]);   // MT3.w = camera-space z of the centre
             // training records: where the Gaussian's instances start in this (unsorted) list and its rectangle, for the
             // backward pass, which writes a gradient row at the slot of every instance
             if (prim_floats == HTGS_PRIM_FLOATS_TRAIN)
-                *reinterpret_cast<uint4 *>(prim + (size_t)prim_floats * i + HTGS_PRIM_FLOATS) = make_uint4(end - n_touched[i], x0 | y0 << 16, w, 0u);
+                *reinterpret_cast<uint4 *>(prim + (size_t)prim_floats * gaussian + HTGS_PRIM_FLOATS) = make_uint4(end - n_touched[i], x0 | y0 << 16, w, 0u);
         }
     }
+    if (ORDERED) s_gaussian[threadIdx.x] = gaussian;
     s_end[threadIdx.x] = end;
     s_x0[threadIdx.x] = x0; s_y0[threadIdx.x] = y0; s_w[threadIdx.x] = w;
     s_rw[threadIdx.x] = 1.0f / (float)w;
@@ -162,8 +167,27 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
         const uint32_t colm = t - row * wl;
         const uint64_t tile = (uint64_t)(s_y0[l] + row) * grid_w + s_x0[l] + colm;
         keys[e] = DEPTH ? (KeyT)((tile << 32) | (uint64_t)s_depth[l]) : (KeyT)tile;
-        vals[e] = (uint32_t)(first + l);
+        vals[e] = ORDERED ? s_gaussian[l] : (uint32_t)(first + l);
     }
+}
+
+// htgs_frame.depth_order: counts and tile rectangles of the Gaussians in depth order (contiguous for the scan and for
+// create_instances_kernel)
+__global__ void __launch_bounds__(256) gather_counts_kernel(const uint32_t *__restrict__ order, const uint32_t *__restrict__ sorted_keys,
+                                                            const uint16_t *__restrict__ bounds, uint32_t *__restrict__ counts,
+                                                            uint16_t *__restrict__ bounds_out, int n)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    // (a culled Gaussian has the key of all ones and no rectangle; the count of the others is their rectangle's area,
+    // preprocess_kernel's n_touched, so one gather does)
+    uint32_t count = 0;
+    if (sorted_keys[i] != 0xffffffffu) {
+        const ushort4 b = *reinterpret_cast<const ushort4 *>(bounds + 4 * (size_t)order[i]);
+        count = ((uint32_t)b.y - b.x) * ((uint32_t)b.w - b.z);
+        *reinterpret_cast<ushort4 *>(bounds_out + 4 * (size_t)i) = b;
+    }
+    counts[i] = count;
 }
 
 // A thread takes the keys of one 16-byte word (and the key before them) and writes a range boundary wherever two
@@ -298,9 +322,20 @@ static int launch_scan(const htgs_frame *f, uint32_t *tile_sums, const char *who
         return fail(HTGS_ERR_ARGUMENT, "%s: more than 2^20 tiles (images beyond 8192 x 8192 pixels are not supported)", who);
     const int tiles = n > 0 ? div_up(n, kScanTile) : 0;
     if (n > 0 && (!f->n_touched || !f->offsets)) return fail(HTGS_ERR_ARGUMENT, "%s: null pointer", who);
+    const uint32_t *counts = f->n_touched;
+    if (frame_depth_ordered(f) && n > 0) {
+        // the Gaussians by depth first; the scan then runs over their counts in that order
+        if (!f->bounds) return fail(HTGS_ERR_ARGUMENT, "%s: null pointer", who);
+        if ((uintptr_t)f->depth_order & 15) return fail(HTGS_ERR_ARGUMENT, "%s: depth_order must be 16-byte aligned", who);
+        const DepthOrder d = depth_order_parts(f);       // (htgs_preprocess has written the pairs to sort)
+        const int rc = sort_u32_pairs(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n);
+        if (rc != HTGS_OK) return rc;
+        hipLaunchKernelGGL(gather_counts_kernel, dim3(div_up(n, 256)), dim3(256), 0, s, d.vals[0], d.keys[0], f->bounds, d.counts, d.bounds, n);
+        counts = d.counts;
+    }
     if (tiles > 0) {
-        hipLaunchKernelGGL(scan_reduce_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, n);
-        hipLaunchKernelGGL(scan_apply_kernel, dim3(tiles), dim3(kScanBlock), 0, s, f->n_touched, tile_sums, f->offsets, f->n_instances_dev, n);
+        hipLaunchKernelGGL(scan_reduce_kernel, dim3(tiles), dim3(kScanBlock), 0, s, counts, tile_sums, n);
+        hipLaunchKernelGGL(scan_apply_kernel, dim3(tiles), dim3(kScanBlock), 0, s, counts, tile_sums, f->offsets, f->n_instances_dev, n);
     } else {
         hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(256), 0, s, f->n_instances_dev, (size_t)1, (uint32_t *)nullptr, (uint32_t *)nullptr);
     }
@@ -314,6 +349,12 @@ using namespace htgs;
 extern "C" size_t htgs_scan_tmp_words(int n_primitives)
 {
     return (size_t)div_up(n_primitives > 0 ? n_primitives : 1, kScanTile);
+}
+
+extern "C" size_t htgs_depth_order_words(int n_primitives)
+{
+    const size_t n = n_primitives > 0 ? (size_t)n_primitives : 0, n4 = (n + 3) & ~(size_t)3;
+    return 7 * n4 + htgs_sort_tmp_words(n);
 }
 
 extern "C" int htgs_scan_offsets(const htgs_frame *f)
@@ -352,18 +393,26 @@ extern "C" int htgs_create_instances(const htgs_frame *f)
     const int tile = tile_size(f->mode);
     const uint32_t grid_w = div_up(f->width, tile);
     const dim3 grid(div_up(f->n_primitives, 256)), block(256);
-    const int kb = htgs_key_bytes(f->mode, f->width, f->height);
+    const int kb = htgs_frame_key_bytes(f);
     const int prim_floats = frame_prim_floats(f);
     if (prim_floats < 0) return fail(HTGS_ERR_ARGUMENT, "htgs_create_instances: prim_floats must be 0, %d or %d", HTGS_PRIM_FLOATS, HTGS_PRIM_FLOATS_TRAIN);
-    if (kb == 8)
+    if (frame_depth_ordered(f)) {
+        const DepthOrder d = depth_order_parts(f);
+        if (kb == 4)
+            hipLaunchKernelGGL((create_instances_kernel<uint32_t, false, true>), grid, block, 0, s, d.counts, f->offsets, d.bounds, f->prim,
+                               (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, d.vals[0]);
+        else
+            hipLaunchKernelGGL((create_instances_kernel<uint16_t, false, true>), grid, block, 0, s, d.counts, f->offsets, d.bounds, f->prim,
+                               (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, d.vals[0]);
+    } else if (kb == 8)
         hipLaunchKernelGGL((create_instances_kernel<uint64_t, true>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
-                           (uint64_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats);
+                           (uint64_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, (const uint32_t *)nullptr);
     else if (kb == 4)
         hipLaunchKernelGGL((create_instances_kernel<uint32_t, false>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
-                           (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats);
+                           (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, (const uint32_t *)nullptr);
     else
         hipLaunchKernelGGL((create_instances_kernel<uint16_t, false>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
-                           (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats);
+                           (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, (const uint32_t *)nullptr);
     return check_launch("create_instances");
 }
 
@@ -389,7 +438,7 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
     if (f->n_instances > 0) {
         if (!f->keys[selector]) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: null pointer");
         if ((uintptr_t)f->keys[selector] & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_extract_ranges: keys must be 16-byte aligned");
-        const int kb = htgs_key_bytes(f->mode, f->width, f->height);
+        const int kb = htgs_frame_key_bytes(f);
         const uint64_t per_block = 256ull * (16 / kb);
         const dim3 grid((unsigned)((f->n_instances + per_block - 1) / per_block)), block(256);
         if (kb == 8)

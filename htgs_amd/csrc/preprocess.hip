@@ -63,7 +63,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     uint32_t *__restrict__ n_touched, uint16_t *__restrict__ bounds, float *__restrict__ prim,
     uint8_t *__restrict__ clamp_info,
     int n, uint32_t grid_w, uint32_t grid_h, float tile, float min_alpha_rcp,
-    int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier, int rec4)
+    int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier, int rec4,
+    uint32_t *__restrict__ depth_keys, uint32_t *__restrict__ depth_vals)
 {
     // One LDS buffer, used twice: first the block's slice of sh_rest (contiguous in memory, loaded with coalesced
     // 16-byte reads and then read back per Gaussian at a stride of 3 * total_sh words), then the block's records
@@ -151,6 +152,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
         }
     }
     if (in_range) n_touched[i] = touched;
+    // htgs_frame.depth_order: the pairs that sort the Gaussians by depth -- the bits of the centre's camera-space depth
+    // (positive for every Gaussian that is not culled, so the bit patterns order like the depths; these are the low 32
+    // bits of the reference's tile | depth keys), all ones for a culled Gaussian, which so ends up behind the others
+    if (depth_keys != nullptr && in_range) {
+        depth_keys[i] = touched != 0 ? float_to_bits(z) : 0xffffffffu;
+        depth_vals[i] = (uint32_t)i;
+    }
     s_visible[threadIdx.x] = visible;
     if (visible)
         *reinterpret_cast<ushort4 *>(bounds + 4 * (size_t)i) = make_ushort4((uint16_t)b0, (uint16_t)b1, (uint16_t)b2, (uint16_t)b3);
@@ -258,9 +266,13 @@ extern "C" int htgs_preprocess(const htgs_frame *f)
     if (prim_floats < 0) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: prim_floats must be 0, %d or %d", HTGS_PRIM_FLOATS, HTGS_PRIM_FLOATS_TRAIN);
     const size_t lds_bytes = sh_bytes > 256 * prim_floats * sizeof(float) ? sh_bytes : 256 * prim_floats * sizeof(float);
     if (lds_bytes > 64 * 1024) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: sh_rest has more than 21 coefficients per Gaussian");
+    const bool ordered = frame_depth_ordered(f);
+    if (ordered && ((uintptr_t)f->depth_order & 15)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: depth_order must be 16-byte aligned");
+    const DepthOrder order = depth_order_parts(f);
     hipLaunchKernelGGL(preprocess_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), lds_bytes, (hipStream_t)f->stream,
                        f->positions, f->scales, f->rotations, f->opacities, f->sh_0, f->sh_rest, f->M, f->VPM, f->cam_position,
                        f->n_touched, f->bounds, f->prim, f->clamp_info, f->n_primitives, grid_w, grid_h, (float)tile,
-                       min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier, prim_floats / 4);
+                       min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier, prim_floats / 4,
+                       ordered ? order.keys[0] : nullptr, ordered ? order.vals[0] : nullptr);
     return check_launch("preprocess");
 }

@@ -37,11 +37,11 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t launched, uint
 }
 inline uint32_t xcd_padded_grid(uint32_t n_blocks) { return (n_blocks + kXcds - 1) / kXcds * kXcds; }
 
-template <typename KeyT>
-__global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
-                                                                                 uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads>
+__global__ void __launch_bounds__(THREADS) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
+                                                                uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
-    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems, kRadix = 1 << SortDigit<KeyT>::bits;
+    constexpr int kSortThreads = THREADS, kSortTile = kSortThreads * kSortItems, kRadix = 1 << SortDigit<KeyT>::bits;
     static_assert(kRadix <= kSortThreads, "one thread per digit");
     __shared__ uint32_t counts[kRadix];
     const uint32_t block = xcd_contiguous_block(blockIdx.x, n_blocks);
@@ -105,12 +105,12 @@ __global__ void __launch_bounds__(kScanThreads) digit_row_scan_kernel(uint32_t *
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-template <typename KeyT>
-__global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel(
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads>
+__global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
     const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
-    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
+    constexpr int kSortThreads = THREADS, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
     constexpr int kBits = SortDigit<KeyT>::bits, kRadix = 1 << kBits, kDigitWaves = kRadix / kWave;
     // (16-bit counters: a block holds 8192 items; with 512 digits and 8-byte keys two blocks still fit a CU's LDS)
     __shared__ uint16_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the wave's base inside the block
@@ -250,30 +250,38 @@ __global__ void __launch_bounds__(SortShape<KeyT>::threads) digit_scatter_kernel
     }
 }
 
-template <typename KeyT>
-static int sort_pairs(const htgs_frame *f, int end_bit, int *selector)
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads>
+static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int *selector)
 {
-    hipStream_t s = (hipStream_t)f->stream;
-    constexpr int kSortThreads = SortShape<KeyT>::threads, kSortTile = kSortThreads * kSortItems;
-    const uint64_t n = f->n_instances;
+    constexpr int kSortThreads = THREADS, kSortTile = kSortThreads * kSortItems;
     const uint32_t n_blocks = (uint32_t)((n + kSortTile - 1) / kSortTile);
     constexpr int kBits = SortDigit<KeyT>::bits, kRadix = 1 << kBits;
-    uint32_t *hist = f->sort_tmp;
-    uint32_t *totals = f->sort_tmp + (size_t)kRadix * n_blocks;
+    uint32_t *hist = sort_tmp;
+    uint32_t *totals = sort_tmp + (size_t)kRadix * n_blocks;
     int cur = 0;
     for (int shift = 0; shift < end_bit; shift += kBits) {
         const int bits = end_bit - shift < kBits ? end_bit - shift : kBits;
         const uint32_t mask = (1u << bits) - 1u;
-        const KeyT *kin = (const KeyT *)f->keys[cur];
-        KeyT *kout = (KeyT *)f->keys[cur ^ 1];
-        hipLaunchKernelGGL((digit_histogram_kernel<KeyT>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
+        const KeyT *kin = (const KeyT *)keys[cur];
+        KeyT *kout = (KeyT *)keys[cur ^ 1];
+        hipLaunchKernelGGL((digit_histogram_kernel<KeyT, THREADS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
         hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
-        hipLaunchKernelGGL((digit_scatter_kernel<KeyT>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, f->vals[cur], kout, f->vals[cur ^ 1],
+        hipLaunchKernelGGL((digit_scatter_kernel<KeyT, THREADS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, vals[cur], kout, vals[cur ^ 1],
                            hist, totals, n, n_blocks, shift, mask);
         cur ^= 1;
     }
     *selector = cur;
     return check_launch("sort");
+}
+
+int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n)
+{
+    static_assert((32 / SortDigit<uint32_t>::bits) % 2 == 0 && 32 % SortDigit<uint32_t>::bits == 0, "an even number of passes: the result is in the first buffers");
+    if (n == 0) return HTGS_OK;
+    void *const k[2] = { keys[0], keys[1] };
+    int selector = 0;
+    // (a few million pairs: blocks of 4096 items, the smallest the kernels take, so that every compute unit has several)
+    return sort_pairs<uint32_t, kSortTileMin / kSortItems>((hipStream_t)stream, k, vals, sort_tmp, n, 32, &selector);
 }
 
 }  // namespace htgs
@@ -297,10 +305,11 @@ extern "C" int htgs_sort_instances(const htgs_frame *f, int *selector)
     if (!f->keys[0] || !f->keys[1] || !f->vals[0] || !f->vals[1] || !f->sort_tmp)
         return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: null pointer");
     if (((uintptr_t)f->keys[0] | (uintptr_t)f->keys[1]) & 15) return fail(HTGS_ERR_ARGUMENT, "htgs_sort_instances: keys must be 16-byte aligned");
-    const int end_bit = htgs_end_bit(f->mode, f->width, f->height);
-    switch (htgs_key_bytes(f->mode, f->width, f->height)) {
-        case 8: return sort_pairs<uint64_t>(f, end_bit, selector);
-        case 4: return sort_pairs<uint32_t>(f, end_bit, selector);
-        default: return sort_pairs<uint16_t>(f, end_bit, selector);
+    const int end_bit = htgs_frame_end_bit(f);
+    hipStream_t s = (hipStream_t)f->stream;
+    switch (htgs_frame_key_bytes(f)) {
+        case 8: return sort_pairs<uint64_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector);
+        case 4: return sort_pairs<uint32_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector);
+        default: return sort_pairs<uint16_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector);
     }
 }

@@ -120,7 +120,8 @@ class FrameBuffers:
 
     def __init__(self, positions, scales, rotations, opacities, sh_0, sh_rest, settings: RasterizerSettings,
                  to_chw: bool = True, use_median_depth: bool = False, train: bool = False,
-                 pool: Optional[ScratchPool] = None, fast: bool = False, long_list_threshold: int = 0, order_tiles: bool = True):
+                 pool: Optional[ScratchPool] = None, fast: bool = False, long_list_threshold: int = 0, order_tiles: bool = True,
+                 order_gaussians: bool = True):
         mode = _mode_value(settings.mode)
         if mode not in (0, 1, 2, 3):
             raise RuntimeError("unsupported rasterizer mode")
@@ -152,9 +153,6 @@ class FrameBuffers:
         self.grid_w = (self.width + self.tile - 1) // self.tile
         self.grid_h = (self.height + self.tile - 1) // self.tile
         self.n_tiles = self.grid_w * self.grid_h
-        self.key_bytes = self.lib.htgs_key_bytes(mode, self.width, self.height)
-        self.end_bit = self.lib.htgs_end_bit(mode, self.width, self.height)
-        self.sort_passes = self.lib.htgs_sort_passes(mode, self.width, self.height)
         self.to_chw = bool(to_chw)
 
         self.pool = pool
@@ -174,6 +172,10 @@ class FrameBuffers:
         # the tiles in the order the blend kernels take them (longest lists first), written with the ranges
         self.tile_order = (self._scratch("tile_order", self.lib.htgs_tile_order_words(mode, self.width, self.height), torch.int32)
                            if order_tiles else None)
+        # GLOBAL_ORDERING inference: the Gaussians sorted by depth before the instances are made, whose keys then hold the
+        # tile alone (two sort passes over 2-byte keys instead of five over 8-byte keys, the same sorted list)
+        self.depth_order = (self._scratch("depth_order", self.lib.htgs_depth_order_words(n), torch.int32)
+                            if order_gaussians and mode == 2 and not train else None)
         self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
                                  dtype=torch.float32, device=dev)
         # the image-only fast path (``fast_rasterize``) writes no depth map
@@ -202,12 +204,16 @@ class FrameBuffers:
         f.ranges = _ptr(self.ranges)
         f.long_tiles = _ptr(self.long_tiles)
         f.tile_order = _ptr(self.tile_order)
+        f.depth_order = _ptr(self.depth_order)
         f.long_list_threshold = int(long_list_threshold)      # 0: the library's default
         f.image, f.depth = _ptr(self.image), _ptr(self.depth)
         f.to_chw, f.use_median_depth, f.fast_math = int(bool(to_chw)), int(bool(use_median_depth)), int(bool(fast))
         f.stream = torch.cuda.current_stream(dev).cuda_stream
         self.frame = f
         self._ref = ctypes.byref(f)
+        self.key_bytes = self.lib.htgs_frame_key_bytes(self._ref)
+        self.end_bit = self.lib.htgs_frame_end_bit(self._ref)
+        self.sort_passes = self.lib.htgs_frame_sort_passes(self._ref)
 
     def _scratch(self, name: str, numel: int, dtype: torch.dtype, headroom: float = 0.0) -> torch.Tensor:
         """A buffer of at least ``numel`` elements: from the pool if the frame has one, else freshly allocated."""

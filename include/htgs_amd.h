@@ -94,9 +94,16 @@ typedef struct htgs_frame {
                                   that stage.  Every kernel that walks tile lists takes its tiles in this order, so the long
                                   lists are not left for the end of the launch; results do not depend on it.  NULL:
                                   tile order (no counterpart in the reference) */
+    uint32_t *depth_order;     /* htgs_depth_order_words(N) words or NULL.  ALPHA_BLEND_GLOBAL_ORDERING, inference entry
+                                  points: htgs_scan_offsets first sorts the Gaussians by the depth of their centres
+                                  (stable), offsets[] then is the prefix sum in that order and htgs_create_instances emits
+                                  the instances in it, with keys that hold the tile alone: the stable sort by tile that
+                                  follows leaves every tile's list in the order of the reference's sort by tile | depth
+                                  (same sorted vals, same ranges) in two passes over 2-byte keys instead of five over
+                                  8-byte keys.  NULL: the reference's keys (no counterpart in the reference) */
     /* ---- per-instance scratch (PerInstanceBuffers, buffer_utils.h:56-84) ---- */
     uint64_t n_instances;      /* host copy of *n_instances_dev, needed from htgs_create_instances on */
-    void *keys[2];             /* [n_instances] of htgs_key_bytes() each, ping-pong, 16-byte aligned */
+    void *keys[2];             /* [n_instances] of htgs_frame_key_bytes() each, ping-pong, 16-byte aligned */
     uint32_t *vals[2];         /* [n_instances] primitive index, ping-pong */
     uint32_t *sort_tmp;        /* htgs_sort_tmp_words(n_instances) words */
     /* ---- outputs (rasterization_api.cu:392-393) ---- */
@@ -143,6 +150,12 @@ int htgs_effective_k(int K);
 int htgs_end_bit(int mode, int width, int height);
 /* 2, 4 or 8: ushort / uint / uint64_t keys (R/src/hybrid_blend/inference.cu:121-129) */
 int htgs_key_bytes(int mode, int width, int height);
+/* the same for a frame: as above unless the frame has depth_order, then those of the tile alone */
+int htgs_frame_end_bit(const htgs_frame *f);
+int htgs_frame_key_bytes(const htgs_frame *f);
+int htgs_frame_sort_passes(const htgs_frame *f);
+/* words of htgs_frame.depth_order for N Gaussians */
+size_t htgs_depth_order_words(int n_primitives);
 /* digit passes htgs_sort_instances takes (8 bits per pass, 9 for 8-byte keys); the sorted pairs end up in keys/vals[passes & 1] */
 int htgs_sort_passes(int mode, int width, int height);
 size_t htgs_scan_tmp_words(int n_primitives);

@@ -1,0 +1,81 @@
+"""ALPHA_BLEND_GLOBAL_ORDERING with the Gaussians sorted by depth before the instances are made (htgs_frame.depth_order):
+the instance keys then hold the tile alone, and the stable sort by tile leaves every tile's list in the order of the
+reference's sort of tile | depth keys (cub::DeviceRadixSort over both, R/src/alpha_blend_global_ordering/inference.cu:117-124).
+The sorted primitive indices and the ranges must be the oracle's, the image the one of the frame with the reference's keys."""
+import numpy as np
+import pytest
+import torch
+
+from htgs_amd.synthetic import make_scene
+from htgs_amd.torch_bindings import FrameBuffers, RasterizerMode, rasterize
+from util import gpu_stages, oracle_render
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("config,n,K", [(0, 3000, 4), (1, 60_000, 16), (2, 200_000, 16), (3, 100_000, 16), (4, 50_000, 8)])
+def test_depth_order_gives_the_reference_lists(cuda, config, n, K):
+    print(f"case config={config} n={n} K={K}", flush=True)
+    scene = make_scene(config, n)
+    ref = oracle_render(scene, 2, K)
+    got = gpu_stages(scene.to(cuda), 2, K, order_gaussians=True)
+    keyed = gpu_stages(scene.to(cuda), 2, K, order_gaussians=False)
+    assert got["fb"].key_bytes == 2 and keyed["fb"].key_bytes == 8
+    assert got["n_instances"] == len(ref["keys"])
+    np.testing.assert_array_equal(got["n_touched"], ref["pre"]["n_touched"])
+    np.testing.assert_array_equal(got["sorted_vals"], ref["sorted_vals"])
+    np.testing.assert_array_equal(got["sorted_keys"], ref["sorted_keys"] >> np.uint64(32))
+    np.testing.assert_array_equal(got["ranges"], ref["ranges"])
+    assert np.array_equal(got["image"], keyed["image"]) and np.array_equal(got["depth"], keyed["depth"])
+    assert np.abs(got["image"] - ref["image"]).max() <= 1e-4 and np.abs(got["depth"] - ref["depth"]).max() <= 1e-4
+    # offsets: the prefix sums of the counts in depth order (culled Gaussians last)
+    order = got["fb"].depth_order[2 * ((n + 3) // 4 * 4):][:n].cpu().numpy().view(np.uint32)
+    depth = got["MT3"][:, 3]
+    seen = got["n_touched"][order] > 0
+    assert not seen[np.argmin(seen):].any() if not seen.all() else True
+    d = depth[order][seen]
+    assert (np.diff(d) >= 0).all()
+    same = np.diff(d) == 0
+    assert (np.diff(order[seen].astype(np.int64))[same] > 0).all()      # equal depths: ascending index (stable)
+    np.testing.assert_array_equal(got["offsets"], np.cumsum(got["n_touched"][order].astype(np.uint64)).astype(np.uint32))
+
+
+def test_depth_order_with_equal_depths(cuda):
+    """Coincident Gaussians (equal depths by the thousand): the order inside a depth is the index order, as in the
+    reference's stable sort of equal keys."""
+    scene = make_scene(0, 1000)
+    rep = lambda t: t.repeat(4, *([1] * (t.dim() - 1))).contiguous()
+    import dataclasses
+    g = torch.Generator().manual_seed(3)
+    scene = dataclasses.replace(scene, name="cfg0-copies", positions=rep(scene.positions), scales=rep(scene.scales), rotations=rep(scene.rotations),
+                                opacities=rep(scene.opacities), sh_0=(rep(scene.sh_0) + 0.3 * torch.randn(4000, *scene.sh_0.shape[1:], generator=g)).contiguous(),
+                                sh_rest=rep(scene.sh_rest))
+    ref = oracle_render(scene, 2, 4)
+    got = gpu_stages(scene.to(cuda), 2, 4, order_gaussians=True)
+    np.testing.assert_array_equal(got["sorted_vals"], ref["sorted_vals"])
+    np.testing.assert_array_equal(got["ranges"], ref["ranges"])
+    assert np.abs(got["image"] - ref["image"]).max() <= 1e-4
+
+
+def test_depth_order_empty_and_all_culled(cuda):
+    scene = make_scene(0, 500).to(cuda)
+    s = scene.settings(RasterizerMode.ALPHA_BLEND_GLOBAL_ORDERING, 4)
+    g = list(scene.gaussians())
+    g[0] = g[0].clone(); g[0][:, 2] = -5.0                     # everything behind the camera
+    image, depth = rasterize(*g, s, True, False)
+    assert float(image.abs().max()) == 0.0
+    empty = [t[:0].contiguous() for t in scene.gaussians()]
+    image, depth = rasterize(*empty, s, True, False)
+    assert float(image.abs().max()) == 0.0
+
+
+def test_rasterize_takes_the_depth_order(cuda):
+    scene = make_scene(1, 100_000).to(cuda)
+    s = scene.settings(RasterizerMode.ALPHA_BLEND_GLOBAL_ORDERING, 16)
+    fb = FrameBuffers(*scene.gaussians(), s, True, False)
+    assert fb.depth_order is not None and fb.key_bytes == 2
+    image, depth = rasterize(*scene.gaussians(), s, True, False)
+    keyed = FrameBuffers(*scene.gaussians(), s, True, False, order_gaussians=False)
+    keyed.run()
+    torch.cuda.synchronize()
+    assert torch.equal(image, keyed.image) and torch.equal(depth.reshape(keyed.depth.shape), keyed.depth)

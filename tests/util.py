@@ -24,10 +24,11 @@ def u32(t: torch.Tensor) -> np.ndarray:
     return a.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
 
 
-def gpu_stages(scene_gpu: Scene, mode: int, K=None, to_chw=True, median=False, scale_modifier=1.0) -> dict:
-    """Runs the frame stage by stage through the C ABI and returns every intermediate as numpy."""
+def gpu_stages(scene_gpu: Scene, mode: int, K=None, to_chw=True, median=False, scale_modifier=1.0, order_gaussians=False) -> dict:
+    """Runs the frame stage by stage through the C ABI and returns every intermediate as numpy.  (GLOBAL_ORDERING with the
+    reference's tile | depth keys unless ``order_gaussians``, so that offsets and keys compare with the oracle's.)"""
     settings = scene_gpu.settings(RasterizerMode(int(mode)), K, scale_modifier)
-    fb = FrameBuffers(*scene_gpu.gaussians(), settings, to_chw, median)
+    fb = FrameBuffers(*scene_gpu.gaussians(), settings, to_chw, median, order_gaussians=order_gaussians)
     fb.n_touched.fill_(-1)
     fb.bounds.zero_()
     fb.prim.zero_()
