@@ -63,8 +63,36 @@ inline DepthOrder depth_order_parts(const htgs_frame *f)
     d.counts = f->depth_order + 4 * n4; d.bounds = reinterpret_cast<uint16_t *>(f->depth_order + 5 * n4); d.sort_tmp = f->depth_order + 7 * n4;
     return d;
 }
-// stable sort of n (32-bit key, value) pairs by all 32 key bits (radix_sort.hip); the result is in keys[0] / vals[0]
-int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n);
+// The keys that sort the Gaussians by depth: the bit pattern of the centre's camera-space depth (for positive depths the
+// patterns order like the depths; these are the low 32 bits of the reference's tile | depth keys) less that of the near
+// plane, which no Gaussian that is not culled lies in front of, `culled` for a culled Gaussian (behind all others).  With
+// the far plane as the upper bound the keys of the usual cameras have 27 bits: three passes of 9-bit digits.
+struct DepthKeys {
+    uint32_t base, culled;
+    int end_bit, digit_bits, passes;
+};
+inline DepthKeys depth_key_range(const htgs_frame *f)
+{
+    DepthKeys k = { 0u, 0xffffffffu, 32, 8, 4 };
+    const float near_plane = f->near_plane, far_plane = f->far_plane;
+    if (near_plane > 0.0f && far_plane >= near_plane && far_plane < __builtin_huge_valf()) {
+        uint32_t lo, hi;
+        __builtin_memcpy(&lo, &near_plane, 4);
+        __builtin_memcpy(&hi, &far_plane, 4);
+        k.base = lo;
+        k.culled = hi - lo + 1u;
+        k.end_bit = 1;
+        while (k.end_bit < 32 && (k.culled >> k.end_bit) != 0u) ++k.end_bit;
+        const int passes8 = (k.end_bit + 7) / 8, passes9 = (k.end_bit + 8) / 9;
+        k.digit_bits = passes9 < passes8 ? 9 : 8;
+        k.passes = passes9 < passes8 ? passes9 : passes8;
+    }
+    return k;
+}
+// stable sort of n (32-bit key, value) pairs by the low end_bit key bits, digit_bits (8 or 9) a pass (radix_sort.hip);
+// the result is in keys / vals[*selector]
+int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int digit_bits,
+                   int *selector);
 
 // host side error reporting (api.hip)
 int fail(int code, const char *fmt, ...);

@@ -175,14 +175,14 @@ __global__ void __launch_bounds__(256) create_instances_kernel(
 // create_instances_kernel)
 __global__ void __launch_bounds__(256) gather_counts_kernel(const uint32_t *__restrict__ order, const uint32_t *__restrict__ sorted_keys,
                                                             const uint16_t *__restrict__ bounds, uint32_t *__restrict__ counts,
-                                                            uint16_t *__restrict__ bounds_out, int n)
+                                                            uint16_t *__restrict__ bounds_out, int n, uint32_t culled)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
-    // (a culled Gaussian has the key of all ones and no rectangle; the count of the others is their rectangle's area,
+    // (a culled Gaussian has the key `culled` and no rectangle; the count of the others is their rectangle's area,
     // preprocess_kernel's n_touched, so one gather does)
     uint32_t count = 0;
-    if (sorted_keys[i] != 0xffffffffu) {
+    if (sorted_keys[i] != culled) {
         const ushort4 b = *reinterpret_cast<const ushort4 *>(bounds + 4 * (size_t)order[i]);
         count = ((uint32_t)b.y - b.x) * ((uint32_t)b.w - b.z);
         *reinterpret_cast<ushort4 *>(bounds_out + 4 * (size_t)i) = b;
@@ -328,9 +328,11 @@ static int launch_scan(const htgs_frame *f, uint32_t *tile_sums, const char *who
         if (!f->bounds) return fail(HTGS_ERR_ARGUMENT, "%s: null pointer", who);
         if ((uintptr_t)f->depth_order & 15) return fail(HTGS_ERR_ARGUMENT, "%s: depth_order must be 16-byte aligned", who);
         const DepthOrder d = depth_order_parts(f);       // (htgs_preprocess has written the pairs to sort)
-        const int rc = sort_u32_pairs(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n);
+        const DepthKeys k = depth_key_range(f);
+        int sel = 0;
+        const int rc = sort_u32_pairs(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n, k.end_bit, k.digit_bits, &sel);
         if (rc != HTGS_OK) return rc;
-        hipLaunchKernelGGL(gather_counts_kernel, dim3(div_up(n, 256)), dim3(256), 0, s, d.vals[0], d.keys[0], f->bounds, d.counts, d.bounds, n);
+        hipLaunchKernelGGL(gather_counts_kernel, dim3(div_up(n, 256)), dim3(256), 0, s, d.vals[sel], d.keys[sel], f->bounds, d.counts, d.bounds, n, k.culled);
         counts = d.counts;
     }
     if (tiles > 0) {
@@ -355,6 +357,13 @@ extern "C" size_t htgs_depth_order_words(int n_primitives)
 {
     const size_t n = n_primitives > 0 ? (size_t)n_primitives : 0, n4 = (n + 3) & ~(size_t)3;
     return 7 * n4 + htgs_sort_tmp_words(n);
+}
+
+extern "C" size_t htgs_depth_order_result_word(const htgs_frame *f)
+{
+    if (!f) return 0;
+    const size_t n = f->n_primitives > 0 ? (size_t)f->n_primitives : 0, n4 = (n + 3) & ~(size_t)3;
+    return (2 + (size_t)(depth_key_range(f).passes & 1)) * n4;
 }
 
 extern "C" int htgs_scan_offsets(const htgs_frame *f)
@@ -400,10 +409,10 @@ extern "C" int htgs_create_instances(const htgs_frame *f)
         const DepthOrder d = depth_order_parts(f);
         if (kb == 4)
             hipLaunchKernelGGL((create_instances_kernel<uint32_t, false, true>), grid, block, 0, s, d.counts, f->offsets, d.bounds, f->prim,
-                               (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, d.vals[0]);
+                               (uint32_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, d.vals[depth_key_range(f).passes & 1]);
         else
             hipLaunchKernelGGL((create_instances_kernel<uint16_t, false, true>), grid, block, 0, s, d.counts, f->offsets, d.bounds, f->prim,
-                               (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, d.vals[0]);
+                               (uint16_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, d.vals[depth_key_range(f).passes & 1]);
     } else if (kb == 8)
         hipLaunchKernelGGL((create_instances_kernel<uint64_t, true>), grid, block, 0, s, f->n_touched, f->offsets, f->bounds, f->prim,
                            (uint64_t *)f->keys[0], f->vals[0], grid_w, f->n_primitives, f->n_instances, prim_floats, (const uint32_t *)nullptr);

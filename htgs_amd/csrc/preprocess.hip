@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     uint8_t *__restrict__ clamp_info,
     int n, uint32_t grid_w, uint32_t grid_h, float tile, float min_alpha_rcp,
     int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier, int rec4,
-    uint32_t *__restrict__ depth_keys, uint32_t *__restrict__ depth_vals)
+    uint32_t *__restrict__ depth_keys, uint32_t *__restrict__ depth_vals, uint32_t depth_base, uint32_t depth_culled)
 {
     // One LDS buffer, used twice: first the block's slice of sh_rest (contiguous in memory, loaded with coalesced
     // 16-byte reads and then read back per Gaussian at a stride of 3 * total_sh words), then the block's records
@@ -152,11 +152,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
         }
     }
     if (in_range) n_touched[i] = touched;
-    // htgs_frame.depth_order: the pairs that sort the Gaussians by depth -- the bits of the centre's camera-space depth
-    // (positive for every Gaussian that is not culled, so the bit patterns order like the depths; these are the low 32
-    // bits of the reference's tile | depth keys), all ones for a culled Gaussian, which so ends up behind the others
+    // htgs_frame.depth_order: the pairs that sort the Gaussians by depth (depth_key_range() in common.h)
     if (depth_keys != nullptr && in_range) {
-        depth_keys[i] = touched != 0 ? float_to_bits(z) : 0xffffffffu;
+        depth_keys[i] = touched != 0 ? float_to_bits(z) - depth_base : depth_culled;
         depth_vals[i] = (uint32_t)i;
     }
     s_visible[threadIdx.x] = visible;
@@ -269,10 +267,11 @@ extern "C" int htgs_preprocess(const htgs_frame *f)
     const bool ordered = frame_depth_ordered(f);
     if (ordered && ((uintptr_t)f->depth_order & 15)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess: depth_order must be 16-byte aligned");
     const DepthOrder order = depth_order_parts(f);
+    const DepthKeys order_keys = depth_key_range(f);
     hipLaunchKernelGGL(preprocess_kernel, dim3(div_up(f->n_primitives, 256)), dim3(256), lds_bytes, (hipStream_t)f->stream,
                        f->positions, f->scales, f->rotations, f->opacities, f->sh_0, f->sh_rest, f->M, f->VPM, f->cam_position,
                        f->n_touched, f->bounds, f->prim, f->clamp_info, f->n_primitives, grid_w, grid_h, (float)tile,
                        min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier, prim_floats / 4,
-                       ordered ? order.keys[0] : nullptr, ordered ? order.vals[0] : nullptr);
+                       ordered ? order.keys[0] : nullptr, ordered ? order.vals[0] : nullptr, order_keys.base, order_keys.culled);
     return check_launch("preprocess");
 }

@@ -37,11 +37,11 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t launched, uint
 }
 inline uint32_t xcd_padded_grid(uint32_t n_blocks) { return (n_blocks + kXcds - 1) / kXcds * kXcds; }
 
-template <typename KeyT, int THREADS = SortShape<KeyT>::threads>
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = SortDigit<KeyT>::bits>
 __global__ void __launch_bounds__(THREADS) digit_histogram_kernel(const KeyT *__restrict__ keys, uint32_t *__restrict__ hist,
                                                                 uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
-    constexpr int kSortThreads = THREADS, kSortTile = kSortThreads * kSortItems, kRadix = 1 << SortDigit<KeyT>::bits;
+    constexpr int kSortThreads = THREADS, kSortTile = kSortThreads * kSortItems, kRadix = 1 << BITS;
     static_assert(kRadix <= kSortThreads, "one thread per digit");
     __shared__ uint32_t counts[kRadix];
     const uint32_t block = xcd_contiguous_block(blockIdx.x, n_blocks);
@@ -105,13 +105,13 @@ __global__ void __launch_bounds__(kScanThreads) digit_row_scan_kernel(uint32_t *
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-template <typename KeyT, int THREADS = SortShape<KeyT>::threads>
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = SortDigit<KeyT>::bits>
 __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
     const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
 {
     constexpr int kSortThreads = THREADS, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
-    constexpr int kBits = SortDigit<KeyT>::bits, kRadix = 1 << kBits, kDigitWaves = kRadix / kWave;
+    constexpr int kBits = BITS, kRadix = 1 << kBits, kDigitWaves = kRadix / kWave;
     // (16-bit counters: a block holds 8192 items; with 512 digits and 8-byte keys two blocks still fit a CU's LDS)
     __shared__ uint16_t counts[kSortWaves][kRadix];    // per wave: running digit count, later the wave's base inside the block
     __shared__ uint32_t digit_start[kRadix];           // first slot of each digit in the block-local order
@@ -250,12 +250,12 @@ __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
     }
 }
 
-template <typename KeyT, int THREADS = SortShape<KeyT>::threads>
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = SortDigit<KeyT>::bits>
 static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int *selector)
 {
     constexpr int kSortThreads = THREADS, kSortTile = kSortThreads * kSortItems;
     const uint32_t n_blocks = (uint32_t)((n + kSortTile - 1) / kSortTile);
-    constexpr int kBits = SortDigit<KeyT>::bits, kRadix = 1 << kBits;
+    constexpr int kBits = BITS, kRadix = 1 << kBits;
     uint32_t *hist = sort_tmp;
     uint32_t *totals = sort_tmp + (size_t)kRadix * n_blocks;
     int cur = 0;
@@ -264,9 +264,9 @@ static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2
         const uint32_t mask = (1u << bits) - 1u;
         const KeyT *kin = (const KeyT *)keys[cur];
         KeyT *kout = (KeyT *)keys[cur ^ 1];
-        hipLaunchKernelGGL((digit_histogram_kernel<KeyT, THREADS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
+        hipLaunchKernelGGL((digit_histogram_kernel<KeyT, THREADS, BITS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
         hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
-        hipLaunchKernelGGL((digit_scatter_kernel<KeyT, THREADS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, vals[cur], kout, vals[cur ^ 1],
+        hipLaunchKernelGGL((digit_scatter_kernel<KeyT, THREADS, BITS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, vals[cur], kout, vals[cur ^ 1],
                            hist, totals, n, n_blocks, shift, mask);
         cur ^= 1;
     }
@@ -274,14 +274,16 @@ static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2
     return check_launch("sort");
 }
 
-int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n)
+int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int digit_bits,
+                   int *selector)
 {
-    static_assert((32 / SortDigit<uint32_t>::bits) % 2 == 0 && 32 % SortDigit<uint32_t>::bits == 0, "an even number of passes: the result is in the first buffers");
+    *selector = 0;
     if (n == 0) return HTGS_OK;
     void *const k[2] = { keys[0], keys[1] };
-    int selector = 0;
-    // (a few million pairs: blocks of 4096 items, the smallest the kernels take, so that every compute unit has several)
-    return sort_pairs<uint32_t, kSortTileMin / kSortItems>((hipStream_t)stream, k, vals, sort_tmp, n, 32, &selector);
+    // a few million pairs: with 8-bit digits blocks of 4096 items, the smallest the kernels take, so that every compute
+    // unit has several; 9-bit digits need a thread per digit (8192 items)
+    if (digit_bits == 9) return sort_pairs<uint32_t, 512, 9>((hipStream_t)stream, k, vals, sort_tmp, n, end_bit, selector);
+    return sort_pairs<uint32_t, kSortTileMin / kSortItems, 8>((hipStream_t)stream, k, vals, sort_tmp, n, end_bit, selector);
 }
 
 }  // namespace htgs

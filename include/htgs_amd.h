@@ -156,6 +156,8 @@ int htgs_frame_key_bytes(const htgs_frame *f);
 int htgs_frame_sort_passes(const htgs_frame *f);
 /* words of htgs_frame.depth_order for N Gaussians */
 size_t htgs_depth_order_words(int n_primitives);
+/* after htgs_scan_offsets: the word of depth_order at which the N Gaussian indices in depth order start (for tests) */
+size_t htgs_depth_order_result_word(const htgs_frame *f);
 /* digit passes htgs_sort_instances takes (8 bits per pass, 9 for 8-byte keys); the sorted pairs end up in keys/vals[passes & 1] */
 int htgs_sort_passes(int mode, int width, int height);
 size_t htgs_scan_tmp_words(int n_primitives);

@@ -29,7 +29,8 @@ def test_depth_order_gives_the_reference_lists(cuda, config, n, K):
     assert np.array_equal(got["image"], keyed["image"]) and np.array_equal(got["depth"], keyed["depth"])
     assert np.abs(got["image"] - ref["image"]).max() <= 1e-4 and np.abs(got["depth"] - ref["depth"]).max() <= 1e-4
     # offsets: the prefix sums of the counts in depth order (culled Gaussians last)
-    order = got["fb"].depth_order[2 * ((n + 3) // 4 * 4):][:n].cpu().numpy().view(np.uint32)
+    fb = got["fb"]
+    order = fb.depth_order[fb.lib.htgs_depth_order_result_word(fb._ref):][:n].cpu().numpy().view(np.uint32)
     depth = got["MT3"][:, 3]
     seen = got["n_touched"][order] > 0
     assert not seen[np.argmin(seen):].any() if not seen.all() else True
@@ -79,3 +80,17 @@ def test_rasterize_takes_the_depth_order(cuda):
     keyed.run()
     torch.cuda.synchronize()
     assert torch.equal(image, keyed.image) and torch.equal(depth.reshape(keyed.depth.shape), keyed.depth)
+
+
+@pytest.mark.parametrize("near,far", [(0.2, 1000.0), (1e-3, 1e6), (0.0, 100.0), (0.5, float("inf"))])
+def test_depth_order_key_ranges(cuda, near, far):
+    """The depth keys are taken relative to the near plane's bit pattern and are as wide as the far plane makes them
+    (three or four digit passes); without a positive near plane or with an infinite far plane they are the full 32 bits."""
+    import dataclasses
+    print(f"case near={near} far={far}", flush=True)
+    scene = dataclasses.replace(make_scene(0, 4000), near_plane=near, far_plane=far)
+    ref = oracle_render(scene, 2, 8)
+    got = gpu_stages(scene.to(cuda), 2, 8, order_gaussians=True)
+    np.testing.assert_array_equal(got["sorted_vals"], ref["sorted_vals"])
+    np.testing.assert_array_equal(got["ranges"], ref["ranges"])
+    assert np.abs(got["image"] - ref["image"]).max() <= 1e-4
