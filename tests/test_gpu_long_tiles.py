@@ -236,3 +236,24 @@ def test_long_tiles_first_k_with_fragments_of_equal_depth(cuda, config, n, K, th
     print(f"  long tiles {long_tiles}, second looks {second_looks}, walked again {walked_again}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
     assert long_tiles > 0 and (second_looks > 0 if twins else walked_again > 0)
     assert err_i <= TOL and err_d <= TOL
+
+
+@pytest.mark.parametrize("mode,K", [(0, 1), (1, 1), (3, 1), (0, 16)])
+def test_long_tiles_on_a_grid_of_four_tiles(cuda, mode, K):
+    """A 16x16 image: the parts that lists may be walked in beyond one per tile are held to the number of tiles, which
+    here is four."""
+    import dataclasses
+    print(f"case mode={mode} K={K} (16x16 image)", flush=True)
+    scene = make_scene(0, 300_000)
+    positions = scene.positions.clone()
+    positions[:, :2] -= 1.6                                 # (the cloud's centre projects to the image's corner, which is the new image)
+    scene = dataclasses.replace(scene, positions=positions, width=16, height=16)
+    m = RasterizerMode(mode)
+    ref = oracle_render(scene, mode, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, 64, mode=m)
+    single, single_depth, none = render(scene.to(cuda), K, NEVER, mode=m)
+    assert long_tiles > 0 and none == 0
+    err = [float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max()),
+           float(np.abs(image - single).max()), float(np.abs(depth - single_depth).max())]
+    print(f"  long tiles {long_tiles}; against the oracle {err[0]:.3g} / {err[1]:.3g}, against the single walk {err[2]:.3g} / {err[3]:.3g}", flush=True)
+    assert max(err) <= TOL
