@@ -94,3 +94,16 @@ def test_depth_order_key_ranges(cuda, near, far):
     np.testing.assert_array_equal(got["sorted_vals"], ref["sorted_vals"])
     np.testing.assert_array_equal(got["ranges"], ref["ranges"])
     assert np.abs(got["image"] - ref["image"]).max() <= 1e-4
+
+
+@pytest.mark.parametrize("n", [1, 5, 257, 4097])
+def test_depth_order_small_counts(cuda, n):
+    """Counts that are no multiple of the buffers' alignment or of a sort block."""
+    print(f"case n={n}", flush=True)
+    scene = make_scene(0, n)
+    ref = oracle_render(scene, 2, 4)
+    got = gpu_stages(scene.to(cuda), 2, 4, order_gaussians=True)
+    assert got["n_instances"] == len(ref["keys"])
+    np.testing.assert_array_equal(got["sorted_vals"], ref["sorted_vals"])
+    np.testing.assert_array_equal(got["ranges"], ref["ranges"])
+    assert np.abs(got["image"] - ref["image"]).max() <= 1e-4
