@@ -163,6 +163,9 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
 // ---------------------------------------------------------------------------------------------
 constexpr uint32_t kLongHeader = 8, kLongRounds = 3, kLongParts = 32;
 constexpr int kLongWaves = 16;
+// waves of a workgroup of the K-buffer kernels: sixteen share a compute unit's registers at 128 a lane, which a K-buffer of
+// 32 slots (96 registers) leaves too few of; eight have 256
+template <int K> constexpr int long_waves() { return K > 16 ? 8 : kLongWaves; }
 constexpr uint32_t kLongListDefault = 8192;
 // What a workgroup leaves of its part of a list, in 64-lane rows: HYBRID's core, tail and the depth of a tie.
 template <int K> constexpr uint32_t long_part_words() { return (3u * K + 7u) * 64u; }
@@ -231,11 +234,12 @@ __device__ __forceinline__ bool long_tile_take(const uint32_t *long_tiles, const
     }
 }
 // share of wave `wave` of [first, last): whole batches of 64
-__device__ __forceinline__ void long_wave_share(uint32_t first, uint32_t last, uint32_t wave, uint32_t &share_first, uint32_t &share_last)
+__device__ __forceinline__ void long_wave_share(uint32_t first, uint32_t last, uint32_t wave, uint32_t &share_first, uint32_t &share_last,
+                                                uint32_t waves = kLongWaves)
 {
     const uint32_t n_batches = (last - first + 63u) / 64u;
-    share_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / kLongWaves);
-    share_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / kLongWaves);
+    share_first = first + 64u * (uint32_t)((uint64_t)n_batches * wave / waves);
+    share_last = first + 64u * (uint32_t)((uint64_t)n_batches * (wave + 1) / waves);
     share_last = share_last < last ? share_last : last;
 }
 // One of several parts is done and the first wave has written what it left (and called __threadfence()): whether the
@@ -402,19 +406,20 @@ __device__ __forceinline__ void hybrid_merge(const float *from, uint32_t lane, f
 // everything else in its tail, as in a single walk; what differs from the single walk is the order in which the tail's
 // sums are added (rounding) and which of two stored fragments of exactly equal depth is kept when a nearer one arrives.
 template <int K, bool FAST>
-__global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
+__global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
     uint32_t *__restrict__ shortlist, uint32_t long_threshold)
 {
-    __shared__ TileStage<64> st[kLongWaves];
+    constexpr int kWaves = long_waves<K>();
+    __shared__ TileStage<64> st[kWaves];
     __shared__ float s_merge[3 * K + 7][64];          // one wave's core, tail and least depth of a tie, lane-minor
     __shared__ uint32_t s_next;
     __shared__ uint32_t s_redo[2];                    // the pixels (lanes) to walk again
-    __shared__ uint32_t s_short[kLongWaves];          // how many instances of each share reach one of them
+    __shared__ uint32_t s_short[kWaves];          // how many instances of each share reach one of them
     __shared__ uint32_t s_whole;                      // this workgroup finished the last part of its tile
     __shared__ float s_last_depth[64];                // depth of the merged core's last entry
-    __shared__ float s_sums[kLongWaves][kAgainPixels][6], s_tails[64][6];   // tails of the pixels looked at again: per wave, whole
+    __shared__ float s_sums[kWaves][kAgainPixels][6], s_tails[64][6];   // tails of the pixels looked at again: per wave, whole
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (long_tiles[0] == 0) return;                   // (the ordinary frame)
     const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
@@ -426,7 +431,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
         const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
         uint32_t n_batches = (last - first + 63u) / 64u;
         uint32_t seg_first, seg_last;
-        long_wave_share(first, last, wave, seg_first, seg_last);
+        long_wave_share(first, last, wave, seg_first, seg_last, kWaves);
         constexpr bool kTies = !FAST;
         HybridTail tail;
         hybrid_tail_init(tail);
@@ -434,7 +439,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
         hybrid_core_init<K>(cd, ca, ci);
         float tie = __FLT_MAX__;                        // least depth at which two fragments of equal depth met at the end of a core
         hybrid_walk<K, FAST, false, kTies>(st[wave], inst, prim, seg_first, seg_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, &tie);
-        for (uint32_t s = 1; s < (uint32_t)kLongWaves; ++s) {
+        for (uint32_t s = 1; s < (uint32_t)kWaves; ++s) {
             __syncthreads();                               // the buffer is free
             if (wave == s) {
 #pragma unroll
@@ -470,7 +475,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                     hybrid_merge<K, FAST>(left + (size_t)other * long_part_words<K>(), lane, cd, ca, ci, tail, tie);
             }
             first = tile_first; last = tile_last; n_batches = (last - first + 63u) / 64u;
-            long_wave_share(first, last, wave, seg_first, seg_last);
+            long_wave_share(first, last, wave, seg_first, seg_last, kWaves);
             __syncthreads();                               // (the parts are read before the shortlist overwrites them)
         }
         if (kTies) {
@@ -514,7 +519,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                                 for (int j = 1; j < kAgainPixels; ++j) mine = lane == (uint32_t)j ? pixel[j] : mine;
                                 if (mine < 64u) {
                                     float T = 1.0f, sum[5] = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f };
-                                    for (int w = 0; w < kLongWaves; ++w) {
+                                    for (int w = 0; w < kWaves; ++w) {
                                         T *= s_sums[w][lane][0];
 #pragma unroll
                                         for (int k = 0; k < 5; ++k) sum[k] += s_sums[w][lane][1 + k];
@@ -529,7 +534,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                     if (lane == 0) s_short[wave] = listed;
                     __syncthreads();
                     bool settled = true;
-                    for (int w = 0; w < kLongWaves; ++w) settled = settled && s_short[w] != ~0u;
+                    for (int w = 0; w < kWaves; ++w) settled = settled && s_short[w] != ~0u;
                     __syncthreads();                            // (s_short is written again below)
                     if (settled) {
                         if (wave == 0) {
@@ -538,8 +543,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                             hybrid_core_init<K>(cd, ca, ci);
                             tail.T = s_tails[lane][0]; tail.c0 = s_tails[lane][1]; tail.c1 = s_tails[lane][2]; tail.c2 = s_tails[lane][3];
                             tail.alpha = s_tails[lane][4]; tail.depth = s_tails[lane][5];
-                            for (uint32_t w = 0; w < (uint32_t)kLongWaves; ++w) {
-                                const uint32_t *entry = shortlist + first + 64u * (uint32_t)((uint64_t)n_batches * w / kLongWaves);
+                            for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
+                                const uint32_t *entry = shortlist + first + 64u * (uint32_t)((uint64_t)n_batches * w / kWaves);
                                 for (uint32_t left = s_short[w]; left != 0; --left, entry += 4) {
                                     float depth = bits_to_float(entry[1]), alpha = bits_to_float(entry[2]), index = bits_to_float(entry[3]);
                                     if (lane == entry[0]) {
@@ -574,8 +579,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_hybrid_long_kernel(
                     hybrid_tail_init(tail);
                     hybrid_core_init<K>(cd, ca, ci);
                     if (shortlist != nullptr) {
-                        for (uint32_t s = 0; s < (uint32_t)kLongWaves; ++s) {
-                            const uint32_t from = first + 64u * (uint32_t)((uint64_t)n_batches * s / kLongWaves);
+                        for (uint32_t s = 0; s < (uint32_t)kWaves; ++s) {
+                            const uint32_t from = first + 64u * (uint32_t)((uint64_t)n_batches * s / kWaves);
                             hybrid_walk<K, FAST, false, false, true>(st[0], shortlist, prim, from, from + s_short[s], lane, px.pt, px.cx, px.cy, cd, ca, ci,
                                                                      tail, nullptr, redo_lanes);
                         }
@@ -720,14 +725,15 @@ __device__ __forceinline__ void first_k_put(float *to, uint32_t lane, const floa
 // replayed on the fragments that are not farther than the merged core's last entry -- or, when they are many or the room
 // for those fragments does not do, the first wave walks the whole list again for them.
 template <int K, bool FAST>
-__global__ void __launch_bounds__(64 * kLongWaves) blend_first_k_long_kernel(
+__global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
     uint32_t *__restrict__ spare, uint32_t long_threshold)
 {
-    __shared__ TileStage<64> st[kLongWaves];
+    constexpr int kWaves = long_waves<K>();
+    __shared__ TileStage<64> st[kWaves];
     __shared__ float s_merge[3 * K + 1][64];
-    __shared__ uint32_t s_next, s_whole, s_redo[2], s_listed[kLongWaves];
+    __shared__ uint32_t s_next, s_whole, s_redo[2], s_listed[kWaves];
     __shared__ float s_last_depth[64];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (long_tiles[0] == 0) return;                   // (the ordinary frame)
@@ -738,13 +744,13 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_first_k_long_kernel(
     while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, entry)) {
         const TilePixel px = quadrant_tile_pixel(entry.tile, grid_w, lane, width, height);
         uint32_t share_first, share_last;
-        long_wave_share(entry.first, entry.last, wave, share_first, share_last);
+        long_wave_share(entry.first, entry.last, wave, share_first, share_last, kWaves);
         float ca[K], cd[K];
         uint32_t ci[K];
         first_k_core_init<K>(cd, ca, ci);
         float tie = __FLT_MAX__;
         first_k_walk<K, FAST, false, kTies>(st[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, &tie);
-        for (uint32_t s = 1; s < (uint32_t)kLongWaves; ++s) {
+        for (uint32_t s = 1; s < (uint32_t)kWaves; ++s) {
             __syncthreads();                               // the buffer is free
             if (wave == s) first_k_put<K>(&s_merge[0][0], lane, cd, ca, ci, tie);
             __syncthreads();
@@ -764,7 +770,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_first_k_long_kernel(
                 for (uint32_t other = 0; other < entry.parts; ++other)
                     first_k_merge<K, FAST>(left + (size_t)other * first_k_part_words<K>(), lane, cd, ca, ci, tie);
             }
-            long_wave_share(entry.tile_first, entry.tile_last, wave, share_first, share_last);
+            long_wave_share(entry.tile_first, entry.tile_last, wave, share_first, share_last, kWaves);
             __syncthreads();                               // (the parts are read before the second look overwrites them)
         }
         if (kTies) {
@@ -790,15 +796,15 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_first_k_long_kernel(
                     if (lane == 0) s_listed[wave] = listed;
                     __syncthreads();
                     settled = true;
-                    for (int w = 0; w < kLongWaves; ++w) settled = settled && s_listed[w] != ~0u;
+                    for (int w = 0; w < kWaves; ++w) settled = settled && s_listed[w] != ~0u;
                 }
                 if (threadIdx.x == 0) atomicAdd(const_cast<uint32_t *>(long_tiles) + (settled ? 6 : 7), settled || !looked ? 1u : 0x10001u);
                 if (wave == 0) {
                     first_k_core_init<K>(cd, ca, ci);
                     if (settled) {
-                        for (uint32_t w = 0; w < (uint32_t)kLongWaves; ++w) {
+                        for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
                             uint32_t from, to;
-                            long_wave_share(entry.tile_first, entry.tile_last, w, from, to);
+                            long_wave_share(entry.tile_first, entry.tile_last, w, from, to, kWaves);
                             const uint32_t *candidate = spare + from;
                             for (uint32_t todo = s_listed[w]; todo != 0; --todo, candidate += 4) {
                                 float depth = bits_to_float(candidate[1]), alpha = bits_to_float(candidate[2]);
@@ -1103,7 +1109,7 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
                        f->use_median_depth, f->long_tiles, threshold, f->vals[selector ^ 1] != nullptr, f->tile_order);
     if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
-        hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
+        hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
                            (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->vals[selector ^ 1], threshold);
 }
@@ -1115,7 +1121,7 @@ static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, u
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
                        f->use_median_depth, f->long_tiles, threshold, f->vals[selector ^ 1] != nullptr, f->tile_order);
     if (f->long_tiles)
-        hipLaunchKernelGGL((blend_first_k_long_kernel<K, FAST>), dim3(256), dim3(64 * kLongWaves), 0, (hipStream_t)f->stream, f->ranges,
+        hipLaunchKernelGGL((blend_first_k_long_kernel<K, FAST>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
                            (uint32_t)f->height, grid_w, f->to_chw, f->use_median_depth, f->vals[selector ^ 1], threshold);
 }
