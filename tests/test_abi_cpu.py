@@ -89,6 +89,35 @@ def test_helper_functions():
     assert lib.htgs_tile_order_words(0, 8, 8) == 1 + 264 and lib.htgs_tile_order_words(9, 8, 8) == 0
 
 
+def test_key_widths_of_a_frame_with_depth_order():
+    """GLOBAL_ORDERING with htgs_frame.depth_order: the instance keys hold the tile alone; the Gaussians' depth keys are
+    taken relative to the near plane and are as wide as the far plane makes them.  (No pointer is followed.)"""
+    lib = _native.lib()
+    f = _native.Frame()
+    f.width, f.height, f.n_primitives = 1920, 1080, 1001
+    f.near_plane, f.far_plane = 0.2, 1000.0
+    ref = ctypes.byref(f)
+    for mode in range(4):
+        f.mode = mode
+        f.depth_order = None
+        plain = (lib.htgs_frame_end_bit(ref), lib.htgs_frame_key_bytes(ref), lib.htgs_frame_sort_passes(ref))
+        assert plain == (lib.htgs_end_bit(mode, 1920, 1080), lib.htgs_key_bytes(mode, 1920, 1080), lib.htgs_sort_passes(mode, 1920, 1080))
+        f.depth_order = 256                                  # any address that is not NULL
+        ordered = (lib.htgs_frame_end_bit(ref), lib.htgs_frame_key_bytes(ref), lib.htgs_frame_sort_passes(ref))
+        assert ordered == ((13, 2, 2) if mode == 2 else plain)
+    # bits(1000.0) - bits(0.2) + 1 = 0x062d3334 has 27 bits: three passes of 9-bit digits, the result in the second buffers
+    f.mode = 2
+    n4 = 1004
+    assert lib.htgs_depth_order_result_word(ref) == 3 * n4
+    f.near_plane = 0.0                                       # all 32 bits, four passes of 8: the first buffers
+    assert lib.htgs_depth_order_result_word(ref) == 2 * n4
+    f.near_plane, f.far_plane = 0.5, float("inf")
+    assert lib.htgs_depth_order_result_word(ref) == 2 * n4
+    f.near_plane, f.far_plane = 1.0, 1.5                     # 0x3fc00000 - 0x3f800000 + 1: 23 bits, three passes of 8
+    assert lib.htgs_depth_order_result_word(ref) == 3 * n4
+    assert lib.htgs_depth_order_words(1001) >= 8 * n4 - n4 and lib.htgs_depth_order_words(0) >= 256
+
+
 def test_entry_points_reject_bad_frames_without_touching_the_gpu():
     lib = _native.lib()
     f = _native.Frame()
