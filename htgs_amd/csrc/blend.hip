@@ -208,7 +208,7 @@ __device__ __forceinline__ bool long_tile_take(const uint32_t *long_tiles, const
         __syncthreads();
         if (threadIdx.x == 0) *s_next = atomicAdd(const_cast<uint32_t *>(long_tiles) + 1 + round, 1u);
         __syncthreads();
-        const uint32_t j = *s_next;
+        const uint32_t j = (uint32_t)__builtin_amdgcn_readfirstlane((int)*s_next);     // (the same in every lane: what follows stays in scalar registers)
         if (j >= n_long) {
             if (++round < kLongRounds) continue;
             if (threadIdx.x == 0) {
@@ -420,14 +420,17 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel
     __shared__ uint32_t s_whole;                      // this workgroup finished the last part of its tile
     __shared__ float s_last_depth[64];                // depth of the merged core's last entry
     __shared__ float s_sums[kWaves][kAgainPixels][6], s_tails[64][6];   // tails of the pixels looked at again: per wave, whole
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
     if (long_tiles[0] == 0) return;                   // (the ordinary frame)
     const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
     uint32_t round = 0;
     LongEntry entry;
     while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, entry)) {
-        const uint32_t tile = entry.tile, part = entry.part, parts = entry.parts, tile_first = entry.tile_first, tile_last = entry.tile_last;
-        uint32_t first = entry.first, last = entry.last;
+        // (the same in every lane; said so, they live in scalar registers through the walks that follow)
+        const auto uniform = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+        const uint32_t tile = uniform(entry.tile), part = uniform(entry.part), parts = uniform(entry.parts), tile_first = uniform(entry.tile_first),
+                       tile_last = uniform(entry.tile_last);
+        uint32_t first = uniform(entry.first), last = uniform(entry.last);
         const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
         uint32_t n_batches = (last - first + 63u) / 64u;
         uint32_t seg_first, seg_last;
@@ -735,16 +738,20 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
     __shared__ float s_merge[3 * K + 1][64];
     __shared__ uint32_t s_next, s_whole, s_redo[2], s_listed[kWaves];
     __shared__ float s_last_depth[64];
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
     if (long_tiles[0] == 0) return;                   // (the ordinary frame)
     const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
     constexpr bool kTies = true;                      // (the fast variant too: a tie decides which fragment a pixel shows)
     uint32_t round = 0;
     LongEntry entry;
     while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, entry)) {
-        const TilePixel px = quadrant_tile_pixel(entry.tile, grid_w, lane, width, height);
+        // (the same in every lane; said so, they live in scalar registers through the walks that follow)
+        const auto uniform = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+        const LongEntry e = { uniform(entry.tile), uniform(entry.part), uniform(entry.parts), uniform(entry.tile_first), uniform(entry.tile_last),
+                              uniform(entry.first), uniform(entry.last) };
+        const TilePixel px = quadrant_tile_pixel(e.tile, grid_w, lane, width, height);
         uint32_t share_first, share_last;
-        long_wave_share(entry.first, entry.last, wave, share_first, share_last, kWaves);
+        long_wave_share(e.first, e.last, wave, share_first, share_last, kWaves);
         float ca[K], cd[K];
         uint32_t ci[K];
         first_k_core_init<K>(cd, ca, ci);
@@ -756,21 +763,21 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
             __syncthreads();
             if (wave == 0) first_k_merge<K, FAST>(&s_merge[0][0], lane, cd, ca, ci, tie);
         }
-        if (entry.parts > 1u) {
-            float *const left = reinterpret_cast<float *>(spare + entry.tile_first);
+        if (e.parts > 1u) {
+            float *const left = reinterpret_cast<float *>(spare + e.tile_first);
             if (wave == 0) {
-                first_k_put<K>(left + (size_t)entry.part * first_k_part_words<K>(), lane, cd, ca, ci, tie);
+                first_k_put<K>(left + (size_t)e.part * first_k_part_words<K>(), lane, cd, ca, ci, tie);
                 __threadfence();
             }
-            if (!long_part_done(long_tiles, n_tiles, entry, &s_whole)) continue;
+            if (!long_part_done(long_tiles, n_tiles, e, &s_whole)) continue;
             if (wave == 0) {
                 __threadfence();
                 first_k_core_init<K>(cd, ca, ci);
                 tie = __FLT_MAX__;
-                for (uint32_t other = 0; other < entry.parts; ++other)
+                for (uint32_t other = 0; other < e.parts; ++other)
                     first_k_merge<K, FAST>(left + (size_t)other * first_k_part_words<K>(), lane, cd, ca, ci, tie);
             }
-            long_wave_share(entry.tile_first, entry.tile_last, wave, share_first, share_last, kWaves);
+            long_wave_share(e.tile_first, e.tile_last, wave, share_first, share_last, kWaves);
             __syncthreads();                               // (the parts are read before the second look overwrites them)
         }
         if (kTies) {
@@ -804,7 +811,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
                     if (settled) {
                         for (uint32_t w = 0; w < (uint32_t)kWaves; ++w) {
                             uint32_t from, to;
-                            long_wave_share(entry.tile_first, entry.tile_last, w, from, to, kWaves);
+                            long_wave_share(e.tile_first, e.tile_last, w, from, to, kWaves);
                             const uint32_t *candidate = spare + from;
                             for (uint32_t todo = s_listed[w]; todo != 0; --todo, candidate += 4) {
                                 float depth = bits_to_float(candidate[1]), alpha = bits_to_float(candidate[2]);
@@ -813,7 +820,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
                             }
                         }
                     } else {
-                        first_k_walk<K, FAST, false>(st[0], inst, prim, entry.tile_first, entry.tile_last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
+                        first_k_walk<K, FAST, false>(st[0], inst, prim, e.tile_first, e.tile_last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
                     }
                     if (px.inside && redo) first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
                 }
@@ -907,7 +914,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_oit_long_kernel(
     __shared__ TileStage<64> st[kLongWaves];
     __shared__ float s_sums[kLongWaves][6][64];
     __shared__ uint32_t s_next, s_whole;
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
     if (long_tiles[0] == 0) return;                   // (the ordinary frame)
     const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
     uint32_t round = 0;
