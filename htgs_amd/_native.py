@@ -91,6 +91,7 @@ SYMBOLS = {
     "htgs_frame_end_bit": (ctypes.c_int, [_FRAME_P]),
     "htgs_frame_key_bytes": (ctypes.c_int, [_FRAME_P]),
     "htgs_frame_sort_passes": (ctypes.c_int, [_FRAME_P]),
+    "htgs_frame_depth_sort_passes": (ctypes.c_int, [_FRAME_P]),
     "htgs_depth_order_words": (ctypes.c_size_t, [ctypes.c_int]),
     "htgs_depth_order_result_word": (ctypes.c_size_t, [_FRAME_P]),
     "htgs_scan_tmp_words": (ctypes.c_size_t, [ctypes.c_int]),

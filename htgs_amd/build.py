@@ -1,5 +1,5 @@
-"""Builds ``libhtgs_amd.so`` (gfx950 only) from ``csrc/*.hip`` with hipcc, and the separate measurement-probe library
-``diagnostics/libhtgs_probes.so`` from ``diagnostics/probes.hip``.
+"""Builds ``libhtgs_amd.so`` (gfx950 only) from ``csrc/*.hip`` with hipcc, and the separate counter-calibration library
+``diagnostics/libhtgs_copy.so`` (a plain copy kernel) from ``diagnostics/copy_kernel.hip``.
 
 Both are built in-tree.  ``python -m htgs_amd.build`` rebuilds them.
 """
@@ -14,8 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libhtgs_amd.so")
 OBJ_DIR = os.path.join(HERE, "build")
-PROBES_SRC = os.path.join(HERE, "diagnostics", "probes.hip")
-PROBES_LIB_PATH = os.path.join(HERE, "diagnostics", "libhtgs_probes.so")
+COPY_SRC = os.path.join(HERE, "diagnostics", "copy_kernel.hip")
+COPY_LIB_PATH = os.path.join(HERE, "diagnostics", "libhtgs_copy.so")
 
 # -ffp-contract=off: a fused multiply-add exists only where the sources write __builtin_fmaf, which is what
 #   makes tile counts and accept/reject decisions reproducible (see csrc/common.h).
@@ -78,11 +78,11 @@ def build(verbose: bool = False) -> str:
             print(" ".join(cmd))
         _run(cmd)
 
-    probes_obj = os.path.join(OBJ_DIR, "probes.o")
+    copy_obj = os.path.join(OBJ_DIR, "copy_kernel.o")
     with ThreadPoolExecutor(max_workers=min(8, len(srcs) + 1)) as pool:
-        list(pool.map(compile_one, [*zip(srcs, objs), (PROBES_SRC, probes_obj)]))
+        list(pool.map(compile_one, [*zip(srcs, objs), (COPY_SRC, copy_obj)]))
     link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wno-unused-command-line-argument"]
-    for lib_objs, path in ((objs, LIB_PATH), ([probes_obj], PROBES_LIB_PATH)):
+    for lib_objs, path in ((objs, LIB_PATH), ([copy_obj], COPY_LIB_PATH)):
         tmp = path + ".tmp"
         _run([*link, *lib_objs, "-o", tmp])
         os.replace(tmp, path)

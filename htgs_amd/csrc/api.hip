@@ -128,6 +128,8 @@ extern "C" int htgs_forward_front(const htgs_frame *f)
 {
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_front: null frame");
     if (!f->clamp_info && f->n_primitives > 0) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_front: clamp_info is required for training");
+    // (the per-Gaussian backward finds a Gaussian's gradient rows through offsets[] in index order)
+    if (frame_depth_ordered(f)) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_front: depth_order is for the inference entry points");
     htgs_frame t = *f;
     t.scale_modifier = 1.0f;   // the training preprocess has no scale modifier (R/include/hybrid_blend/kernels/forward.cuh:10-76)
     int rc = htgs_preprocess(&t);
@@ -138,6 +140,7 @@ extern "C" int htgs_forward_front(const htgs_frame *f)
 extern "C" int htgs_forward_back(const htgs_frame *f, int *selector)
 {
     if (!f || !selector) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_back: null argument");
+    if (frame_depth_ordered(f)) return fail(HTGS_ERR_ARGUMENT, "htgs_forward_back: depth_order is for the inference entry points");
     int rc = htgs_create_instances(f);
     if (rc != HTGS_OK) return rc;
     rc = htgs_sort_instances(f, selector);

@@ -951,6 +951,7 @@ extern "C" int htgs_blend_backward(const htgs_frame *f, int selector)
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0 || f->n_primitives < 0)
         return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: bad argument");
+    if (frame_depth_ordered(f)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: depth_order is for the inference entry points");
     if (f->prim_floats != HTGS_PRIM_FLOATS_TRAIN) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: the training kernels read records of HTGS_PRIM_FLOATS_TRAIN floats (prim_floats)");
     if (f->n_primitives == 0 || f->n_instances == 0) return HTGS_OK;
     if (f->n_primitives >= (1 << 27)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_backward: 2^27 Gaussians or more");
@@ -1009,9 +1010,9 @@ extern "C" int htgs_preprocess_backward(const htgs_frame *f)
     if (f->n_primitives < 0 || f->total_sh_bases < 0) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: bad sizes");
     if (f->n_primitives == 0) return HTGS_OK;
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
-    if (!f->offsets || (f->n_instances > 0 && !f->grad_rows)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: null pointer");
     // (a Gaussian's gradient rows are found through offsets[], which must be in index order)
     if (frame_depth_ordered(f)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: depth_order is for the inference entry points");
+    if (!f->offsets || (f->n_instances > 0 && !f->grad_rows)) return fail(HTGS_ERR_ARGUMENT, "htgs_preprocess_backward: null pointer");
     if (!f->positions || !f->scales || !f->rotations || !f->n_touched || !f->clamp_info || !f->M || !f->VPM ||
         !f->cam_position || !f->grad_positions || !f->grad_scales || !f->grad_rotations || !f->grad_opacities || !f->grad_sh_0 ||
         (f->total_sh_bases > 0 && (!f->sh_rest || !f->grad_sh_rest)))

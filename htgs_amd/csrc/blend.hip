@@ -154,9 +154,8 @@ __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim
 // caller provided that list, and a second launch of workgroups of kLongWaves waves takes those: one wave walks one tile at some
 // 200 ns per instance once it has a SIMD to itself, so a single list of 300 000 instances would otherwise hold the
 // launch for 70 ms.
-// long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = parts granted beyond one per
-// tile -- all zeroed with the ranges and again by the last workgroup of the second launch; [6], [7] = tiles with
-// pixels settled by a second look / walked again in one piece (upper half: of these, after a second look that ran out of
+// long_tiles[0] = entries on the list, [1..3] = work counters, [4] = workgroups done, [5] = unused -- all zeroed with the
+// ranges and again by the last workgroup of the second launch; [6], [7] = tiles with pixels settled by a second look / walked again in one piece (upper half: of these, after a second look that ran out of
 // room) since the ranges were made (for the tests); then 2 n_tiles words for the entries (tile | part << 20 |
 // (parts - 1) << 25: a tile is on the list once per part, and the parts beyond the first of all tiles together are held
 // to n_tiles, so the list cannot overflow) and n_tiles words that count a tile's finished parts.
@@ -170,23 +169,24 @@ constexpr uint32_t kLongListDefault = 8192;
 // What a workgroup leaves of its part of a list, in 64-lane rows: HYBRID's core, tail and the depth of a tie.
 template <int K> constexpr uint32_t long_part_words() { return (3u * K + 7u) * 64u; }
 // The parts a list of this length is walked in by separate workgroups (1: by one).  A part is at least four times the
-// threshold long, and long enough that what the parts leave behind (part_words each) fits into the list's own stretch of
-// the spare value buffer.
-__device__ __forceinline__ uint32_t long_parts(uint32_t length, uint32_t long_threshold, uint32_t part_words)
+// threshold long, long enough that what the parts leave behind (part_words each) fits into the list's own stretch of
+// the spare value buffer, and at least as long as the frame's average list (part_floor = instances / tiles, rounded
+// up): the parts beyond the first of all tiles together then cannot exceed the number of tiles, which is what the list
+// of entries has room for, and how a list is split is a function of its length and of the frame alone -- no budget
+// shared between workgroups, nothing that depends on the order in which they run.
+__device__ __forceinline__ uint32_t long_parts(uint32_t length, uint32_t long_threshold, uint32_t part_words, uint32_t part_floor)
 {
-    const uint32_t least = 4u * long_threshold > part_words ? 4u * long_threshold : part_words;
+    uint32_t least = 4u * long_threshold > part_words ? 4u * long_threshold : part_words;
+    least = least > part_floor ? least : part_floor;
     const uint32_t parts = length / least;
     return parts < 1u ? 1u : parts > kLongParts ? kLongParts : parts;
 }
-// (one lane of the tile's wave) enters the tile
+// (one lane of the tile's wave) enters the tile; part_floor = 0: in one part
 __device__ __forceinline__ void long_tile_enter(uint32_t *__restrict__ long_tiles, uint32_t tile, uint32_t n_tiles, uint32_t length,
-                                                uint32_t long_threshold, uint32_t part_words, bool in_parts)
+                                                uint32_t long_threshold, uint32_t part_words, uint32_t part_floor)
 {
-    uint32_t parts = in_parts ? long_parts(length, long_threshold, part_words) : 1u;
-    if (parts > 1u) {
-        if (atomicAdd(long_tiles + 5, parts - 1u) + parts - 1u > n_tiles) parts = 1u;
-        else long_tiles[kLongHeader + 2u * n_tiles + tile] = 0u;
-    }
+    const uint32_t parts = part_floor != 0u ? long_parts(length, long_threshold, part_words, part_floor) : 1u;
+    if (parts > 1u) long_tiles[kLongHeader + 2u * n_tiles + tile] = 0u;
     const uint32_t at = kLongHeader + atomicAdd(long_tiles, parts);
     for (uint32_t part = 0; part < parts; ++part) long_tiles[at + part] = tile | part << 20 | (parts - 1u) << 25;
 }
@@ -257,14 +257,14 @@ template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
-    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, int in_parts, const uint32_t *__restrict__ tile_order)
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
     __shared__ TileStage<64> st;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, long_part_words<K>(), in_parts);
+        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, long_part_words<K>(), part_floor);
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -671,14 +671,14 @@ template <int K, bool FAST>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
-    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, int in_parts, const uint32_t *__restrict__ tile_order)
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
     __shared__ TileStage<64> st;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, first_k_part_words<K>(), in_parts);
+        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, first_k_part_words<K>(), part_floor);
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -884,14 +884,14 @@ template <bool FAST>
 __global__ void __launch_bounds__(64) blend_oit_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw,
-    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, int in_parts, const uint32_t *__restrict__ tile_order)
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
     __shared__ TileStage<64> st;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, kOitPartWords, in_parts);
+        if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, kOitPartWords, part_floor);
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -1108,13 +1108,21 @@ __global__ void __launch_bounds__(256) check_tile_cull_16_kernel(
     }
 }
 
+// the least length of a part of a long list (0: lists are not split, there is no spare value buffer to leave the parts' results in)
+static uint32_t long_part_floor(const htgs_frame *f, int selector, uint32_t n_tiles)
+{
+    if (f->vals[selector ^ 1] == nullptr) return 0u;
+    const uint64_t floor = (f->n_instances + n_tiles - 1) / n_tiles;
+    return floor < 1u ? 1u : (uint32_t)floor;
+}
+
 template <int K, bool FAST>
 static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
     const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth, f->long_tiles, threshold, f->vals[selector ^ 1] != nullptr, f->tile_order);
+                       f->use_median_depth, f->long_tiles, threshold, long_part_floor(f, selector, n_tiles), f->tile_order);
     if (f->long_tiles)      // (one workgroup per compute unit; they find an empty list on ordinary frames)
         hipLaunchKernelGGL((blend_hybrid_long_kernel<K, FAST>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
@@ -1126,7 +1134,7 @@ static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, u
     const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     hipLaunchKernelGGL((blend_first_k_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
                        (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth, f->long_tiles, threshold, f->vals[selector ^ 1] != nullptr, f->tile_order);
+                       f->use_median_depth, f->long_tiles, threshold, long_part_floor(f, selector, n_tiles), f->tile_order);
     if (f->long_tiles)
         hipLaunchKernelGGL((blend_first_k_long_kernel<K, FAST>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0, (hipStream_t)f->stream, f->ranges,
                            f->vals[selector], (const float4 *)f->prim, f->long_tiles, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width,
@@ -1169,7 +1177,7 @@ static void launch_blend(const htgs_frame *f, int selector, uint32_t grid_w, uin
             const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
             hipLaunchKernelGGL(blend_oit_kernel<FAST>, dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[selector], (const float4 *)f->prim,
                                f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw, f->long_tiles, threshold,
-                               f->vals[selector ^ 1] != nullptr, f->tile_order);
+                               long_part_floor(f, selector, n_tiles), f->tile_order);
             if (f->long_tiles)
                 hipLaunchKernelGGL(blend_oit_long_kernel<FAST>, dim3(256), dim3(64 * kLongWaves), 0, s, f->ranges, f->vals[selector],
                                    (const float4 *)f->prim, f->long_tiles, f->image, depth, (uint32_t)f->width, (uint32_t)f->height, grid_w,

@@ -341,6 +341,7 @@ extern "C" int htgs_blend_forward(const htgs_frame *f, int selector)
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: null frame");
     if (f->mode < 0 || f->mode > 3) return fail(HTGS_ERR_MODE, "unsupported rasterizer mode");
     if (selector < 0 || selector > 1 || f->width <= 0 || f->height <= 0) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: bad argument");
+    if (frame_depth_ordered(f)) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: depth_order is for the inference entry points");
     if (f->prim_floats != HTGS_PRIM_FLOATS_TRAIN) return fail(HTGS_ERR_ARGUMENT, "htgs_blend_forward: the training kernels read records of HTGS_PRIM_FLOATS_TRAIN floats (prim_floats)");
     const bool needs_core = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K;
     const bool needs_tail = f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_OIT_BLEND;

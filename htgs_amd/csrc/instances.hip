@@ -366,6 +366,11 @@ extern "C" size_t htgs_depth_order_result_word(const htgs_frame *f)
     return (2 + (size_t)(depth_key_range(f).passes & 1)) * n4;
 }
 
+extern "C" int htgs_frame_depth_sort_passes(const htgs_frame *f)
+{
+    return f && frame_depth_ordered(f) ? depth_key_range(f).passes : 0;
+}
+
 extern "C" int htgs_scan_offsets(const htgs_frame *f)
 {
     if (!f) return fail(HTGS_ERR_ARGUMENT, "htgs_scan_offsets: null frame");

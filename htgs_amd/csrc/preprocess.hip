@@ -154,7 +154,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     if (in_range) n_touched[i] = touched;
     // htgs_frame.depth_order: the pairs that sort the Gaussians by depth (depth_key_range() in common.h)
     if (depth_keys != nullptr && in_range) {
-        depth_keys[i] = touched != 0 ? float_to_bits(z) - depth_base : depth_culled;
+        // (a depth that is not a number passes the cull above, as in the reference, where its bit pattern sorts behind every
+        // valid depth; here its key is held below `culled`, so it is neither dropped nor sorted by bits that the sort ignores)
+        const uint32_t key = float_to_bits(z) - depth_base;
+        depth_keys[i] = touched != 0 ? (key < depth_culled - 1u ? key : depth_culled - 1u) : depth_culled;
         depth_vals[i] = (uint32_t)i;
     }
     s_visible[threadIdx.x] = visible;

@@ -1,17 +1,15 @@
-"""ctypes binding of the measurement probes (``include/htgs_probes.h``, ``libhtgs_probes.so``): a plain copy kernel
-that calibrates the HBM traffic counters and micro-kernels that time single vector instructions.  Only the benchmark
-uses them; the rasterizer library does not contain them."""
+"""Measurement aids of the benchmark, outside the rasterizer library: ``counters.py`` turns rocprofv3 counter runs into
+the HBM-traffic record ``bench.py`` reports, and ``libhtgs_copy.so`` (``copy_kernel.hip``) is the plain copy of known
+size that calibrates those counters (``bench.py --calibrate``)."""
 from __future__ import annotations
 
 import ctypes
 import os
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libhtgs_probes.so")
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libhtgs_copy.so")
 
 SYMBOLS = {
-    "htgs_probe_issue_cost_name": (ctypes.c_char_p, [ctypes.c_int]),
-    "htgs_probe_issue_cost_launch": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
-    "htgs_probe_copy_bytes": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "htgs_diag_copy_bytes": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
 }
 
 _lib = None

@@ -35,24 +35,17 @@ def test_library_exports_every_declared_symbol():
     _native.lib()
 
 
-def test_probe_library_is_separate_and_exports_its_header():
-    """The measurement probes live in their own library and header, not in the drop-in boundary."""
+def test_calibration_copy_kernel_is_a_library_of_its_own():
+    """The plain copy that calibrates the traffic counters is not part of the drop-in boundary: its own library, no
+    declaration in include/, no symbol in the product."""
     from htgs_amd import diagnostics
-    names = declared_functions(os.path.join(ROOT, "include", "htgs_probes.h"))
-    assert sorted(diagnostics.SYMBOLS) == names and len(names) == 3
+    assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["htgs_amd.h"]
     product = ctypes.CDLL(_native.LIB_PATH)
-    for name in names:
+    for name in diagnostics.SYMBOLS:
         assert hasattr(diagnostics.lib(), name)
         assert not hasattr(product, name)
-    lib = diagnostics.lib()
-    probes = []
-    while lib.htgs_probe_issue_cost_name(len(probes)) is not None:
-        probes.append(lib.htgs_probe_issue_cost_name(len(probes)).decode())
-    assert probes[0] == "v_fma_f32" and "v_mov_b32" in probes and "v_swap_b32" in probes and len(set(probes)) == len(probes)
-    assert lib.htgs_probe_issue_cost_name(-1) is None
-    assert lib.htgs_probe_issue_cost_launch(len(probes), None, 1, 1, None) == 2        # no such instruction (and no buffer)
-    assert lib.htgs_probe_issue_cost_launch(0, None, 1, 1, None) == 2
-    assert lib.htgs_probe_copy_bytes(None, None, 16, None) == 2
+    assert diagnostics.lib().htgs_diag_copy_bytes(None, None, 16, None) == 2
+    assert diagnostics.lib().htgs_diag_copy_bytes(1, 1, 8, None) == 2          # not a multiple of 16
 
 
 def test_frame_struct_layout_matches_the_header(tmp_path):
@@ -135,6 +128,23 @@ def test_entry_points_reject_bad_frames_without_touching_the_gpu():
     assert lib.htgs_preprocess(None) == 2
     f.n_primitives = -1
     assert lib.htgs_preprocess(ctypes.byref(f)) == 2
+
+
+def test_training_entry_points_refuse_a_frame_with_depth_order():
+    """htgs_frame.depth_order belongs to the inference entry points (the per-Gaussian backward finds a Gaussian's gradient
+    rows through offsets[] in index order): every training entry point refuses such a frame before it launches anything."""
+    lib = _native.lib()
+    f = _native.Frame()
+    f.mode, f.width, f.height, f.n_primitives, f.n_instances = 2, 64, 64, 10, 10
+    f.prim_floats = _native.PRIM_FLOATS_TRAIN
+    f.clamp_info = 256                                       # any address that is not NULL
+    f.depth_order = 256
+    ref, sel = ctypes.byref(f), ctypes.c_int(0)
+    for status in (lib.htgs_forward_front(ref), lib.htgs_forward_back(ref, ctypes.byref(sel)), lib.htgs_blend_forward(ref, 0),
+                   lib.htgs_blend_backward(ref, 0), lib.htgs_preprocess_backward(ref), lib.htgs_backward(ref, 0)):
+        assert status == 2 and b"depth_order is for the inference entry points" in lib.htgs_last_error()
+    f.mode = 0                                               # depth_order is ignored outside GLOBAL_ORDERING
+    assert lib.htgs_blend_forward(ref, 0) == 2 and b"null pointer" in lib.htgs_last_error()
 
 
 def test_record_size_is_checked_by_every_entry_point_that_reads_records():

@@ -107,3 +107,31 @@ def test_depth_order_small_counts(cuda, n):
     np.testing.assert_array_equal(got["sorted_vals"], ref["sorted_vals"])
     np.testing.assert_array_equal(got["ranges"], ref["ranges"])
     assert np.abs(got["image"] - ref["image"]).max() <= 1e-4
+
+
+def test_depth_that_is_not_a_number_sorts_behind_the_valid_ones(cuda):
+    """A camera row with a NaN makes a Gaussian's depth NaN while its screen rectangle stays finite; the depth cull
+    (``z < near || z > far``, R/include/kernel_utils.cuh:89-90) lets it through.  With the reference's tile | depth keys
+    its bit pattern sorts behind every valid depth, equal patterns in index order; the frame with depth_order must list
+    the same instances in the same order (its key is held just below the key of a culled Gaussian).  Also one NaN
+    position, which both paths cull."""
+    import dataclasses
+    scene = make_scene(0, 3000)
+    pos = scene.positions.clone()
+    pos[17] = float("nan")
+    scene = dataclasses.replace(scene, positions=pos)
+    for nan_row in (False, True):
+        print(f"case nan_row={nan_row}", flush=True)
+        sc = scene
+        if nan_row:
+            M = scene.M.clone()
+            M[2, 3] = float("nan")
+            sc = dataclasses.replace(scene, M=M)
+        got = gpu_stages(sc.to(cuda), 2, 4, order_gaussians=True)
+        keyed = gpu_stages(sc.to(cuda), 2, 4, order_gaussians=False)
+        assert got["n_instances"] == keyed["n_instances"] > 0
+        np.testing.assert_array_equal(got["n_touched"], keyed["n_touched"])
+        assert got["n_touched"][17] == 0
+        np.testing.assert_array_equal(got["sorted_vals"], keyed["sorted_vals"])
+        np.testing.assert_array_equal(got["ranges"], keyed["ranges"])
+        assert np.array_equal(got["image"], keyed["image"], equal_nan=True)

@@ -93,23 +93,6 @@ def test_refined_reciprocal_equals_division_on_the_whole_guarded_range(cuda):
     assert wrong == 0
 
 
-def test_issue_cost_micro_kernels_run(cuda):
-    """The measurement aid behind ``bench.py --issue-cost`` (separate probe library): every micro-kernel launches and
-    fills its output."""
-    from htgs_amd import diagnostics
-    lib = diagnostics.lib()
-    marker = 0x7FC12345                                   # a NaN pattern no kernel produces
-    out = torch.empty(4 * 256, dtype=torch.int32, device=cuda)
-    i = 0
-    while lib.htgs_probe_issue_cost_name(i) is not None:
-        out.fill_(marker)
-        assert lib.htgs_probe_issue_cost_launch(i, out.data_ptr(), 4, 2, torch.cuda.current_stream().cuda_stream) == 0
-        torch.cuda.synchronize()
-        assert not bool((out == marker).any()), lib.htgs_probe_issue_cost_name(i)
-        i += 1
-    assert i >= 10
-
-
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 @pytest.mark.parametrize("config,n", [(0, 5000), (1, 60_000)])
 def test_fast_rasterize_against_the_oracle(cuda, config, n, mode):
