@@ -63,41 +63,42 @@ __device__ __forceinline__ void hybrid_core_init(float (&cd)[K], float (&ca)[K],
 // PIXELS: only the pixels of the lanes in pixel_lanes are wanted; instances that do not reach one of them are left out
 // (the other lanes' cores and tails come out incomplete).
 template <int K, bool FAST, bool SOLO, bool TIES = false, bool PIXELS = false>
-__device__ __forceinline__ void hybrid_walk(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
-                                            uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K], float (&ca)[K],
-                                            float (&ci)[K], HybridTail &tail, float *tie = nullptr, uint64_t pixel_lanes = 0)
+__device__ __forceinline__ void hybrid_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+                                            uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K],
+                                            float (&ca)[K], float (&ci)[K], HybridTail &tail, float *tie = nullptr, uint64_t pixel_lanes = 0)
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    constexpr int N = kStageSlots;
+    stage_dummy_init(st, lane);
     for (uint32_t base = first; base < last; base += 64) {
         if (SOLO) __syncthreads(); else wave_lds_sync();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, PIXELS ? kCullPixels : kCullAlpha, true>(st, prim, inst, base + lane, last, lane,
-                                                                                                                 cx, cy, pixel_lanes));
+        const uint32_t bits = tile_stage_load<MODE, N, true, PIXELS ? kCullPixels : kCullAlpha, true>(st, prim, inst, base + lane, last, lane + 1, cx, cy,
+                                                                                                      pixel_lanes);
+        const uint32_t n_turns = quadrant_lists_build(ql, bits, lane, st);
         if (SOLO) __syncthreads(); else wave_lds_sync();
-        {
-            // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
-            const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-                // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
-                // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
-                // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
-                TileFrag f;
-                const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-                f.den_rcp = frag_rcp<FAST>(f.den);
-                const float4 col = stage_row<64, 5>(addr);
-                if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach)) return;
-                float depth = tile_frag_depth<64>(addr, pt, f);
-                float p3 = f.alpha;
-                tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
-                tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
-                tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
-                if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
-                    float pi = col.w;
-                    core_exchange_walk<K>(depth, p3, pi, cd, ca, ci);
-                    if (TIES && p3 > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
-                }
-                hybrid_tail_add<FAST>(tail, depth, p3);
-            });
-        }
+        // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
+        quadrant_list_walk(ql, n_turns, lane, [&](uint32_t addr) {
+            // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
+            // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
+            // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
+            TileFrag f;
+            const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+            f.den_rcp = frag_rcp<FAST>(f.den);
+            const float4 col = stage_row<N, 5>(addr);
+            if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach)) return;
+            float depth = tile_frag_depth<N>(addr, pt, f);
+            float p3 = f.alpha;
+            tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
+            tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
+            tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
+            if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
+                float pi = col.w;
+                if constexpr (FAST && !TIES) core_quick_walk<K>(depth, p3, pi, cd, ca, ci);
+                else core_exchange_walk<K>(depth, p3, pi, cd, ca, ci);
+                if (TIES && p3 > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
+            }
+            hybrid_tail_add<FAST>(tail, depth, p3);
+        });
     }
 }
 
@@ -259,7 +260,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
     uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
@@ -272,7 +274,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     hybrid_tail_init(tail);
     float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
     hybrid_core_init<K>(cd, ca, ci);
-    hybrid_walk<K, FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
+    hybrid_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
     if (!px.inside) return;
     hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
 }
@@ -412,7 +414,8 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel
     uint32_t *__restrict__ shortlist, uint32_t long_threshold)
 {
     constexpr int kWaves = long_waves<K>();
-    __shared__ TileStage<64> st[kWaves];
+    __shared__ TileStageQ st[kWaves];
+    __shared__ QuadrantLists ql[kWaves];
     __shared__ float s_merge[3 * K + 7][64];          // one wave's core, tail and least depth of a tie, lane-minor
     __shared__ uint32_t s_next;
     __shared__ uint32_t s_redo[2];                    // the pixels (lanes) to walk again
@@ -441,7 +444,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel
         float cd[K], ca[K], ci[K];
         hybrid_core_init<K>(cd, ca, ci);
         float tie = __FLT_MAX__;                        // least depth at which two fragments of equal depth met at the end of a core
-        hybrid_walk<K, FAST, false, kTies>(st[wave], inst, prim, seg_first, seg_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, &tie);
+        hybrid_walk<K, FAST, false, kTies>(st[wave], ql[wave], inst, prim, seg_first, seg_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, &tie);
         for (uint32_t s = 1; s < (uint32_t)kWaves; ++s) {
             __syncthreads();                               // the buffer is free
             if (wave == s) {
@@ -513,7 +516,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel
                     }
                     __syncthreads();
                     const uint32_t listed = pixels_again<HTGS_MODE_HYBRID_BLEND, false>(
-                        st[wave], inst, prim, seg_first, seg_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, s_sums[wave], shortlist + seg_first,
+                        reinterpret_cast<TileStage<64> &>(st[wave]), inst, prim, seg_first, seg_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, s_sums[wave], shortlist + seg_first,
                         (seg_last - seg_first) / 4u, [&](const uint32_t (&pixel)[kAgainPixels]) {
                             __syncthreads();
                             if (wave == 0 && lane < (uint32_t)kAgainPixels) {      // the waves' sums of a pixel, in list order
@@ -567,7 +570,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel
                     uint32_t kept = 0;
                     for (uint32_t base = seg_first; base < seg_last; base += 64) {
                         const uint32_t fetch = base + lane;
-                        const bool reaches = tile_stage_load<HTGS_MODE_HYBRID_BLEND, 64, true, kCullPixels, true>(st[wave], prim, inst, fetch, seg_last, lane,
+                        const bool reaches = tile_stage_load<HTGS_MODE_HYBRID_BLEND, 64, true, kCullPixels, true>(reinterpret_cast<TileStage<64> &>(st[wave]), prim, inst, fetch, seg_last, lane,
                                                                                                                px.cx, px.cy, redo_lanes) != 0;
                         const uint64_t keep = __ballot(reaches);
                         if (reaches) shortlist[seg_first + kept + (uint32_t)__popcll(keep & ((1ull << lane) - 1ull))] = inst[fetch];
@@ -584,11 +587,11 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_hybrid_long_kernel
                     if (shortlist != nullptr) {
                         for (uint32_t s = 0; s < (uint32_t)kWaves; ++s) {
                             const uint32_t from = first + 64u * (uint32_t)((uint64_t)n_batches * s / kWaves);
-                            hybrid_walk<K, FAST, false, false, true>(st[0], shortlist, prim, from, from + s_short[s], lane, px.pt, px.cx, px.cy, cd, ca, ci,
+                            hybrid_walk<K, FAST, false, false, true>(st[0], ql[0], shortlist, prim, from, from + s_short[s], lane, px.pt, px.cx, px.cy, cd, ca, ci,
                                                                      tail, nullptr, redo_lanes);
                         }
                     } else {
-                        hybrid_walk<K, FAST, false, false, true>(st[0], inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, nullptr, redo_lanes);
+                        hybrid_walk<K, FAST, false, false, true>(st[0], ql[0], inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail, nullptr, redo_lanes);
                     }
                     if (px.inside && redo) hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
                 }

@@ -418,6 +418,64 @@ __device__ __forceinline__ void quadrant_walk(QuadrantHits &hits, uint32_t stage
         if (addr != kNoHit) turn(addr + stage_base);
     }
 }
+// Quadrant lists: the same walk with the scalar bit scans taken out of the loop.  After a batch is staged, the slots that
+// reach quadrant q are written, in list order, to a short list in LDS (their LDS addresses), padded up to the length of
+// the longest of the four lists with the address of a slot that no fragment passes (entry 0 of every row of a stage with
+// kStageSlots entries per row: a cut-off quadratic above its |d|^2, opacity 0).  A turn of the loop is then one LDS read
+// per lane -- entry `turn` of its quadrant's list -- instead of eight scalar and nine vector instructions that pick the
+// next set bit of four masks and hand it to the quadrant's lanes, and a quadrant that has run out of hits evaluates the
+// dummy slot, which fails the walk's own test, instead of being masked off: one exec level less.
+constexpr int kStageSlots = 65;
+typedef TileStage<kStageSlots> TileStageQ;
+struct QuadrantLists {
+    uint32_t a[4][64];
+    uint32_t beyond;            // (the walk reads one entry ahead)
+};
+typedef __attribute__((address_space(3))) const uint32_t lds_u32;
+// (one lane) the slot that fails every test: |m|^2 / cut-off = 1 everywhere, |d|^2 = 1/2, opacity 0
+__device__ __forceinline__ void stage_dummy_init(TileStageQ &st, uint32_t lane)
+{
+    if (lane == 0) {
+        st.q[0][0] = make_float4(1.0f, 0.0f, 0.0f, 0.0f);
+        st.q[1][0] = make_float4(0.0f, 0.0f, 0.5f, 0.0f);
+        st.q[2][0] = st.q[3][0] = st.q[4][0] = st.q[5][0] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+}
+// LDS address of the q[0] entry of staged slot `slot` (0 .. 63)
+__device__ __forceinline__ uint32_t stage_slot_address(const TileStageQ &st, uint32_t slot) { return stage_address(st) + 16u * (slot + 1u); }
+// Called by the wave after tile_stage_load (bits: the lane's slot's quadrant bits): writes the four lists and returns the
+// number of turns, the length of the longest (wave-uniform).  Every lane writes one entry per list: a slot that reaches
+// the quadrant its address at the number of such slots before it, the others the dummy address behind all of them.
+__device__ __forceinline__ uint32_t quadrant_lists_build(QuadrantLists &ql, uint32_t bits, uint32_t lane, const TileStageQ &st)
+{
+    const uint32_t dummy = stage_address(st), mine = stage_slot_address(st, lane);
+    uint32_t most = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const bool hit = (bits >> q) & 1u;
+        const uint64_t h = __ballot(hit);
+        const uint32_t count = (uint32_t)__popcll(h);
+        const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(h >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)h, 0u));
+        ql.a[q][hit ? below : count + (lane - below)] = hit ? mine : dummy;
+        most = most > count ? most : count;
+    }
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)most);
+}
+// turn(addr) is called n_turns times, by all lanes: addr = the LDS address of the q[0] entry of the slot the lane's quadrant
+// (lanes 16 q .. 16 q + 15) evaluates in this turn.
+template <typename Turn>
+__device__ __forceinline__ void quadrant_list_walk(const QuadrantLists &ql, uint32_t n_turns, uint32_t lane, Turn &&turn)
+{
+    // (the entry of the next turn is read while this turn's slot is evaluated: one LDS round trip per turn, not two)
+    uint32_t p = (uint32_t)(uintptr_t)(lds_u32 *)&ql.a[lane >> 4][0];
+    uint32_t addr = *(lds_u32 *)(uintptr_t)p;
+    for (uint32_t t = 0; t < n_turns; ++t) {
+        asm volatile("v_add_u32 %0, 4, %0" : "+v"(p));
+        const uint32_t next = *(lds_u32 *)(uintptr_t)p;
+        turn(addr);
+        addr = next;
+    }
+}
 // The per-pixel records of the training pass are kept tile by tile: the 64 pixels of an 8x8 tile, row-major, are
 // contiguous, so a tile's workgroup writes and reads whole lines whatever order the tiles are taken in.  A record plane
 // has 64 entries per tile of the launch (gridDim.x tiles, the pixels beyond the image included).
@@ -532,6 +590,51 @@ __device__ __forceinline__ void core_exchange_walk(float &depth, float &alpha, I
         } else {
 #pragma unroll
             for (int i = g0; i < g0 + kInsertGroup && i < K; ++i) exchange_step(depth, alpha, index, cd[i], ca[i], ci[i], all);
+        }
+    }
+}
+
+// The image-only fast path inserts by shifting instead: the entry that moves down the core alternates between two register
+// triples, so that a slot costs two moves per register (slot -> the other triple, this triple -> slot) instead of an
+// exchange through a scratch register.  Both triples start out as the fragment; a lane joins at the first slot that is
+// not nearer than its fragment and from there on moves every slot down by one (<=: once it has joined, the entry it carries
+// is the previous slot's, which is never deeper than the next slot's).  This is the stable insertion, not the reference's
+// exchange walk: where two stored fragments have exactly the same depth the two differ in which of them ends up in front,
+// which the fast path does not promise to reproduce.  On return (depth, alpha, index) is what was pushed out.
+#define HTGS_QUICK_SLOT(n, R, W)                                                                                         \
+    "v_cmpx_le_f32 vcc, %[d" #R "], %[D" #n "]\n\t"                                                                     \
+    "v_mov_b32 %[d" #W "], %[D" #n "]\n\tv_mov_b32 %[D" #n "], %[d" #R "]\n\t"                                         \
+    "v_mov_b32 %[a" #W "], %[A" #n "]\n\tv_mov_b32 %[A" #n "], %[a" #R "]\n\t"                                         \
+    "v_mov_b32 %[x" #W "], %[I" #n "]\n\tv_mov_b32 %[I" #n "], %[x" #R "]\n\t"                                         \
+    "s_mov_b64 exec, %[all]\n\t"
+template <typename IndexT>
+__device__ __forceinline__ void quick_step4(float &d0, float &a0, IndexT &x0, float &d1, float &a1, IndexT &x1, float &D0, float &A0, IndexT &I0,
+                                            float &D1, float &A1, IndexT &I1, float &D2, float &A2, IndexT &I2, float &D3, float &A3, IndexT &I3)
+{
+    static_assert(sizeof(IndexT) == 4, "one register");
+    uint64_t all;
+    asm volatile("s_mov_b64 %[all], exec\n\t" HTGS_QUICK_SLOT(0, 0, 1) HTGS_QUICK_SLOT(1, 1, 0) HTGS_QUICK_SLOT(2, 0, 1) HTGS_QUICK_SLOT(3, 1, 0)
+                 : [d0] "+v"(d0), [a0] "+v"(a0), [x0] "+v"(x0), [d1] "+v"(d1), [a1] "+v"(a1), [x1] "+v"(x1), [D0] "+v"(D0), [A0] "+v"(A0),
+                   [I0] "+v"(I0), [D1] "+v"(D1), [A1] "+v"(A1), [I1] "+v"(I1), [D2] "+v"(D2), [A2] "+v"(A2), [I2] "+v"(I2), [D3] "+v"(D3),
+                   [A3] "+v"(A3), [I3] "+v"(I3), [all] "=&s"(all)
+                 :
+                 : "vcc");
+}
+#undef HTGS_QUICK_SLOT
+template <int K, typename IndexT>
+__device__ __forceinline__ void core_quick_walk(float &depth, float &alpha, IndexT &index, float (&cd)[K], float (&ca)[K], IndexT (&ci)[K])
+{
+    if constexpr (K % 4 != 0) core_exchange_walk<K>(depth, alpha, index, cd, ca, ci);
+    else {
+        float d1 = depth, a1 = alpha;
+        IndexT x1 = index;
+#pragma unroll
+        for (int g0 = 0; g0 < K; g0 += 4) {
+            // (a group that no lane's entry is nearer than the end of: nothing moves there; a group is an even number of
+            // slots, so the entry is back in the first triple at every group's start)
+            if (K > 4 && !__any(depth < cd[g0 + 3])) continue;
+            quick_step4(depth, alpha, index, d1, a1, x1, cd[g0], ca[g0], ci[g0], cd[g0 + 1], ca[g0 + 1], ci[g0 + 1], cd[g0 + 2], ca[g0 + 2], ci[g0 + 2],
+                        cd[g0 + 3], ca[g0 + 3], ci[g0 + 3]);
         }
     }
 }

