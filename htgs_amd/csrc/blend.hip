@@ -69,37 +69,28 @@ __device__ __forceinline__ void hybrid_walk(TileStageQ &st, QuadrantLists &ql, c
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
     constexpr int N = kStageSlots;
-    stage_dummy_init(st, lane);
-    for (uint32_t base = first; base < last; base += 64) {
-        if (SOLO) __syncthreads(); else wave_lds_sync();
-        const uint32_t bits = tile_stage_load<MODE, N, true, PIXELS ? kCullPixels : kCullAlpha, true>(st, prim, inst, base + lane, last, lane + 1, cx, cy,
-                                                                                                      pixel_lanes);
-        const uint32_t n_turns = quadrant_lists_build(ql, bits, lane, st);
-        if (SOLO) __syncthreads(); else wave_lds_sync();
-        // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
-        quadrant_list_walk(ql, n_turns, lane, [&](uint32_t addr) {
-            // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
-            // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
-            // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
-            TileFrag f;
-            const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
-            f.den_rcp = frag_rcp<FAST>(f.den);
-            const float4 col = stage_row<N, 5>(addr);
-            if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach)) return;
-            float depth = tile_frag_depth<N>(addr, pt, f);
-            float p3 = f.alpha;
-            tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
-            tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
-            tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
-            if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
-                float pi = col.w;
-                if constexpr (FAST && !TIES) core_quick_walk<K>(depth, p3, pi, cd, ca, ci);
-                else core_exchange_walk<K>(depth, p3, pi, cd, ca, ci);
-                if (TIES && p3 > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
-            }
-            hybrid_tail_add<FAST>(tail, depth, p3);
-        });
-    }
+    tile_list_walk<MODE, true, PIXELS ? kCullPixels : kCullAlpha, SOLO>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
+        // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
+        // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+        f.den_rcp = frag_rcp<FAST>(f.den);
+        const float4 col = stage_row<N, 5>(addr);
+        if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach)) return;
+        float depth = tile_frag_depth<N>(addr, pt, f);
+        float p3 = f.alpha;
+        tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
+        tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
+        tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
+        if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
+            float pi = col.w;
+            if constexpr (FAST && !TIES) core_quick_walk<K>(depth, p3, pi, cd, ca, ci);
+            else core_exchange_walk<K>(depth, p3, pi, cd, ca, ci);
+            if (TIES && p3 > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
+        }
+        hybrid_tail_add<FAST>(tail, depth, p3);
+    }, pixel_lanes);
 }
 
 // core + tail -> pixel (R/include/hybrid_blend/kernels/inference.cuh:172-213)
@@ -618,31 +609,24 @@ __device__ __forceinline__ void first_k_core_init(float (&cd)[K], float (&ca)[K]
 // walks of blend_first_k_long_kernel): `tie` receives the least depth at which an entry was pushed out of the core that is
 // exactly as deep as the entry that is now last.
 template <int K, bool FAST, bool SOLO, bool TIES = false>
-__device__ __forceinline__ void first_k_walk(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
-                                             uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K], float (&ca)[K],
-                                             uint32_t (&ci)[K], float *tie = nullptr)
+__device__ __forceinline__ void first_k_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+                                             uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K],
+                                             float (&ca)[K], uint32_t (&ci)[K], float *tie = nullptr)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
-    for (uint32_t base = first; base < last; base += 64) {
-        if (SOLO) __syncthreads(); else wave_lds_sync();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        if (SOLO) __syncthreads(); else wave_lds_sync();
-        {
-            const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-                TileFrag f;
-                const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-                f.den_rcp = frag_rcp<FAST>(f.den);
-                float depth = tile_frag_depth<64>(addr, pt, f);
-                if (!(in_reach && depth < cd[K - 1])) return;          // depth test before the exponential (:151)
-                if (!tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f)) return;
-                float alpha = f.alpha;
-                uint32_t idx = stage_index<64>(addr);
-                core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
-                if (TIES && alpha > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
-            });
-        }
-    }
+    constexpr int N = kStageSlots;
+    tile_list_walk<MODE, true, kCullAlpha, SOLO>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+        f.den_rcp = frag_rcp<FAST>(f.den);
+        float depth = tile_frag_depth<N>(addr, pt, f);
+        if (!(in_reach && depth < cd[K - 1])) return;          // depth test before the exponential (:151)
+        if (!tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f)) return;
+        float alpha = f.alpha;
+        uint32_t idx = stage_index<N>(addr);
+        core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
+        if (TIES && alpha > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
+    });
 }
 template <int K>
 __device__ __forceinline__ void first_k_composite(const float4 *__restrict__ prim, const float (&cd)[K], const float (&ca)[K], const uint32_t (&ci)[K],
@@ -676,7 +660,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
     uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
@@ -688,7 +673,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     float ca[K], cd[K];
     uint32_t ci[K];
     first_k_core_init<K>(cd, ca, ci);
-    first_k_walk<K, FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
+    first_k_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
     if (!px.inside) return;
     first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
 }
@@ -737,7 +722,8 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
     uint32_t *__restrict__ spare, uint32_t long_threshold)
 {
     constexpr int kWaves = long_waves<K>();
-    __shared__ TileStage<64> st[kWaves];
+    __shared__ TileStageQ st[kWaves];
+    __shared__ QuadrantLists ql[kWaves];
     __shared__ float s_merge[3 * K + 1][64];
     __shared__ uint32_t s_next, s_whole, s_redo[2], s_listed[kWaves];
     __shared__ float s_last_depth[64];
@@ -759,7 +745,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
         uint32_t ci[K];
         first_k_core_init<K>(cd, ca, ci);
         float tie = __FLT_MAX__;
-        first_k_walk<K, FAST, false, kTies>(st[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, &tie);
+        first_k_walk<K, FAST, false, kTies>(st[wave], ql[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, cd, ca, ci, &tie);
         for (uint32_t s = 1; s < (uint32_t)kWaves; ++s) {
             __syncthreads();                               // the buffer is free
             if (wave == s) first_k_put<K>(&s_merge[0][0], lane, cd, ca, ci, tie);
@@ -801,7 +787,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
                 if (spare != nullptr && __popcll(redo_lanes) <= kAgainMost) {
                     looked = true;
                     const uint32_t listed = pixels_again<HTGS_MODE_ALPHA_BLEND_FIRST_K, FAST>(
-                        st[wave], inst, prim, share_first, share_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, nullptr, spare + share_first,
+                        reinterpret_cast<TileStage<64> &>(st[wave]), inst, prim, share_first, share_last, lane, px.cx, px.cy, redo_lanes, s_last_depth, nullptr, spare + share_first,
                         (share_last - share_first) / 4u, [](const uint32_t (&)[kAgainPixels]) {});
                     if (lane == 0) s_listed[wave] = listed;
                     __syncthreads();
@@ -823,7 +809,7 @@ __global__ void __launch_bounds__(64 * long_waves<K>()) blend_first_k_long_kerne
                             }
                         }
                     } else {
-                        first_k_walk<K, FAST, false>(st[0], inst, prim, e.tile_first, e.tile_last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
+                        first_k_walk<K, FAST, false>(st[0], ql[0], inst, prim, e.tile_first, e.tile_last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
                     }
                     if (px.inside && redo) first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
                 }
@@ -843,32 +829,25 @@ struct OitSums {
 };
 // The walk over instances [first, last) of a tile's list by one wave (SOLO: the wave is the whole workgroup).
 template <bool FAST, bool SOLO>
-__device__ __forceinline__ void oit_walk(TileStage<64> &st, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first, uint32_t last,
-                                         uint32_t lane, const PixelTerms &pt, float cx, float cy, OitSums &sum)
+__device__ __forceinline__ void oit_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, uint32_t first,
+                                         uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, OitSums &sum)
 {
     constexpr int MODE = HTGS_MODE_OIT_BLEND;
-    for (uint32_t base = first; base < last; base += 64) {
-        if (SOLO) __syncthreads(); else wave_lds_sync();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        if (SOLO) __syncthreads(); else wave_lds_sync();
-        {
-            const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-            quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-                TileFrag f;
-                const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-                f.den_rcp = frag_rcp<FAST>(f.den);
-                const float4 col = stage_row<64, 5>(addr);
-                if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<64>(addr), f) && in_reach)) return;
-                const float depth = FAST ? 0.0f : tile_frag_depth<64>(addr, pt, f);
-                sum.a0 = __builtin_fmaf(f.alpha, col.x, sum.a0);
-                sum.a1 = __builtin_fmaf(f.alpha, col.y, sum.a1);
-                sum.a2 = __builtin_fmaf(f.alpha, col.z, sum.a2);
-                if (!FAST) sum.a3 = __builtin_fmaf(f.alpha, depth, sum.a3);
-                sum.alpha += f.alpha;
-                sum.T *= 1.0f - f.alpha;
-            });
-        }
-    }
+    constexpr int N = kStageSlots;
+    tile_list_walk<MODE, true, kCullAlpha, SOLO>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+        f.den_rcp = frag_rcp<FAST>(f.den);
+        const float4 col = stage_row<N, 5>(addr);
+        if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach)) return;
+        const float depth = FAST ? 0.0f : tile_frag_depth<N>(addr, pt, f);
+        sum.a0 = __builtin_fmaf(f.alpha, col.x, sum.a0);
+        sum.a1 = __builtin_fmaf(f.alpha, col.y, sum.a1);
+        sum.a2 = __builtin_fmaf(f.alpha, col.z, sum.a2);
+        if (!FAST) sum.a3 = __builtin_fmaf(f.alpha, depth, sum.a3);
+        sum.alpha += f.alpha;
+        sum.T *= 1.0f - f.alpha;
+    });
 }
 __device__ __forceinline__ void oit_composite(const OitSums &sum, float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height,
                                               uint32_t x, uint32_t y, int chw)
@@ -889,7 +868,8 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw,
     uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
@@ -899,7 +879,7 @@ __global__ void __launch_bounds__(64) blend_oit_kernel(
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
     OitSums sum = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f };
-    oit_walk<FAST, true>(st, inst, prim, first, last, lane, px.pt, px.cx, px.cy, sum);
+    oit_walk<FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, sum);
     if (!px.inside) return;
     oit_composite(sum, image, depths, width, height, px.x, px.y, chw);
 }
@@ -914,7 +894,8 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_oit_long_kernel(
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw,
     uint32_t *__restrict__ left, uint32_t long_threshold)
 {
-    __shared__ TileStage<64> st[kLongWaves];
+    __shared__ TileStageQ st[kLongWaves];
+    __shared__ QuadrantLists ql[kLongWaves];
     __shared__ float s_sums[kLongWaves][6][64];
     __shared__ uint32_t s_next, s_whole;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -927,7 +908,7 @@ __global__ void __launch_bounds__(64 * kLongWaves) blend_oit_long_kernel(
         uint32_t share_first, share_last;
         long_wave_share(entry.first, entry.last, wave, share_first, share_last);
         OitSums sum = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 1.0f };
-        oit_walk<FAST, false>(st[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, sum);
+        oit_walk<FAST, false>(st[wave], ql[wave], inst, prim, share_first, share_last, lane, px.pt, px.cx, px.cy, sum);
         s_sums[wave][0][lane] = sum.a0; s_sums[wave][1][lane] = sum.a1; s_sums[wave][2][lane] = sum.a2; s_sums[wave][3][lane] = sum.a3;
         s_sums[wave][4][lane] = sum.alpha; s_sums[wave][5][lane] = sum.T;
         __syncthreads();

@@ -476,6 +476,23 @@ __device__ __forceinline__ void quadrant_list_walk(const QuadrantLists &ql, uint
         addr = next;
     }
 }
+// The walk over instances [first, last) of a tile's list (whole batches of 64 from `first` on) by one wave, lanes =
+// pixels by quadrants: every batch is staged (tile_stage_load with the CULL asked for), its quadrant lists are built and
+// turn(addr) is called for every turn.  SOLO: the wave is the whole workgroup (its barriers are the workgroup's).
+template <int MODE, bool DEPTH, int CULL, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4, typename Turn>
+__device__ __forceinline__ void tile_list_walk(TileStageQ &st, QuadrantLists &ql, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
+                                               uint32_t first, uint32_t last, uint32_t lane, float cx, float cy, Turn &&turn, uint64_t pixel_lanes = 0)
+{
+    stage_dummy_init(st, lane);
+    for (uint32_t base = first; base < last; base += 64) {
+        if (SOLO) __syncthreads(); else wave_lds_sync();
+        const uint32_t bits = tile_stage_load<MODE, kStageSlots, DEPTH, CULL, true, REC4>(st, prim, inst, base + lane, last, lane + 1, cx, cy, pixel_lanes);
+        const uint32_t n_turns = quadrant_lists_build(ql, bits, lane, st);
+        if (SOLO) __syncthreads(); else wave_lds_sync();
+        // lanes outside the image run along (their results are never stored): the loop stays wave-uniform
+        quadrant_list_walk(ql, n_turns, lane, turn);
+    }
+}
 // The per-pixel records of the training pass are kept tile by tile: the 64 pixels of an 8x8 tile, row-major, are
 // contiguous, so a tile's workgroup writes and reads whole lines whatever order the tiles are taken in.  A record plane
 // has 64 entries per tile of the launch (gridDim.x tiles, the pixels beyond the image included).

@@ -23,7 +23,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -44,30 +45,24 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
-    for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
-        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-            TileFrag f;
-            const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-            f.den_rcp = rcp_exact(f.den);
-            const float4 col = stage_row<64, 5>(addr);
-            if (!(tile_frag_alpha<MODE>(stage_opacity<64>(addr), f) && in_reach)) return;
-            float depth = tile_frag_depth<64>(addr, pt, f);
-            float p3 = f.alpha;
-            tail0 = __builtin_fmaf(p3, col.x, tail0);
-            tail1 = __builtin_fmaf(p3, col.y, tail1);
-            tail2 = __builtin_fmaf(p3, col.z, tail2);
-            if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
-                uint32_t idx = stage_index<64>(addr);
-                core_exchange_walk<K>(depth, p3, idx, cd, c3, ci);
-            }
-            tail3 += p3;
-            T_tail *= 1.0f - p3;
-        });
-    }
+    tile_list_walk<MODE, true, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<kStageSlots>(addr, pt, f);
+        f.den_rcp = rcp_exact(f.den);
+        const float4 col = stage_row<kStageSlots, 5>(addr);
+        if (!(tile_frag_alpha<MODE>(stage_opacity<kStageSlots>(addr), f) && in_reach)) return;
+        float depth = tile_frag_depth<kStageSlots>(addr, pt, f);
+        float p3 = f.alpha;
+        tail0 = __builtin_fmaf(p3, col.x, tail0);
+        tail1 = __builtin_fmaf(p3, col.y, tail1);
+        tail2 = __builtin_fmaf(p3, col.z, tail2);
+        if (depth < cd[K - 1] && f.alpha >= kMinAlphaCore) {
+            uint32_t idx = stage_index<kStageSlots>(addr);
+            core_exchange_walk<K>(depth, p3, idx, cd, c3, ci);
+        }
+        tail3 += p3;
+        T_tail *= 1.0f - p3;
+    });
     if (!inside) return;
 
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
@@ -141,7 +136,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -159,23 +155,17 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
-    for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, true, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
-        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-            TileFrag f;
-            const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-            f.den_rcp = rcp_exact(f.den);
-            float depth = tile_frag_depth<64>(addr, pt, f);
-            if (!(in_reach && depth < cd[K - 1])) return;
-            if (!tile_frag_alpha<MODE>(stage_opacity<64>(addr), f)) return;
-            float alpha = f.alpha;
-            uint32_t idx = stage_index<64>(addr);
-            core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
-        });
-    }
+    tile_list_walk<MODE, true, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<kStageSlots>(addr, pt, f);
+        f.den_rcp = rcp_exact(f.den);
+        float depth = tile_frag_depth<kStageSlots>(addr, pt, f);
+        if (!(in_reach && depth < cd[K - 1])) return;
+        if (!tile_frag_alpha<MODE>(stage_opacity<kStageSlots>(addr), f)) return;
+        float alpha = f.alpha;
+        uint32_t idx = stage_index<kStageSlots>(addr);
+        core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
+    });
     if (!inside) return;
 
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
@@ -227,7 +217,8 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     float *__restrict__ image, float *__restrict__ tail_info, uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order)
 {
     constexpr int MODE = HTGS_MODE_OIT_BLEND;
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -238,24 +229,18 @@ __global__ void __launch_bounds__(64) blend_oit_forward_kernel(
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, alpha_sum = 0.0f, T = 1.0f;
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
-    for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
-        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-            TileFrag f;
-            const bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-            f.den_rcp = rcp_exact(f.den);
-            const float4 col = stage_row<64, 5>(addr);
-            if (!(tile_frag_alpha<MODE>(stage_opacity<64>(addr), f) && in_reach)) return;
-            a0 = __builtin_fmaf(f.alpha, col.x, a0);
-            a1 = __builtin_fmaf(f.alpha, col.y, a1);
-            a2 = __builtin_fmaf(f.alpha, col.z, a2);
-            alpha_sum += f.alpha;
-            T *= 1.0f - f.alpha;
-        });
-    }
+    tile_list_walk<MODE, false, kCullAlpha, true, HTGS_PRIM_FLOATS_TRAIN / 4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<kStageSlots>(addr, pt, f);
+        f.den_rcp = rcp_exact(f.den);
+        const float4 col = stage_row<kStageSlots, 5>(addr);
+        if (!(tile_frag_alpha<MODE>(stage_opacity<kStageSlots>(addr), f) && in_reach)) return;
+        a0 = __builtin_fmaf(f.alpha, col.x, a0);
+        a1 = __builtin_fmaf(f.alpha, col.y, a1);
+        a2 = __builtin_fmaf(f.alpha, col.z, a2);
+        alpha_sum += f.alpha;
+        T *= 1.0f - f.alpha;
+    });
     if (!inside) return;
     const size_t pix = (size_t)width * y + x, np = (size_t)width * height;
     const size_t rp = record_pixel(tile, x, y), rnp = record_plane();

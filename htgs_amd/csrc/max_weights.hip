@@ -24,7 +24,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     constexpr bool kCore = MODE != HTGS_MODE_OIT_BLEND;
     constexpr bool kTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = kCore ? K : 1;
-    __shared__ TileStage<64> st;
+    __shared__ TileStageQ st;
+    __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
@@ -42,30 +43,24 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     }
 
     const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
-    for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, kCore, kCullAlpha, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
-        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-            TileFrag f;
-            bool in_reach = tile_frag_cutoff<64>(addr, pt, f);
-            f.den_rcp = rcp_exact(f.den);
-            float depth = 0.0f;
-            if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
-                depth = tile_frag_depth<64>(addr, pt, f);
-                in_reach = in_reach && depth < cd[KS - 1];
-            }
-            if (!(tile_frag_alpha<MODE>(stage_opacity<64>(addr), f) && in_reach)) return;
-            float alpha = f.alpha;
-            if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth<64>(addr, pt, f);
-            if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
-                uint32_t idx = stage_index<64>(addr);
-                core_exchange_walk<KS>(depth, alpha, idx, cd, ca, ci);
-            }
-            if (kTail) { alpha_sum += alpha; T_tail *= 1.0f - alpha; }
-        });
-    }
+    tile_list_walk<MODE, kCore, kCullAlpha, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        bool in_reach = tile_frag_cutoff<kStageSlots>(addr, pt, f);
+        f.den_rcp = rcp_exact(f.den);
+        float depth = 0.0f;
+        if (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K) {
+            depth = tile_frag_depth<kStageSlots>(addr, pt, f);
+            in_reach = in_reach && depth < cd[KS - 1];
+        }
+        if (!(tile_frag_alpha<MODE>(stage_opacity<kStageSlots>(addr), f) && in_reach)) return;
+        float alpha = f.alpha;
+        if (MODE == HTGS_MODE_HYBRID_BLEND) depth = tile_frag_depth<kStageSlots>(addr, pt, f);
+        if (kCore && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || (depth < cd[KS - 1] && alpha >= kMinAlphaCore))) {
+            uint32_t idx = stage_index<kStageSlots>(addr);
+            core_exchange_walk<KS>(depth, alpha, idx, cd, ca, ci);
+        }
+        if (kTail) { alpha_sum += alpha; T_tail *= 1.0f - alpha; }
+    });
     float T_core = 1.0f;
     if (kCore && inside) {
 #pragma unroll
@@ -83,20 +78,14 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     if (!__any(active)) return;
     // second walk over the tile's list: alpha * tail weight for every fragment that passes the cut-off (no alpha
     // threshold here, R/include/hybrid_blend/kernels/update_max_weights.cuh:197-204)
-    for (uint32_t base = first; base < last; base += 64) {
-        __syncthreads();
-        QuadrantHits hits = quadrant_ballot(tile_stage_load<MODE, 64, false, kCullCutoff, true>(st, prim, inst, base + lane, last, lane, cx, cy));
-        __syncthreads();
-        const uint32_t stage_base = __builtin_amdgcn_readfirstlane(stage_address(st));
-        quadrant_walk(hits, stage_base, [&](uint32_t addr) {
-            TileFrag f;
-            if (!active || !tile_frag_cutoff<64>(addr, pt, f)) return;
-            const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * rcp_exact(f.den));
-            const float a = stage_opacity<64>(addr) * G;
-            const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
-            if (!(w < weight_threshold)) raise_max(max_weights, stage_index<64>(addr), w);
-        });
-    }
+    tile_list_walk<MODE, false, kCullCutoff, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        if (!active || !tile_frag_cutoff<kStageSlots>(addr, pt, f)) return;
+        const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * rcp_exact(f.den));
+        const float a = stage_opacity<kStageSlots>(addr) * G;
+        const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
+        if (!(w < weight_threshold)) raise_max(max_weights, stage_index<kStageSlots>(addr), w);
+    });
 }
 
 __global__ void __launch_bounds__(256) max_weights_global_kernel(
