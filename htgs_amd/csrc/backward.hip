@@ -16,7 +16,7 @@
 // its row-major position in the Gaussian's tile rectangle, both read from the Gaussian's 128-byte training record, which
 // the gather brings in anyway -- so the rows of a Gaussian are contiguous and the
 // per-Gaussian kernel adds them up in a fixed order: no atomics, no zero-fill, bit-reproducible gradients.
-#include "blend_common.h"
+#include "blend_long.h"
 
 namespace htgs {
 
@@ -339,34 +339,44 @@ __device__ __forceinline__ void backward_batch(const BackwardBatch &b, uint8_t *
 // densification row (HELPER) is a sum of absolute values per fragment and cannot go through the moments: it takes
 // the fourth components of the fragment's dL/dVPMT rows, which need m and the two plane normals at the pixel.
 // ---------------------------------------------------------------------------------------------
+// LDS of a workgroup of the kernels below
+template <int K, bool HELPER>
+struct BackwardTileTerms {
+    static constexpr int KS = K > 0 ? K : 1;
+    // per-pixel terms, pixels in the order and with the skew of pixel_slot (one 16-byte word per quadrant)
+    __attribute__((aligned(16))) uint32_t s_idx[64 * KS + 16];      // [pixel][slot]: Gaussian << 5 | slot
+    float4 s_core[64 * KS + 4];   // (weight * g, dC/dalpha . g)
+    float4 s_tail[64 + 4];        // (full weight * g, common)
+    float s_tail_a[64 + 4];
+    float s_pos[HELPER ? 64 : 1][6];   // per pixel: (dL/dpx.w, dL/dpy.w) of a fragment -> its dL/dposition
+    uint8_t s_pairs[kBackwardWaves][256];   // per wave: the batch's (staging lane << 2 | quadrant) pairs, in list order
+};
+// The workgroup's work on instances [first, last) of a tile's list: the tile's per-pixel terms go into LDS, then the four
+// waves take the batches of 64 in turn.  Every instance writes a gradient row of its own, so a list may be cut anywhere
+// and its pieces given to different workgroups.  (All threads; the caller synchronises before the LDS is used again.)
 template <int K, int MODE, bool HELPER>
-__global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_waves_per_eu(HELPER ? 3 : 5))) blend_tail_backward_moments_kernel(
-    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+__device__ __forceinline__ void backward_tile(BackwardTileTerms<K, HELPER> &lds, uint32_t tile, uint32_t first, uint32_t last, uint32_t n_tiles,
+    const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
     const float *__restrict__ grad_image, const float *__restrict__ VPM, float4 *__restrict__ grad_rows, float *__restrict__ helper_rows,
-    uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order)
+    uint32_t width, uint32_t height, uint32_t grid_w)
 {
     constexpr bool kHasTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int KS = K > 0 ? K : 1;
-    // per-pixel terms, pixels in the order and with the skew of pixel_slot (one 16-byte word per quadrant)
-    __shared__ __attribute__((aligned(16))) uint32_t s_idx[64 * KS + 16];      // [pixel][slot]: Gaussian << 5 | slot
-    __shared__ float4 s_core[64 * KS + 4];   // (weight * g, dC/dalpha . g)
-    __shared__ float4 s_tail[64 + 4];        // (full weight * g, common)
-    __shared__ float s_tail_a[64 + 4];
-    __shared__ float s_pos[HELPER ? 64 : 1][6];   // per pixel: (dL/dpx.w, dL/dpy.w) of a fragment -> its dL/dposition
-    __shared__ uint8_t s_pairs[kBackwardWaves][256];   // per wave: the batch's (staging lane << 2 | quadrant) pairs, in list order
-    const uint32_t tile = block_tile(tile_order);
+    uint32_t *const s_idx = lds.s_idx;
+    float4 *const s_core = lds.s_core, *const s_tail = lds.s_tail;
+    float *const s_tail_a = lds.s_tail_a;
+    float (*const s_pos)[6] = lds.s_pos;
+    uint8_t (*const s_pairs)[256] = lds.s_pairs;
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t x0 = (tile % grid_w) * 8, y0 = (tile / grid_w) * 8;
     const size_t np = (size_t)width * height;
-    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
-    if (first == last) return;               // nothing was drawn into this tile (whole workgroup)
     {
         // per-pixel terms into LDS: lane = pixel; the tail's by the first wave, the K core slots shared out over the four
         const uint32_t x = x0 + (lane & 7), y = y0 + (lane >> 3);
         const bool inside = x < width && y < height;
         const size_t pix = inside ? (size_t)width * y + x : 0;
-        const size_t rp = record_pixel(tile, x, y), rnp = record_plane();     // (the forward pass's per-pixel records: tile by tile)
+        const size_t rp = record_pixel(tile, x, y), rnp = (size_t)n_tiles * 64u;     // (the forward pass's per-pixel records: tile by tile)
         const uint32_t ps = pixel_slot_of_lane(lane), pq = pixel_quadrant_of_lane(lane);
         float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f;
         if (inside) { g0 = grad_image[pix]; g1 = grad_image[np + pix]; g2 = grad_image[2 * np + pix]; }
@@ -420,6 +430,46 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
                                   tile, x0, y0, width, height, grid_w, cx, cy, lane, base, last };
         backward_batch<K, MODE, HELPER>(b, s_pairs[wave]);
     }
+}
+
+template <int K, int MODE, bool HELPER>
+__global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_waves_per_eu(HELPER ? 3 : 5))) blend_tail_backward_moments_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
+    const float *__restrict__ grad_image, const float *__restrict__ VPM, float4 *__restrict__ grad_rows, float *__restrict__ helper_rows,
+    uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *__restrict__ tile_order, uint32_t *__restrict__ long_tiles, uint32_t long_threshold,
+    uint32_t part_floor)
+{
+    __shared__ BackwardTileTerms<K, HELPER> lds;
+    const uint32_t tile = block_tile(tile_order);
+    const uint32_t first = ranges[2 * tile], last = ranges[2 * tile + 1];
+    if (first == last) return;               // nothing was drawn into this tile (whole workgroup)
+    // a very long list is left to blend_tail_backward_long_kernel, in parts (no part leaves anything behind for the others)
+    if (long_tiles != nullptr && last - first > long_threshold) {
+        if (threadIdx.x == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, 0u, part_floor);
+        return;
+    }
+    backward_tile<K, MODE, HELPER>(lds, tile, first, last, gridDim.x, inst, prim, core_idx, core_info, tail_info, grad_image, VPM, grad_rows, helper_rows, width,
+                                   height, grid_w);
+}
+
+// The tiles with very long lists (and their parts): the workgroups take them off the list the kernel above made, longest first.
+template <int K, int MODE, bool HELPER>
+__global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_waves_per_eu(HELPER ? 3 : 5))) blend_tail_backward_long_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+    const uint32_t *__restrict__ core_idx, const float4 *__restrict__ core_info, const float *__restrict__ tail_info,
+    const float *__restrict__ grad_image, const float *__restrict__ VPM, float4 *__restrict__ grad_rows, float *__restrict__ helper_rows,
+    uint32_t width, uint32_t height, uint32_t grid_w, const uint32_t *long_tiles, uint32_t long_threshold)
+{
+    __shared__ BackwardTileTerms<K, HELPER> lds;
+    __shared__ uint32_t s_next;
+    if (long_tiles[0] == 0) return;                   // (the ordinary frame)
+    const uint32_t n_tiles = grid_w * ((height + 7u) / 8u);
+    uint32_t round = 0;
+    LongEntry e;
+    while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, e))
+        backward_tile<K, MODE, HELPER>(lds, e.tile, e.first, e.last, n_tiles, inst, prim, core_idx, core_info, tail_info, grad_image, VPM, grad_rows, helper_rows,
+                                       width, height, grid_w);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -927,18 +977,27 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
     }
 }
 
+template <int K, int MODE, bool HELPER>
+static void launch_tail_backward_kernels(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
+{
+    const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
+    // the least length of a part of a long list: the frame's average list, so that the parts of all tiles fit the list of entries
+    const uint64_t floor = (f->n_instances + n_tiles - 1) / n_tiles;
+    hipLaunchKernelGGL((blend_tail_backward_moments_kernel<K, MODE, HELPER>), dim3(n_tiles), dim3(64 * kBackwardWaves), 0, (hipStream_t)f->stream,
+                       f->ranges, f->vals[sel], (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image,
+                       f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order, f->long_tiles, threshold,
+                       floor < 1u ? 1u : (uint32_t)floor);
+    if (f->long_tiles)      // (four workgroups per compute unit; they find an empty list on ordinary frames)
+        hipLaunchKernelGGL((blend_tail_backward_long_kernel<K, MODE, HELPER>), dim3(1024), dim3(64 * kBackwardWaves), 0, (hipStream_t)f->stream,
+                           f->ranges, f->vals[sel], (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image,
+                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->long_tiles, threshold);
+}
 template <int K, int MODE>
 static void launch_tail_backward(const htgs_frame *f, int sel, uint32_t grid_w, uint32_t n_tiles)
 {
     // the third densification row needs |dL/dposition|_1 fragment by fragment
-    if (f->dens_helper)
-        hipLaunchKernelGGL((blend_tail_backward_moments_kernel<K, MODE, true>), dim3(n_tiles), dim3(64 * kBackwardWaves), 0, (hipStream_t)f->stream,
-                           f->ranges, f->vals[sel], (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image,
-                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
-    else
-        hipLaunchKernelGGL((blend_tail_backward_moments_kernel<K, MODE, false>), dim3(n_tiles), dim3(64 * kBackwardWaves), 0, (hipStream_t)f->stream,
-                           f->ranges, f->vals[sel], (const float4 *)f->prim, f->core_idx, (const float4 *)f->core_info, f->tail_info, f->grad_image,
-                           f->VPM, (float4 *)f->grad_rows, f->dens_helper, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->tile_order);
+    if (f->dens_helper) launch_tail_backward_kernels<K, MODE, true>(f, sel, grid_w, n_tiles);
+    else launch_tail_backward_kernels<K, MODE, false>(f, sel, grid_w, n_tiles);
 }
 
 }  // namespace htgs

@@ -166,9 +166,9 @@ class FrameBuffers:
         self.scan_tmp = self._scratch("scan_tmp", self.lib.htgs_scan_tmp_words(n), torch.int32)
         self.n_instances_dev = self._scratch("n_instances_dev", 1, torch.int32)    # written by the scan
         self.ranges = self._scratch("ranges", 2 * self.n_tiles, torch.int32)[:2 * self.n_tiles].view(self.n_tiles, 2)
-        # inference in the modes that walk all of a list (every one but GLOBAL_ORDERING): the list of tiles with very long
-        # instance lists, which several waves walk together
-        self.long_tiles = self._scratch("long_tiles", 3 * self.n_tiles + 8, torch.int32) if mode != 2 and not train else None
+        # the modes that walk all of a list (every one but GLOBAL_ORDERING): the list of tiles with very long instance
+        # lists, which several waves or workgroups walk together (inference, training forward and backward, max weights)
+        self.long_tiles = self._scratch("long_tiles", 3 * self.n_tiles + 8, torch.int32) if mode != 2 else None
         # the tiles in the order the blend kernels take them (longest lists first), written with the ranges
         self.tile_order = (self._scratch("tile_order", self.lib.htgs_tile_order_words(mode, self.width, self.height), torch.int32)
                            if order_tiles else None)
