@@ -115,7 +115,7 @@ def oracle_frame(oracle, scene_cpu, mode, K):
                         scene_cpu.active_sh_bases, scene_cpu.width, scene_cpu.height, scene_cpu.near_plane, scene_cpu.far_plane)
 
 
-def bench_training(scene_cpu, scene, config, n_override, mode, K, steps, warmup, densification_rows=0, cpu_baseline=True):
+def bench_training(scene_cpu, scene, config, n_override, mode, K, steps, warmup, densification_rows=0, cpu_baseline=True, long_list_threshold=0):
     """One step = diff_rasterize forward + backward w.r.t. all six Gaussian tensors from a fixed upstream
     gradient ~N(0,1).  Reported as milliseconds per step with the forward / backward split."""
     import torch
@@ -127,12 +127,12 @@ def bench_training(scene_cpu, scene, config, n_override, mode, K, steps, warmup,
     info = torch.zeros((densification_rows, scene.positions.shape[0]), device=gauss[0].device) if densification_rows else None
 
     def step():
-        fb = FrameBuffers(*gauss, settings, True, False, train=True)
+        fb = FrameBuffers(*gauss, settings, True, False, train=True, long_list_threshold=long_list_threshold)
         fb.run_forward()
         return fb, fb.run_backward(grad_image, info, info is not None)
 
     ms_per_step = timed_steps(step, steps, warmup)
-    fb = FrameBuffers(*gauss, settings, True, False, train=True)
+    fb = FrameBuffers(*gauss, settings, True, False, train=True, long_list_threshold=long_list_threshold)
     fb.run_forward()
     fwd_blend = statistics.median(event_ms(fb.blend_forward, 10))
     bwd = statistics.median(event_ms(lambda: fb.run_backward(grad_image, info, info is not None), 10))
@@ -347,6 +347,16 @@ def bench_all_configs(dev, headline_scene):
     scene = scene_cpu.to(dev)
     for mode in (0, 1, 2, 3):
         out[f"cfg4/{MODE_NAMES[mode]}/train"] = compact(bench_training(scene_cpu, scene, 4, None, mode, 16, EXTRA_STEPS, EXTRA_WARMUP, cpu_baseline=False))
+    del scene
+    release()
+    # a training step on the stress scene's distributions (1 M Gaussians): tiles with very long lists are shared between
+    # waves and workgroups; beside it the same step with one wave (workgroup) per tile, as the reference walks them
+    scene_cpu = make_scene(3, 1_000_000)
+    scene = scene_cpu.to(dev)
+    entry = compact(bench_training(scene_cpu, scene, 3, 1_000_000, 0, 16, 10, 3, cpu_baseline=False))
+    single = bench_training(scene_cpu, scene, 3, 1_000_000, 0, 16, 5, 2, cpu_baseline=False, long_list_threshold=2 ** 31 - 1)
+    entry["one_wave_per_tile"] = {"ms_per_step": single["ms_per_step"], "stages": single["stages"]}
+    out["cfg3-n1000000/HYBRID_BLEND/train"] = entry
     del scene
     release()
     return out

@@ -75,6 +75,7 @@ class Frame(ctypes.Structure):
         ("densification_info", ctypes.c_void_p),
         ("densification_rows", ctypes.c_int32),
         ("use_distance_scaling", ctypes.c_int32),
+        ("pixel_scratch", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
     ]
 

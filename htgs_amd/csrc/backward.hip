@@ -446,7 +446,8 @@ __global__ void __launch_bounds__(64 * kBackwardWaves) __attribute__((amdgpu_wav
     if (first == last) return;               // nothing was drawn into this tile (whole workgroup)
     // a very long list is left to blend_tail_backward_long_kernel, in parts (no part leaves anything behind for the others)
     if (long_tiles != nullptr && last - first > long_threshold) {
-        if (threadIdx.x == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold, 0u, part_floor);
+        // (parts of one threshold's length: nothing is merged afterwards, so the finer the parts the better they spread)
+        if (threadIdx.x == 0) long_tile_enter(long_tiles, tile, gridDim.x, last - first, long_threshold / 4u, 0u, part_floor);
         return;
     }
     backward_tile<K, MODE, HELPER>(lds, tile, first, last, gridDim.x, inst, prim, core_idx, core_info, tail_info, grad_image, VPM, grad_rows, helper_rows, width,

@@ -4,7 +4,7 @@
 // R/include/alpha_blend_global_ordering/kernels/update_max_weights.cuh:59-131 and
 // R/include/oit_blend/kernels/update_max_weights.cuh:58-165.  The maximum is taken on the bit patterns of the
 // (non-negative) weights with integer atomicMax, which makes the result independent of the order of arrival.
-#include "blend_common.h"
+#include "blend_long.h"
 
 namespace htgs {
 
@@ -19,7 +19,8 @@ __device__ __forceinline__ void raise_max(uint32_t *__restrict__ max_weights, ui
 template <int K, int MODE>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) max_weights_tile_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold, const uint32_t *__restrict__ tile_order)
+    uint32_t *__restrict__ max_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold, const uint32_t *__restrict__ tile_order,
+    uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor)
 {
     constexpr bool kCore = MODE != HTGS_MODE_OIT_BLEND;
     constexpr bool kTail = MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K;
@@ -28,6 +29,15 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
     const uint32_t lane = threadIdx.x;
+    {
+        // a tile with a very long list is left to the kernels that share a list between waves and workgroups
+        const uint32_t length = ranges[2 * tile + 1] - ranges[2 * tile];
+        if (long_tiles != nullptr && length > long_threshold) {
+            constexpr uint32_t part_words = MODE == HTGS_MODE_HYBRID_BLEND ? long_part_words<KS>() : MODE == HTGS_MODE_OIT_BLEND ? kOitPartWords : first_k_part_words<KS>();
+            if (lane == 0) long_tile_enter(long_tiles, tile, gridDim.x, length, long_threshold, part_words, part_floor);
+            return;
+        }
+    }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
     const bool inside = px.inside;
     const PixelTerms pt = px.pt;
@@ -127,11 +137,142 @@ __global__ void __launch_bounds__(256) max_weights_global_kernel(
     }
 }
 
+// What the pass does with a pixel's finished core and tail when the tile's list was walked by the kernels for very long
+// lists: the weights of the core's entries, and the weight of a tail fragment per unit of alpha into tail_weights[64 tile +
+// lane] (0: no tail fragment of this pixel can reach the threshold) for the second walk (max_weights_tail_long_kernel).
+struct MaxWeightsHybrid {
+    uint32_t *max_weights;
+    float *tail_weights;
+    float weight_threshold;
+    template <int K>
+    __device__ __forceinline__ void operator()(const float4 *__restrict__, uint32_t tile, const TilePixel &, float (&)[K], float (&ca)[K], float (&ci)[K],
+                                               HybridTail &tail) const
+    {
+        float T_core = 1.0f;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const float w = T_core * ca[i];
+            T_core *= 1.0f - ca[i];
+            if (T_core < kTransmittanceThreshold) T_core = 0.0f;
+            if (ca[i] > 0.0f && !(w < weight_threshold)) raise_max(max_weights, float_to_bits(ci[i]), w);
+        }
+        float tail_weight = 0.0f;
+        if (tail.alpha >= weight_threshold) tail_weight = (T_core * (1.0f - tail.T)) * (1.0f / tail.alpha);
+        tail_weights[64u * (size_t)tile + (threadIdx.x & 63u)] = tail_weight >= weight_threshold ? tail_weight : 0.0f;
+    }
+};
+struct MaxWeightsFirstK {
+    uint32_t *max_weights;
+    float weight_threshold;
+    template <int K>
+    __device__ __forceinline__ void operator()(const float4 *__restrict__, uint32_t, const TilePixel &, const float (&)[K], const float (&ca)[K],
+                                               const uint32_t (&ci)[K]) const
+    {
+        float T_core = 1.0f;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const float w = T_core * ca[i];
+            T_core *= 1.0f - ca[i];
+            if (T_core < kTransmittanceThreshold) T_core = 0.0f;
+            if (!(w < weight_threshold)) raise_max(max_weights, ci[i], w);
+        }
+    }
+};
+struct MaxWeightsOit {
+    float *tail_weights;
+    float weight_threshold;
+    __device__ __forceinline__ void operator()(uint32_t tile, const TilePixel &, const OitSums &sum) const
+    {
+        float tail_weight = 0.0f;
+        if (sum.alpha >= weight_threshold) tail_weight = (1.0f * (1.0f - sum.T)) * (1.0f / sum.alpha);
+        tail_weights[64u * (size_t)tile + (threadIdx.x & 63u)] = tail_weight >= weight_threshold ? tail_weight : 0.0f;
+    }
+};
+
+// After the kernels for very long lists have left the tail weights of such tiles: the tiles are entered on the list again,
+// in parts, for the second walk.
+__global__ void __launch_bounds__(256) max_weights_tail_enter_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ long_tiles, uint32_t n_tiles,
+                                                                    uint32_t long_threshold, uint32_t part_floor)
+{
+    const uint32_t tile = blockIdx.x * 256 + threadIdx.x;
+    if (tile >= n_tiles) return;
+    const uint32_t length = ranges[2 * tile + 1] - ranges[2 * tile];
+    if (length > long_threshold) long_tile_enter(long_tiles, tile, n_tiles, length, long_threshold / 4u, 0u, part_floor);   // (parts of one threshold's length)
+}
+// The second walk (alpha * tail weight for every fragment that passes the cut-off) over the parts of the very long lists:
+// a workgroup of four waves per part, every wave a share of it; the maximum is order independent, nothing to merge.
+constexpr int kTailWaves = 4;
+template <int MODE>
+__global__ void __launch_bounds__(64 * kTailWaves) max_weights_tail_long_kernel(
+    const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim, const uint32_t *long_tiles,
+    uint32_t *__restrict__ max_weights, const float *__restrict__ tail_weights, uint32_t width, uint32_t height, uint32_t grid_w, float weight_threshold,
+    uint32_t long_threshold)
+{
+    __shared__ TileStageQ st[kTailWaves];
+    __shared__ QuadrantLists ql[kTailWaves];
+    __shared__ uint32_t s_next;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+    if (long_tiles[0] == 0) return;                   // (the ordinary frame)
+    uint32_t round = 0;
+    LongEntry e;
+    while (long_tile_take(long_tiles, ranges, long_threshold, round, &s_next, e)) {
+        const TilePixel px = quadrant_tile_pixel(e.tile, grid_w, lane, width, height);
+        const PixelTerms pt = px.pt;
+        const float tail_weight = px.inside ? tail_weights[64u * (size_t)e.tile + lane] : 0.0f;
+        const bool active = tail_weight > 0.0f;
+        if (__syncthreads_or(active) == 0) continue;
+        uint32_t share_first, share_last;
+        long_wave_share(e.first, e.last, wave, share_first, share_last, kTailWaves);
+        tile_list_walk<MODE, false, kCullCutoff, false>(st[wave], ql[wave], prim, inst, share_first, share_last, lane, px.cx, px.cy, [&](uint32_t addr) {
+            TileFrag f;
+            if (!active || !tile_frag_cutoff<kStageSlots>(addr, pt, f)) return;
+            const float G = d_exp2((f.num * ModeCfg<MODE>::exp2_scale) * rcp_exact(f.den));
+            const float a = stage_opacity<kStageSlots>(addr) * G;
+            const float w = (a < kMaxFragmentAlpha ? a : kMaxFragmentAlpha) * tail_weight;
+            if (!(w < weight_threshold)) raise_max(max_weights, stage_index<kStageSlots>(addr), w);
+        });
+    }
+}
+
+// the least length of a part of a long list; 0: lists are not split (there is no spare value buffer for what the parts leave behind)
+static uint32_t part_floor_of(const htgs_frame *f, int sel, uint32_t n_tiles, bool needs_spare)
+{
+    if (needs_spare && f->vals[sel ^ 1] == nullptr) return 0u;
+    const uint64_t floor = (f->n_instances + n_tiles - 1) / n_tiles;
+    return floor < 1u ? 1u : (uint32_t)floor;
+}
+// the tiles with very long lists are taken by the kernels that share a list only when the caller provided the list for such
+// tiles and, in the modes with a tail, the per-pixel scratch for the tail weights between the two walks
+template <int MODE>
+static bool shares_long_lists(const htgs_frame *f) { return f->long_tiles != nullptr && (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K || f->pixel_scratch != nullptr); }
+
 template <int K, int MODE>
 static void launch_tile(const htgs_frame *f, int sel, uint32_t *max_weights, float thr, uint32_t grid_w, uint32_t n_tiles)
 {
-    hipLaunchKernelGGL((max_weights_tile_kernel<K, MODE>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[sel],
-                       (const float4 *)f->prim, max_weights, (uint32_t)f->width, (uint32_t)f->height, grid_w, thr, f->tile_order);
+    hipStream_t s = (hipStream_t)f->stream;
+    const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
+    const bool shared = shares_long_lists<MODE>(f);
+    const uint32_t w = (uint32_t)f->width, h = (uint32_t)f->height;
+    hipLaunchKernelGGL((max_weights_tile_kernel<K, MODE>), dim3(n_tiles), dim3(64), 0, s, f->ranges, f->vals[sel], (const float4 *)f->prim, max_weights, w, h, grid_w,
+                       thr, f->tile_order, shared ? f->long_tiles : nullptr, threshold, part_floor_of(f, sel, n_tiles, true));
+    if (!shared) return;
+    constexpr int REC4 = HTGS_PRIM_FLOATS / 4;
+    if constexpr (MODE == HTGS_MODE_HYBRID_BLEND)
+        hipLaunchKernelGGL((blend_hybrid_long_kernel<K, false, REC4, MaxWeightsHybrid>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0, s,
+                           f->ranges, f->vals[sel], (const float4 *)f->prim, f->long_tiles, w, h, grid_w, f->vals[sel ^ 1], threshold,
+                           MaxWeightsHybrid{ max_weights, f->pixel_scratch, thr });
+    else if constexpr (MODE == HTGS_MODE_ALPHA_BLEND_FIRST_K)
+        hipLaunchKernelGGL((blend_first_k_long_kernel<K, false, REC4, MaxWeightsFirstK>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0, s,
+                           f->ranges, f->vals[sel], (const float4 *)f->prim, f->long_tiles, w, h, grid_w, f->vals[sel ^ 1], threshold, MaxWeightsFirstK{ max_weights, thr });
+    else
+        hipLaunchKernelGGL((blend_oit_long_kernel<false, REC4, MaxWeightsOit, false>), dim3(256), dim3(64 * kLongWaves), 0, s, f->ranges, f->vals[sel],
+                           (const float4 *)f->prim, f->long_tiles, w, h, grid_w, f->vals[sel ^ 1], threshold, MaxWeightsOit{ f->pixel_scratch, thr });
+    if constexpr (MODE != HTGS_MODE_ALPHA_BLEND_FIRST_K) {
+        hipLaunchKernelGGL(max_weights_tail_enter_kernel, dim3((n_tiles + 255) / 256), dim3(256), 0, s, f->ranges, f->long_tiles, n_tiles, threshold,
+                           part_floor_of(f, sel, n_tiles, false));
+        hipLaunchKernelGGL(max_weights_tail_long_kernel<MODE>, dim3(1024), dim3(64 * kTailWaves), 0, s, f->ranges, f->vals[sel], (const float4 *)f->prim, f->long_tiles,
+                           max_weights, f->pixel_scratch, w, h, grid_w, thr, threshold);
+    }
 }
 
 template <int MODE>

@@ -417,16 +417,27 @@ def update_max_weights(
 ) -> None:
     """Raises ``max_weights`` ([N] or [N,1] float32, in place) to the largest blending weight each Gaussian reaches in
     this view; weights below ``weight_threshold`` are ignored (reference: rasterization.py:189-206)."""
+    run_max_weights(max_weights, positions, scales, rotations, opacities, settings, weight_threshold)
+
+
+def run_max_weights(max_weights, positions, scales, rotations, opacities, settings, weight_threshold, long_list_threshold: int = 0) -> FrameBuffers:
+    """``update_max_weights`` with the length beyond which a tile's list is shared between waves and workgroups made
+    explicit (0: the library's default); returns the frame."""
     n = positions.shape[0]
     if not (isinstance(max_weights, torch.Tensor) and max_weights.is_cuda and max_weights.dtype == torch.float32
             and max_weights.is_contiguous() and max_weights.numel() == n):
         raise RuntimeError("max_weights must be a contiguous float32 GPU tensor with one element per Gaussian")
     with torch.no_grad():
         fb = FrameBuffers(positions, scales, rotations, opacities, None, None, settings, True, False,
-                          pool=ScratchPool.current(positions.device))
+                          pool=ScratchPool.current(positions.device), long_list_threshold=long_list_threshold)
+        if fb.mode in (0, 3):
+            # the tail weights of the tiles with very long lists, kept between the pass's two walks
+            fb.pixel_scratch = fb._scratch("pixel_scratch", 64 * fb.n_tiles, torch.float32)
+            fb.frame.pixel_scratch = _ptr(fb.pixel_scratch)
         _native.check(fb.lib.htgs_max_weights_front(fb._ref))
         fb.alloc_instances(fb.read_instance_count())
         _native.check(fb.lib.htgs_max_weights_back(fb._ref, max_weights.data_ptr(), float(weight_threshold)))
+    return fb
 
 
 def rasterize(

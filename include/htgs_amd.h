@@ -135,6 +135,10 @@ typedef struct htgs_frame {
     float *densification_info; /* [densification_rows,N] updated in place, or NULL (rasterization_api.cu:219-223) */
     int32_t densification_rows; /* 0, 2 or 3 */
     int32_t use_distance_scaling;
+    /* ---- htgs_max_weights_blend ---- */
+    float *pixel_scratch;      /* [64 n_tiles] floats or NULL.  With long_tiles, in the modes with a tail (HYBRID_BLEND, OIT_BLEND):
+                                  the weight of a tail fragment per unit of alpha at every pixel of the tiles with very long
+                                  lists, kept between the pass's two walks.  NULL: such tiles are walked by one wave there */
     /* ---- execution ---- */
     void *stream;              /* hipStream_t */
 } htgs_frame;

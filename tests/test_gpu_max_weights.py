@@ -62,3 +62,32 @@ def test_two_views_accumulate(cuda):
     assert bool((mw >= first).all()) and bool((mw > first).any())
     with pytest.raises(RuntimeError):
         update_max_weights(mw[:10], *scene.gaussians()[:4], s, 0.02)
+
+
+@pytest.mark.parametrize("config,n,K,long_threshold", [(0, 6000, 4, 40), (1, 50_000, 16, 24), (3, 30_000, 8, 300), (3, 30_000, 1, 100)])
+@pytest.mark.parametrize("mode", [0, 1, 3])
+def test_max_weights_with_very_long_lists(cuda, config, n, K, mode, long_threshold):
+    """Tiles whose lists exceed the threshold (forced down here) go to the kernels that share a list between waves and
+    workgroups -- the core's weights from the merged K-buffers, the tail's from a second walk in parts -- and the result
+    is the oracle's: bit for bit in ALPHA_BLEND_FIRST_K (the maximum does not depend on the order of arrival), to the rounding of
+    the tail's sums -- which the shares of a list add up in another order -- in the modes with a tail."""
+    from htgs_amd.torch_bindings.rasterization import run_max_weights
+    print(f"case config={config} n={n} mode={mode} K={K} long_threshold={long_threshold}", flush=True)
+    scene = make_scene(config, n)
+    want = np.zeros(n, dtype=np.float32)
+    threshold = 0.01
+    oracle.update_max_weights(oracle_frame(scene, mode, K), want, *[t.numpy() for t in scene.gaussians()[:4]], threshold)
+    sg = scene.to(cuda)
+    got = torch.zeros(n, 1, device=cuda)
+    fb = run_max_weights(got, *sg.gaussians()[:4], sg.settings(RasterizerMode(mode), K), threshold, long_list_threshold=long_threshold)
+    torch.cuda.synchronize()
+    lengths = (fb.ranges[:, 1] - fb.ranges[:, 0]).to(torch.int64)
+    assert int((lengths > long_threshold).sum()) > 0 and not bool(fb.long_tiles[:6].any())
+    if mode == 1:
+        np.testing.assert_array_equal(got.cpu().numpy().reshape(-1).view(np.uint32), want.view(np.uint32))
+    else:
+        # (a weight within rounding of the threshold may fall on the other side of it: compared where both sides kept it)
+        g = got.cpu().numpy().reshape(-1)
+        both = (g > 0) & (want > 0)
+        np.testing.assert_allclose(g[both], want[both], rtol=1e-5)
+        assert (both != ((g > 0) | (want > 0))).sum() <= 2
