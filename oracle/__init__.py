@@ -228,6 +228,21 @@ def blend(frame: Frame, pre: dict, ranges: np.ndarray, sorted_vals: np.ndarray, 
     return image, depth, alpha
 
 
+def blend_hybrid_literal(frame: Frame, pre: dict, ranges: np.ndarray, sorted_vals: np.ndarray, use_median_depth: bool = False, margin: float = 1e-3):
+    """The HYBRID_BLEND inference image by the word-for-word fp32 restatement of the reference's blend kernel (plane form,
+    libm expf, premultiplied core, tail fed by what leaves the core): ``(image [3,H,W], depth [H,W], flags [H,W])`` where
+    a flag marks a pixel one of whose decisions fell within ``margin`` (relative) of its bound."""
+    h, w = frame.height, frame.width
+    image = np.zeros((3, h, w), np.float32)
+    depth = np.zeros((h, w), np.float32)
+    flags = np.zeros((h, w), np.uint8)
+    cam = frame.c_struct(0)
+    lib().oracle_blend_hybrid_literal(ctypes.byref(cam), _p(ranges), _p(sorted_vals), _p(pre["VPMT1"]), _p(pre["VPMT2"]), _p(pre["VPMT4"]),
+                                      _p(pre["MT3"]), _p(pre["rgba"]), ctypes.c_int(bool(use_median_depth)), ctypes.c_float(margin),
+                                      _p(image), _p(depth), _p(flags))
+    return image, depth, flags
+
+
 def render(frame: Frame, positions, scales, rotations, opacities, sh_0, sh_rest,
            to_chw: bool = True, use_median_depth: bool = False) -> dict:
     """Whole inference path; returns every intermediate so that tests can compare stage by stage."""

@@ -825,6 +825,115 @@ O_EXPORT void oracle_blend(
     }
 }
 
+/* ---- HYBRID_BLEND inference once more, word for word ------------------------------------------------
+ * R/include/hybrid_blend/kernels/inference.cuh:137-213 as the source states it: the two planes per pixel
+ * (VPMT1 - VPMT4 * pixel_x, :137-138), m and d from them (:141-142), the cut-off against max_cutoff_sq * |d|^2
+ * (:145), libm's expf (:147), a premultiplied RGBA core that is exchanged slot by slot (:158-167), and a tail that
+ * receives only what leaves (or never enters) the core (:168-170).  No fused operations, no polynomial exp, no
+ * tile-relative form, no colour bookkeeping: nothing of what the production path above (hybrid_pixel) shares with
+ * the HIP kernels.  It is the independent fp32 statement that hybrid_pixel is checked against image-wise
+ * (tests/test_oracle_pinning.py); the two differ by rounding, except where a decision (cut-off, alpha thresholds,
+ * an exchange between nearly equal depths, the transmittance threshold, the tail's alpha threshold) falls within
+ * `margin` (relative) of its bound -- such pixels are reported in flags[] and left out of the comparison.
+ * pinned by: nothing further -- it is itself a pin. */
+static void hybrid_pixel_literal(const blend_in *in, uint32_t first, uint32_t last, int x, int y, int K, int median, float margin,
+                                 float out[4], uint8_t *flag)
+{
+    const float pixel_x = (float)x, pixel_y = (float)y;
+    const float cutoff_sq = mode_cutoff_sq(MODE_HYBRID), min_alpha = mode_min_alpha(MODE_HYBRID);
+    float transmittance_tail = 1.0f, tail[4] = { 0, 0, 0, 0 }, depth_tail = 0.0f;
+    float core[KMAX][4], depths_core[KMAX];
+    int near = 0;
+#define NEAR(a, b) (fabsf((a) - (b)) <= margin * fmaxf(fabsf(a), fabsf(b)))
+    for (int i = 0; i < K; ++i) { core[i][0] = core[i][1] = core[i][2] = core[i][3] = 0.0f; depths_core[i] = FLT_MAX; }
+    for (uint32_t j = first; j < last; ++j) {
+        const size_t g = in->inst[j];
+        const float *V1 = in->VPMT1 + 4 * g, *V2 = in->VPMT2 + 4 * g, *V4 = in->VPMT4 + 4 * g, *MT3 = in->MT3 + 4 * g, *rgba = in->rgba + 4 * g;
+        float px[4], py[4], m[3], d[3];
+        for (int k = 0; k < 4; ++k) { px[k] = V1[k] - V4[k] * pixel_x; py[k] = V2[k] - V4[k] * pixel_y; }
+        for (int k = 0; k < 3; ++k) m[k] = px[3] * py[k] - px[k] * py[3];
+        d[0] = px[1] * py[2] - px[2] * py[1]; d[1] = px[2] * py[0] - px[0] * py[2]; d[2] = px[0] * py[1] - px[1] * py[0];
+        const float numerator_rho2 = m[0] * m[0] + m[1] * m[1] + m[2] * m[2];
+        const float denominator = d[0] * d[0] + d[1] * d[1] + d[2] * d[2];
+        /* (the cancellation in VPMT1 - VPMT4 * x leaves rho^2 with a relative error of some 1e-4 at the benchmark cameras, in
+         * either form: the margin of this test scales with it through the caller's `margin`) */
+        near |= NEAR(numerator_rho2, cutoff_sq * denominator);
+        if (numerator_rho2 > cutoff_sq * denominator) continue;
+        const float denominator_rcp = 1.0f / denominator;
+        const float G = expf(-0.5f * numerator_rho2 * denominator_rcp);
+        const float alpha = fminf(rgba[3] * G, MAX_FRAGMENT_ALPHA);
+        near |= NEAR(alpha, min_alpha) | NEAR(alpha, MIN_ALPHA_CORE);
+        if (alpha < min_alpha) continue;
+        const float e[3] = { (d[1] * m[2] - d[2] * m[1]) * denominator_rcp, (d[2] * m[0] - d[0] * m[2]) * denominator_rcp,
+                             (d[0] * m[1] - d[1] * m[0]) * denominator_rcp };
+        float depth = (MT3[0] * e[0] + MT3[1] * e[1] + MT3[2] * e[2]) + MT3[3];
+        float pm[4] = { rgba[0] * alpha, rgba[1] * alpha, rgba[2] * alpha, alpha };
+        if (alpha >= MIN_ALPHA_CORE)
+            for (int i = 0; i < K; ++i) near |= depths_core[i] < FLT_MAX && NEAR(depth, depths_core[i]);
+        if (depth < depths_core[K - 1] && alpha >= MIN_ALPHA_CORE) {
+            for (int i = 0; i < K; ++i) {
+                if (depth < depths_core[i]) {
+                    float t = depth; depth = depths_core[i]; depths_core[i] = t;
+                    for (int k = 0; k < 4; ++k) { t = pm[k]; pm[k] = core[i][k]; core[i][k] = t; }
+                }
+            }
+        }
+        for (int k = 0; k < 4; ++k) tail[k] += pm[k];
+        if (!median) depth_tail += depth * pm[3];
+        transmittance_tail *= 1.0f - pm[3];
+    }
+    float rgb[3] = { 0, 0, 0 }, depth_pixel = 0.0f, transmittance_core = 1.0f;
+    for (int i = 0; i < K && transmittance_core >= TRANSMITTANCE_THRESHOLD; ++i) {
+        for (int k = 0; k < 3; ++k) rgb[k] += transmittance_core * core[i][k];
+        const float depth = depths_core[i];
+        if (median) { near |= NEAR(transmittance_core, 0.5f); depth_pixel = (transmittance_core > 0.5f && depth < FLT_MAX) ? depth : depth_pixel; }
+        else depth_pixel += transmittance_core * core[i][3] * depth;
+        transmittance_core *= 1.0f - core[i][3];
+        near |= NEAR(transmittance_core, TRANSMITTANCE_THRESHOLD);
+    }
+    float total_alpha = 0.0f;
+    if (!median) total_alpha = 1.0f - transmittance_core;
+    near |= NEAR(tail[3], min_alpha);
+    if (transmittance_core >= TRANSMITTANCE_THRESHOLD && tail[3] >= min_alpha) {
+        const float weight_tail = transmittance_core * (1.0f - transmittance_tail);
+        for (int k = 0; k < 3; ++k) rgb[k] += weight_tail * (1.0f / tail[3]) * tail[k];
+        if (!median) { depth_pixel += weight_tail * (1.0f / tail[3]) * depth_tail; total_alpha += weight_tail; }
+    }
+    if (!median) depth_pixel = total_alpha > 0.0f ? depth_pixel / total_alpha : 0.0f;
+#undef NEAR
+    out[0] = saturate(rgb[0]); out[1] = saturate(rgb[1]); out[2] = saturate(rgb[2]); out[3] = depth_pixel;
+    *flag = (uint8_t)near;
+}
+
+/* The HYBRID_BLEND inference image by hybrid_pixel_literal: image [3,H,W], depths [H,W], flags [H,W] (1: a decision of
+ * this pixel fell within `margin`, relative, of its bound). */
+O_EXPORT void oracle_blend_hybrid_literal(
+    const oracle_cam *c, const uint32_t *ranges, const uint32_t *inst,
+    const float *VPMT1, const float *VPMT2, const float *VPMT4, const float *MT3, const float *rgba,
+    int use_median_depth, float margin, float *image, float *depths, uint8_t *flags)
+{
+    const int grid_w = (c->width + c->tile_w - 1) / c->tile_w;
+    const int grid_h = (c->height + c->tile_h - 1) / c->tile_h;
+    const blend_in in = { ranges, inst, VPMT1, VPMT2, VPMT4, MT3, rgba, NULL, 0, c->tile_w, c->tile_h };
+    const int K = round_k(c->K);
+    const size_t np = (size_t)c->width * c->height;
+    #pragma omp parallel for schedule(dynamic, 4)
+    for (int t = 0; t < grid_w * grid_h; ++t) {
+        const int tx = t % grid_w, ty = t / grid_w;
+        const uint32_t first = ranges[2 * t], last = ranges[2 * t + 1];
+        for (int ly = 0; ly < c->tile_h; ++ly)
+            for (int lx = 0; lx < c->tile_w; ++lx) {
+                const int x = tx * c->tile_w + lx, y = ty * c->tile_h + ly;
+                if (x >= c->width || y >= c->height) continue;
+                float out[4];
+                const size_t pix = (size_t)c->width * y + x;
+                hybrid_pixel_literal(&in, first, last, x, y, K, use_median_depth, margin, out, flags + pix);
+                image[pix] = out[0]; image[np + pix] = out[1]; image[2 * np + pix] = out[2];
+                depths[pix] = out[3];
+            }
+    }
+}
+
 /* ========================================================================= */
 /* training: forward with per-pixel records, backward                        */
 /* ========================================================================= */

@@ -64,3 +64,42 @@ def load_golden(name: str = "small_scene"):
     scene = Scene(name, t("positions"), t("scales"), t("rotations"), t("opacities"), t("sh_0"), t("sh_rest"), t("M"), t("VPM"),
                   t("cam_position"), width, height, float(z["planes"][0]), float(z["planes"][1]), int(z["active_sh_bases"]), int(z["K"]))
     return scene, z
+
+
+def tie_scene(depths, opacities, colours):
+    """Isotropic Gaussians on the optical axis of a 64x64 pinhole camera whose principal point maps to pixel (32, 32):
+    at that pixel the ray passes through every centre, so fragment k has alpha = opacities[k] and depth = depths[k]
+    exactly (|m|^2 = 0, exp(0) = 1, the point of maximum contribution is the centre), in list order = index order.
+    Gaussians given the same depth are coincident (same shape): their fragments have bit-identical depths at every
+    pixel.  SH degree 0 with the given colours."""
+    from htgs_amd.synthetic import SH_C0, pinhole
+    n = len(depths)
+    pos = torch.zeros(n, 3)
+    pos[:, 2] = torch.tensor(depths, dtype=torch.float32)
+    scales = torch.full((n, 3), 0.05) * pos[:, 2:3]              # the same angular size
+    rot = torch.zeros(n, 4)
+    rot[:, 0] = 1.0
+    opac = torch.tensor(opacities, dtype=torch.float32).reshape(n, 1)
+    sh_0 = ((torch.tensor(colours, dtype=torch.float32) - 0.5) / SH_C0).reshape(n, 1, 3)
+    M, VPM, cam = pinhole(64, 64, 100.0, 100.0, 32.5, 32.5, 0.1, 100.0)
+    return Scene("ties", pos, scales.contiguous(), rot, opac, sh_0.contiguous(), torch.zeros(n, 0, 3), M, VPM, cam, 64, 64, 0.1, 100.0, 1, 4)
+
+
+def hybrid_pixel_by_hand(order, tail, depths, opacities, colours):
+    """HYBRID_BLEND's pixel in float64 from its definition, for a core given as a list of fragment numbers in the order
+    they are blended and the fragments in the tail: (rgb, depth) (R/include/hybrid_blend/kernels/inference.cuh:172-200)."""
+    a, c, d = np.asarray(opacities, np.float64), np.asarray(colours, np.float64), np.asarray(depths, np.float64)
+    rgb, depth, T = np.zeros(3), 0.0, 1.0
+    for k in order:
+        rgb += T * a[k] * c[k]
+        depth += T * a[k] * d[k]
+        T *= 1.0 - a[k]
+    total_alpha = 1.0 - T
+    if tail:
+        alpha_sum = sum(a[k] for k in tail)
+        T_tail = np.prod([1.0 - a[k] for k in tail])
+        w = T * (1.0 - T_tail) / alpha_sum
+        rgb += w * sum(a[k] * c[k] for k in tail)
+        depth += w * sum(a[k] * d[k] for k in tail)
+        total_alpha += T * (1.0 - T_tail)
+    return np.clip(rgb, 0.0, 1.0), depth / total_alpha
