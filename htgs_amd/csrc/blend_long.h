@@ -66,15 +66,20 @@ __device__ __forceinline__ void hybrid_walk(TileStageQ &st, QuadrantLists &ql, c
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
     constexpr int N = kStageSlots;
-    tile_list_walk<MODE, true, PIXELS ? kCullPixels : kCullAlpha, SOLO, REC4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+    tile_list_walk<MODE, true, PIXELS ? kCullPixels : kCullAlpha, SOLO, REC4, FAST>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
         // cut-off and alpha threshold are tested together: the lanes of a quadrant that its instance does not
         // reach run along to the second test (one exec level less for the scalar unit to manage; the staging
         // cull leaves hardly a turn in which no lane passes, so there is nothing to skip)
         TileFrag f;
-        const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
-        f.den_rcp = frag_rcp<FAST>(f.den);
+        bool fragment;
+        if constexpr (FAST) fragment = tile_frag_fast<MODE, N>(addr, pt, f);
+        else {
+            const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+            f.den_rcp = frag_rcp<FAST>(f.den);
+            fragment = tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach;
+        }
         const float4 col = stage_row<N, 5>(addr);
-        if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach)) return;
+        if (!fragment) return;
         float depth = tile_frag_depth<N>(addr, pt, f);
         float p3 = f.alpha;
         tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
@@ -857,12 +862,17 @@ __device__ __forceinline__ void oit_walk(TileStageQ &st, QuadrantLists &ql, cons
 {
     constexpr int MODE = HTGS_MODE_OIT_BLEND;
     constexpr int N = kStageSlots;
-    tile_list_walk<MODE, DEPTH, kCullAlpha, SOLO, REC4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+    tile_list_walk<MODE, DEPTH, kCullAlpha, SOLO, REC4, FAST>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
         TileFrag f;
-        const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
-        f.den_rcp = frag_rcp<FAST>(f.den);
+        bool fragment;
+        if constexpr (FAST) fragment = tile_frag_fast<MODE, N>(addr, pt, f);
+        else {
+            const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+            f.den_rcp = frag_rcp<FAST>(f.den);
+            fragment = tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach;
+        }
         const float4 col = stage_row<N, 5>(addr);
-        if (!(tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach)) return;
+        if (!fragment) return;
         const float depth = DEPTH ? tile_frag_depth<N>(addr, pt, f) : 0.0f;
         sum.a0 = __builtin_fmaf(f.alpha, col.x, sum.a0);
         sum.a1 = __builtin_fmaf(f.alpha, col.y, sum.a1);

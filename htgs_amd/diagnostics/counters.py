@@ -54,7 +54,7 @@ def scale_factor(db_path: str, counter: str) -> float:
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--key", required=True, help="workload key, as bench.py builds it: cfg<c>[-n<N>]/mode<m>/K<k>/<rasterize|fast_rasterize|train<rows>>")
-    ap.add_argument("--kernel", required=True, help="substring naming the dominant kernel of that workload")
+    ap.add_argument("--kernel", required=True, help="substring naming the dominant kernel (or kernels: their bytes add up) of that workload")
     ap.add_argument("--fetch", required=True)
     ap.add_argument("--write", required=True)
     ap.add_argument("--cal-fetch", required=True)
@@ -64,12 +64,15 @@ def main():
 
     fs, ws = scale_factor(args.cal_fetch, "FETCH_SIZE"), scale_factor(args.cal_write, "WRITE_SIZE")
     fetch, write = per_kernel_median(args.fetch, "FETCH_SIZE"), per_kernel_median(args.write, "WRITE_SIZE")
-    names = [k for k in fetch if args.kernel in k]
-    if len(names) != 1:
-        raise SystemExit(f"--kernel {args.kernel!r} matches {names}")
-    name = names[0]
-    read_b, write_b = fetch[name] * 1024.0 * fs, write.get(name, 0.0) * 1024.0 * ws
-    entry = {"kernel": name, "fetch_KiB": fetch[name], "write_KiB": write.get(name, 0.0), "fetch_scale": round(fs, 4),
+    # (the dominant stage of a workload may be two launches -- the kernel with one wave per tile and the one for the tiles
+    # with very long lists: every kernel whose name contains the pattern counts, their bytes add up)
+    names = sorted(k for k in fetch if args.kernel in k)
+    if not names:
+        raise SystemExit(f"--kernel {args.kernel!r} matches no kernel of {args.fetch}")
+    fetch_kib = sum(fetch[k] for k in names)
+    write_kib = sum(write.get(k, 0.0) for k in names)
+    read_b, write_b = fetch_kib * 1024.0 * fs, write_kib * 1024.0 * ws
+    entry = {"kernel": " + ".join(names), "fetch_KiB": fetch_kib, "write_KiB": write_kib, "fetch_scale": round(fs, 4),
              "write_scale": round(ws, 4), "read_bytes": int(read_b), "written_bytes": int(write_b), "traffic_bytes": int(read_b + write_b)}
     digest = csrc_digest()
     try:

@@ -79,27 +79,60 @@ class ScratchPool:
     """Grow-only device scratch that inference frames on one (device, stream, host thread) reuse, so that a steady
     stream of ``rasterize`` calls allocates nothing but its outputs.  A frame is issued front to back by one thread and
     ordered by the stream, which is what makes the reuse safe; frames issued on another stream or by another thread
-    get another pool.  Training frames do not use it (their scratch has to survive until backward)."""
+    get another pool.  Training frames do not use it (their scratch has to survive until backward).
+
+    The pools are bounded: the pool of a thread that has ended is dropped the next time a pool is looked up, and with
+    ``ScratchPool.max_bytes`` set the pools used least recently are dropped (never the one being asked for) until the
+    others fit under it.  Dropping a pool only releases the references; torch's stream-ordered allocator keeps the memory
+    valid for work already queued."""
 
     _pools: dict = {}
     _lock = threading.Lock()
+    _tick = 0
+    max_bytes: Optional[int] = None       # cap on the bytes held by all pools together (None: no cap)
 
     def __init__(self):
         self.buffers: dict = {}
+        self.last_used = 0
+
+    def nbytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self.buffers.values())
+
+    @staticmethod
+    def _stream_id(device: torch.device) -> int:
+        return torch.cuda.current_stream(device).cuda_stream if device.type == "cuda" else 0
 
     @classmethod
     def current(cls, device: torch.device) -> "ScratchPool":
-        key = (device.index, torch.cuda.current_stream(device).cuda_stream, threading.get_ident())
+        key = (device.type, device.index, cls._stream_id(device), threading.get_ident())
         with cls._lock:
             pool = cls._pools.get(key)
             if pool is None:
                 pool = cls._pools[key] = ScratchPool()
+                alive = {t.ident for t in threading.enumerate()}
+                for other in [k for k in cls._pools if k[3] not in alive]:
+                    del cls._pools[other]
+            cls._tick += 1
+            pool.last_used = cls._tick
+            if cls.max_bytes is not None:
+                others = sorted((k for k in cls._pools if k != key), key=lambda k: cls._pools[k].last_used)
+                held = sum(p.nbytes() for p in cls._pools.values())
+                for k in others:
+                    if held <= cls.max_bytes:
+                        break
+                    held -= cls._pools[k].nbytes()
+                    del cls._pools[k]
         return pool
 
     @classmethod
     def clear(cls):
         with cls._lock:
             cls._pools.clear()
+
+    @classmethod
+    def total_bytes(cls) -> int:
+        with cls._lock:
+            return sum(p.nbytes() for p in cls._pools.values())
 
     def get(self, name: str, numel: int, dtype: torch.dtype, device: torch.device, headroom: float = 0.0) -> torch.Tensor:
         buf = self.buffers.get(name)
