@@ -77,15 +77,16 @@ typedef struct htgs_frame {
     uint32_t *n_instances_dev; /* [1] total number of instances, written by the scan */
     /* ---- per-tile scratch (PerTileBuffers, buffer_utils.h:86-94) ---- */
     uint32_t *ranges;          /* [n_tiles,2] first,last+1 into the sorted instance list */
-    uint32_t *long_tiles;      /* [8 + 3 n_tiles] or NULL.  Inference in HYBRID_BLEND, ALPHA_BLEND_FIRST_K and OIT_BLEND
-                                  (the modes that walk all of a list): tiles whose list is longer than
+    uint32_t *long_tiles;      /* [8 + 3 n_tiles] or NULL.  HYBRID_BLEND, ALPHA_BLEND_FIRST_K and OIT_BLEND (the modes that
+                                  walk all of a list), every blend stage: htgs_blend, htgs_blend_forward,
+                                  htgs_blend_backward, htgs_max_weights_blend.  Tiles whose list is longer than
                                   long_list_threshold are collected here (word 0: entries on the list, words 1-5: work
                                   counters, words 6-7: how the tiles with fragments of equal depth were settled, for
                                   tests; the eight header words are zeroed by htgs_extract_ranges, words 0-5 again by
-                                  htgs_blend when it is done with the list; then 2 n_tiles words of entries -- a list
+                                  every stage when it is done with the list; then 2 n_tiles words of entries -- a list
                                   of several times the threshold is entered in up to 32 parts -- and a counter per
-                                  tile) and walked by several waves each, the longest first; htgs_blend then also
-                                  overwrites vals[1 - selector], see there.
+                                  tile) and walked by several waves or workgroups each, the longest first; the forward
+                                  stages then also overwrite vals[1 - selector], see htgs_blend.
                                   NULL: every tile is walked by one wave (no counterpart in the reference, which
                                   does that) */
     int32_t long_list_threshold; /* 0 = the default (8192 instances) */
@@ -200,7 +201,8 @@ int htgs_extract_ranges(const htgs_frame *f, int selector);
  * HYBRID's tail and of OIT (pixels at which fragments of exactly equal depth met get the reference's insertion replayed in
  * list order on the fragments that decide the K-buffer; FIRST_K comes out bit for bit).  That launch uses the spare
  * value buffer vals[1 - selector] as scratch (its content is lost; NULL: a slower path without it, one workgroup per
- * tile).  Without long_tiles the stage reads vals[selector] only. */
+ * tile).  Without long_tiles the stage reads vals[selector] only.  How a long list is split over workgroups depends on its
+ * length and on n_instances alone: results do not depend on the order in which workgroups run. */
 int htgs_blend(const htgs_frame *f, int selector);
 
 /* <mode>::inference split at its one host/device synchronisation point (inference.cu:118-119):
@@ -218,9 +220,12 @@ int htgs_render_back(const htgs_frame *f);
 int htgs_forward_front(const htgs_frame *f);
 /* create instances + sort + ranges + forward blend; *selector as in htgs_sort_instances */
 int htgs_forward_back(const htgs_frame *f, int *selector);
-/* blend_cu (forward) of the frame's mode, R/include/<mode>/kernels/forward.cuh */
+/* blend_cu (forward) of the frame's mode, R/include/<mode>/kernels/forward.cuh.  With f->long_tiles the tiles with very long
+ * lists are walked as in htgs_blend (same kernels, same use of vals[1 - selector]); the recorded core indices are those
+ * of the single walk. */
 int htgs_blend_forward(const htgs_frame *f, int selector);
-/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: writes grad_rows and dens_helper */
+/* blend_cu (backward), R/include/<mode>/kernels/backward.cuh: writes grad_rows and dens_helper.  With f->long_tiles a
+ * very long list is cut into parts for separate workgroups (every instance writes a row of its own). */
 int htgs_blend_backward(const htgs_frame *f, int selector);
 /* preprocess_cu (backward), R/include/hybrid_blend/kernels/backward.cuh:10-102: grad_rows -> the six gradients */
 int htgs_preprocess_backward(const htgs_frame *f);
