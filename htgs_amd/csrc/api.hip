@@ -81,7 +81,7 @@ extern "C" int htgs_key_bytes(int mode, int width, int height)
 extern "C" int htgs_frame_end_bit(const htgs_frame *f)
 {
     if (!f) return 0;
-    return htgs_end_bit(f->mode, f->width, f->height) - (frame_depth_ordered(f) ? 32 : 0);
+    return htgs_end_bit(f->mode, f->width, f->height) - (frame_depth_ordered(f) && f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING ? 32 : 0);
 }
 
 extern "C" int htgs_frame_key_bytes(const htgs_frame *f)

@@ -44,8 +44,17 @@ inline int frame_prim_floats(const htgs_frame *f)
     return f->prim_floats == 0 || f->prim_floats == HTGS_PRIM_FLOATS ? HTGS_PRIM_FLOATS : f->prim_floats == HTGS_PRIM_FLOATS_TRAIN ? HTGS_PRIM_FLOATS_TRAIN : -1;
 }
 
-// ALPHA_BLEND_GLOBAL_ORDERING with the Gaussians sorted by depth before the instances are made (htgs_frame.depth_order)
-inline bool frame_depth_ordered(const htgs_frame *f) { return f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING && f->depth_order != nullptr; }
+// The Gaussians are sorted by depth before the instances are made (htgs_frame.depth_order): ALPHA_BLEND_GLOBAL_ORDERING,
+// whose lists must be in depth order, and the image-only fast path of the two modes with a sorted core, whose lists may
+// be in any order and whose insertions become rare when the fragments arrive roughly front to back (coarse keys, one pass)
+inline bool frame_coarse_depth_ordered(const htgs_frame *f)
+{
+    return f->depth_order != nullptr && f->fast_math && (f->mode == HTGS_MODE_HYBRID_BLEND || f->mode == HTGS_MODE_ALPHA_BLEND_FIRST_K);
+}
+inline bool frame_depth_ordered(const htgs_frame *f)
+{
+    return (f->mode == HTGS_MODE_ALPHA_BLEND_GLOBAL_ORDERING && f->depth_order != nullptr) || frame_coarse_depth_ordered(f);
+}
 // the parts of depth_order, n4 = N rounded up to a multiple of four words each: depth keys and Gaussian indices (two
 // buffers each for the sort, which leaves its result in the first ones after four passes; htgs_preprocess writes the
 // pairs), the counts and the tile rectangles in depth order, scratch of the sort
@@ -67,13 +76,15 @@ inline DepthOrder depth_order_parts(const htgs_frame *f)
 // patterns order like the depths; these are the low 32 bits of the reference's tile | depth keys) less that of the near
 // plane, which no Gaussian that is not culled lies in front of, `culled` for a culled Gaussian (behind all others).  With
 // the far plane as the upper bound the keys of the usual cameras have 27 bits: three passes of 9-bit digits.
+// Coarse keys (frame_coarse_depth_ordered): the same keys shifted down until nine bits are left, one pass.
 struct DepthKeys {
     uint32_t base, culled;
-    int end_bit, digit_bits, passes;
+    int end_bit, digit_bits, passes, shift;
 };
+constexpr int kCoarseDepthBits = 9;
 inline DepthKeys depth_key_range(const htgs_frame *f)
 {
-    DepthKeys k = { 0u, 0xffffffffu, 32, 8, 4 };
+    DepthKeys k = { 0u, 0xffffffffu, 32, 8, 4, 0 };
     const float near_plane = f->near_plane, far_plane = f->far_plane;
     if (near_plane > 0.0f && far_plane >= near_plane && far_plane < __builtin_huge_valf()) {
         uint32_t lo, hi;
@@ -86,6 +97,12 @@ inline DepthKeys depth_key_range(const htgs_frame *f)
         const int passes8 = (k.end_bit + 7) / 8, passes9 = (k.end_bit + 8) / 9;
         k.digit_bits = passes9 < passes8 ? 9 : 8;
         k.passes = passes9 < passes8 ? passes9 : passes8;
+    }
+    if (frame_coarse_depth_ordered(f)) {
+        // (culled, the largest key, must fit the bits that are left)
+        while (k.end_bit - k.shift > kCoarseDepthBits || ((k.culled - 1u) >> k.shift) + 1u >= (1u << kCoarseDepthBits)) ++k.shift;
+        k.culled = ((k.culled - 1u) >> k.shift) + 1u;
+        k.end_bit = kCoarseDepthBits; k.digit_bits = kCoarseDepthBits; k.passes = 1;
     }
     return k;
 }

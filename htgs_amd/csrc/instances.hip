@@ -234,13 +234,20 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(uint32_t *p, size_t n, u
     if (i < kOrderWords && also_order) also_order[i] = 0;
 }
 
-// The order in which the blend kernels take the tiles: longest lists first.  One workgroup walks one tile, the hardware
-// hands out workgroups in index order, and lists differ in length by an order of magnitude; with the long ones at the
-// end of the launch a few compute units finish them while the rest of the device idles (blend of 3 M Gaussians at
-// 1080p: 1.43 ms in tile order, 1.30 ms longest first, 1.31 ms with the bins used here).  Tiles are binned by list
-// length, four bins per power of two, and laid out bin after bin (a counting sort; the order inside a bin is whatever
-// the atomics give, which no result depends on -- keeping it fixed costs 0.02 ms more and gains nothing).
+// The order in which the blend kernels take the tiles: longest lists first, in groups of neighbours.  One workgroup walks
+// one tile, the hardware hands out workgroups in index order, and lists differ in length by an order of magnitude; with
+// the long ones at the end of the launch a few compute units finish them while the rest of the device idles (blend of
+// 3 M Gaussians at 1080p: 1.43 ms in tile order, 1.30 ms longest first).  A Gaussian reaches several neighbouring
+// tiles, whose workgroups each fetch its record: the tiles are therefore ordered in groups of sixteen neighbours (a 4x4
+// patch: strips of four tile rows, gone through column by column, cut into runs of sixteen), and the workgroup index b
+// goes to the accelerator die b mod 8, each with a cache of its own, so a group is given the sixteen indices
+// 8 (16 p + t) + x, t = 0 .. 15: its tiles run on one die at about the same time and all but the first fetch of a
+// record hit that die's cache.  Groups are binned by the total length of their lists, four bins per power of two, and
+// laid out bin after bin (a counting sort; the order inside a bin is whatever the atomics give, which no result
+// depends on); the groups left over when their number is not a multiple of eight, and the tiles left over when theirs
+// is not a multiple of sixteen, follow at the end, one after the other.
 // order: [n_tiles] tiles, then kOrderBuckets bin totals and kOrderBuckets bin cursors, zeroed beforehand.
+constexpr uint32_t kOrderGroup = 16, kOrderStrip = 4, kOrderDies = 8;
 __device__ __forceinline__ uint32_t order_bucket(uint32_t length)
 {
     if (length == 0) return 129u;                          // empty lists last
@@ -248,25 +255,48 @@ __device__ __forceinline__ uint32_t order_bucket(uint32_t length)
     const uint32_t sub = p >= 2u ? (length >> (p - 2u)) & 3u : (length << (2u - p)) & 3u;
     return 128u - (4u * p + sub);                          // 1 .. 128, longer lists first
 }
-__global__ void __launch_bounds__(256) tile_order_count_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t n_tiles)
+// the i-th tile in strip order
+__device__ __forceinline__ uint32_t strip_order_tile(uint32_t i, uint32_t grid_w, uint32_t grid_h)
+{
+    const uint32_t per_strip = kOrderStrip * grid_w, full = grid_h / kOrderStrip * per_strip;
+    if (i < full) {
+        const uint32_t strip = i / per_strip, r = i % per_strip;
+        return (kOrderStrip * strip + r % kOrderStrip) * grid_w + r / kOrderStrip;
+    }
+    const uint32_t rows = grid_h % kOrderStrip, r = i - full;
+    return (grid_h - rows + r % rows) * grid_w + r / rows;
+}
+__device__ __forceinline__ uint32_t order_group_length(const uint32_t *__restrict__ ranges, uint32_t group, uint32_t grid_w, uint32_t grid_h)
+{
+    uint32_t length = 0;
+    for (uint32_t t = 0; t < kOrderGroup; ++t) {
+        const uint32_t tile = strip_order_tile(kOrderGroup * group + t, grid_w, grid_h);
+        length += ranges[2 * tile + 1] - ranges[2 * tile];
+    }
+    return length;
+}
+__global__ void __launch_bounds__(256) tile_order_count_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t grid_w,
+                                                               uint32_t grid_h)
 {
     __shared__ uint32_t count[kOrderBuckets];
     if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
     __syncthreads();
-    const uint32_t tile = blockIdx.x * 256 + threadIdx.x;
-    if (tile < n_tiles) atomicAdd(&count[order_bucket(ranges[2 * tile + 1] - ranges[2 * tile])], 1u);
+    const uint32_t n_tiles = grid_w * grid_h, group = blockIdx.x * 256 + threadIdx.x;
+    if (group < n_tiles / kOrderGroup) atomicAdd(&count[order_bucket(order_group_length(ranges, group, grid_w, grid_h))], 1u);
     __syncthreads();
     if (threadIdx.x < kOrderBuckets && count[threadIdx.x]) atomicAdd(order + n_tiles + threadIdx.x, count[threadIdx.x]);
 }
-__global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t n_tiles)
+__global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t grid_w,
+                                                               uint32_t grid_h)
 {
     __shared__ uint32_t count[kOrderBuckets], total[kOrderBuckets], base[kOrderBuckets];
+    const uint32_t n_tiles = grid_w * grid_h, n_groups = n_tiles / kOrderGroup;
     if (threadIdx.x < kOrderBuckets) { count[threadIdx.x] = 0; total[threadIdx.x] = order[n_tiles + threadIdx.x]; }
     __syncthreads();
-    const uint32_t tile = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t group = blockIdx.x * 256 + threadIdx.x;
     uint32_t bucket = 0, rank = 0;
-    if (tile < n_tiles) {
-        bucket = order_bucket(ranges[2 * tile + 1] - ranges[2 * tile]);
+    if (group < n_groups) {
+        bucket = order_bucket(order_group_length(ranges, group, grid_w, grid_h));
         rank = atomicAdd(&count[bucket], 1u);
     }
     __syncthreads();
@@ -277,7 +307,15 @@ __global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *_
         base[threadIdx.x] = start + atomicAdd(order + n_tiles + kOrderBuckets + threadIdx.x, count[threadIdx.x]);
     }
     __syncthreads();
-    if (tile < n_tiles) order[base[bucket] + rank] = tile;
+    if (group < n_groups) {
+        const uint32_t place = base[bucket] + rank, interleaved = n_groups / kOrderDies * kOrderDies;
+        for (uint32_t t = 0; t < kOrderGroup; ++t) {
+            const uint32_t at = place < interleaved ? kOrderDies * (kOrderGroup * (place / kOrderDies) + t) + place % kOrderDies : kOrderGroup * place + t;
+            order[at] = strip_order_tile(kOrderGroup * group + t, grid_w, grid_h);
+        }
+    } else if (group == n_groups) {
+        for (uint32_t i = kOrderGroup * n_groups; i < n_tiles; ++i) order[i] = strip_order_tile(i, grid_w, grid_h);
+    }
 }
 
 // Scratch of htgs_scan_offsets_static: the per-block sums of the scan, held in the library's own device image so
@@ -463,9 +501,10 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
             hipLaunchKernelGGL((extract_ranges_kernel<uint16_t, 0>), grid, block, 0, s, (const uint16_t *)f->keys[selector], f->ranges, f->n_instances);
     }
     if (f->tile_order) {
-        const dim3 grid((unsigned)((n_tiles + 255) / 256)), block(256);
-        hipLaunchKernelGGL(tile_order_count_kernel, grid, block, 0, s, f->ranges, f->tile_order, (uint32_t)n_tiles);
-        hipLaunchKernelGGL(tile_order_place_kernel, grid, block, 0, s, f->ranges, f->tile_order, (uint32_t)n_tiles);
+        const uint32_t grid_w = (uint32_t)div_up(f->width, tile), grid_h = (uint32_t)div_up(f->height, tile);
+        const dim3 grid((unsigned)((n_tiles / kOrderGroup + 1 + 255) / 256)), block(256);
+        hipLaunchKernelGGL(tile_order_count_kernel, grid, block, 0, s, f->ranges, f->tile_order, grid_w, grid_h);
+        hipLaunchKernelGGL(tile_order_place_kernel, grid, block, 0, s, f->ranges, f->tile_order, grid_w, grid_h);
     }
     return check_launch("extract_ranges");
 }

@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     uint8_t *__restrict__ clamp_info,
     int n, uint32_t grid_w, uint32_t grid_h, float tile, float min_alpha_rcp,
     int active_sh, int total_sh, float near_plane, float far_plane, float scale_modifier, int rec4,
-    uint32_t *__restrict__ depth_keys, uint32_t *__restrict__ depth_vals, uint32_t depth_base, uint32_t depth_culled)
+    uint32_t *__restrict__ depth_keys, uint32_t *__restrict__ depth_vals, uint32_t depth_base, uint32_t depth_culled, int depth_shift)
 {
     // One LDS buffer, used twice: first the block's slice of sh_rest (contiguous in memory, loaded with coalesced
     // 16-byte reads and then read back per Gaussian at a stride of 3 * total_sh words), then the block's records
@@ -156,7 +156,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     if (depth_keys != nullptr && in_range) {
         // (a depth that is not a number passes the cull above, as in the reference, where its bit pattern sorts behind every
         // valid depth; here its key is held below `culled`, so it is neither dropped nor sorted by bits that the sort ignores)
-        const uint32_t key = float_to_bits(z) - depth_base;
+        const uint32_t key = (float_to_bits(z) - depth_base) >> depth_shift;
         depth_keys[i] = touched != 0 ? (key < depth_culled - 1u ? key : depth_culled - 1u) : depth_culled;
         depth_vals[i] = (uint32_t)i;
     }
@@ -275,6 +275,6 @@ extern "C" int htgs_preprocess(const htgs_frame *f)
                        f->positions, f->scales, f->rotations, f->opacities, f->sh_0, f->sh_rest, f->M, f->VPM, f->cam_position,
                        f->n_touched, f->bounds, f->prim, f->clamp_info, f->n_primitives, grid_w, grid_h, (float)tile,
                        min_alpha_rcp, f->active_sh_bases, f->total_sh_bases, f->near_plane, f->far_plane, f->scale_modifier, prim_floats / 4,
-                       ordered ? order.keys[0] : nullptr, ordered ? order.vals[0] : nullptr, order_keys.base, order_keys.culled);
+                       ordered ? order.keys[0] : nullptr, ordered ? order.vals[0] : nullptr, order_keys.base, order_keys.culled, order_keys.shift);
     return check_launch("preprocess");
 }

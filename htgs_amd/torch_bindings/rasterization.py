@@ -206,9 +206,11 @@ class FrameBuffers:
         self.tile_order = (self._scratch("tile_order", self.lib.htgs_tile_order_words(mode, self.width, self.height), torch.int32)
                            if order_tiles else None)
         # GLOBAL_ORDERING inference: the Gaussians sorted by depth before the instances are made, whose keys then hold the
-        # tile alone (two sort passes over 2-byte keys instead of five over 8-byte keys, the same sorted list)
+        # tile alone (two sort passes over 2-byte keys instead of five over 8-byte keys, the same sorted list).  The
+        # image-only fast path of the two modes with a sorted core: the same with coarse depth keys (one pass), so that a
+        # tile's fragments arrive roughly front to back and few of them have to be inserted in front of others
         self.depth_order = (self._scratch("depth_order", self.lib.htgs_depth_order_words(n), torch.int32)
-                            if order_gaussians and mode == 2 and not train else None)
+                            if order_gaussians and not train and (mode == 2 or (fast and mode in (0, 1))) else None)
         self.image = torch.empty((3, self.height, self.width) if to_chw else (self.height, self.width, 3),
                                  dtype=torch.float32, device=dev)
         # the image-only fast path (``fast_rasterize``) writes no depth map

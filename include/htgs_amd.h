@@ -101,7 +101,12 @@ typedef struct htgs_frame {
                                   the instances in it, with keys that hold the tile alone: the stable sort by tile that
                                   follows leaves every tile's list in the order of the reference's sort by tile | depth
                                   (same sorted vals, same ranges) in two passes over 2-byte keys instead of five over
-                                  8-byte keys.  NULL: the reference's keys (no counterpart in the reference) */
+                                  8-byte keys.  NULL: the reference's keys (no counterpart in the reference).
+                                  HYBRID_BLEND and ALPHA_BLEND_FIRST_K with fast_math set (htgs_preprocess reads it then):
+                                  the same with the depth keys cut to nine bits, one pass -- every tile's list holds the
+                                  instances of the reference's list, roughly front to back instead of by Gaussian
+                                  index, which the image-only blend does not mind and which spares it most insertions
+                                  into the sorted core.  Ignored in the other cases */
     /* ---- per-instance scratch (PerInstanceBuffers, buffer_utils.h:56-84) ---- */
     uint64_t n_instances;      /* host copy of *n_instances_dev, needed from htgs_create_instances on */
     void *keys[2];             /* [n_instances] of htgs_frame_key_bytes() each, ping-pong, 16-byte aligned */
@@ -112,9 +117,10 @@ typedef struct htgs_frame {
     float *depth;              /* [H,W] */
     int32_t to_chw;
     int32_t use_median_depth;
-    int32_t fast_math;         /* htgs_blend only: image-only variant with the hardware's reciprocal and 2^x (one ulp each)
+    int32_t fast_math;         /* htgs_blend: image-only variant with the hardware's reciprocal and 2^x (one ulp each)
                                   instead of the exactly reproducible routines; depth is not written and may be NULL
-                                  (the reference's fast_inference kernels, <mode>/kernels/fast_inference.cuh) */
+                                  (the reference's fast_inference kernels, <mode>/kernels/fast_inference.cuh).  The
+                                  stages before it read it only to tell what depth_order is for */
     /* ---- training: per-pixel records (PerPixelBuffers, buffer_utils.h:96-108).  Written by the forward blend, read by the
      * backward blend, opaque to the caller.  R = 64 * n_tiles entries per plane, tile by tile: entry 64 * tile +
      * 8 * (y & 7) + (x & 7) belongs to pixel (x, y), so that a tile's 64 pixels are contiguous ---- */

@@ -135,3 +135,38 @@ def test_depth_that_is_not_a_number_sorts_behind_the_valid_ones(cuda):
         np.testing.assert_array_equal(got["sorted_vals"], keyed["sorted_vals"])
         np.testing.assert_array_equal(got["ranges"], keyed["ranges"])
         assert np.array_equal(got["image"], keyed["image"], equal_nan=True)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("config,n", [(0, 5000), (1, 60_000), (3, 60_000)])
+def test_fast_path_lists_are_the_reference_lists_roughly_front_to_back(cuda, config, n, mode):
+    """The image-only fast path of the two modes with a sorted core sorts the Gaussians by nine bits of their depth keys
+    before the instances are made: every tile's list must hold exactly the instances of the oracle's list, and along a
+    list the depths may fall only by what one step of the coarse keys is worth (a key step is at most 2^18 steps of the
+    depth's bit pattern for near / far planes within the usual nine powers of two, 3.2 % of the depth)."""
+    print(f"case config={config} n={n} mode={mode}", flush=True)
+    scene = make_scene(config, n)
+    ref = oracle_render(scene, mode, 16)
+    sg = scene.to(cuda)
+    fb = FrameBuffers(*sg.gaussians(), sg.settings(RasterizerMode(mode), 16), True, False, fast=True)
+    assert fb.depth_order is not None
+    fb.run()
+    torch.cuda.synchronize()
+    exact = FrameBuffers(*sg.gaussians(), sg.settings(RasterizerMode(mode), 16), True, False)
+    assert exact.depth_order is None                                   # the exact path keeps the reference's order
+    from util import u32
+    assert fb.lib.htgs_frame_depth_sort_passes(fb._ref) == 1
+    ranges = u32(fb.ranges).astype(np.int64)
+    np.testing.assert_array_equal(ranges, ref["ranges"])
+    vals = u32(fb.vals[fb.selector])[:fb.n_instances].astype(np.int64)
+    assert len(vals) == len(ref["sorted_vals"])
+    depth = ref["pre"]["MT3"][:, 3].astype(np.float64)                 # camera-space depth of the centre
+    worst = 0.0
+    for a, b in ranges[ranges[:, 1] > ranges[:, 0]]:
+        assert np.array_equal(np.sort(vals[a:b]), ref["sorted_vals"][a:b].astype(np.int64))
+        d = depth[vals[a:b]]
+        worst = max(worst, float(np.max(np.maximum.accumulate(d) / d)))
+    assert worst <= 1.07
+    image = fb.image.cpu().numpy()
+    diff = np.abs(image - ref["image"])
+    assert float((diff > 1e-5).mean()) < 1e-3 and float(diff.max()) <= 5e-2

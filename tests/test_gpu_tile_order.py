@@ -1,5 +1,7 @@
-"""``htgs_extract_ranges`` also writes the order in which the blend kernels take the tiles: longest lists first, binned by
-length with four bins per power of two.  The order must be a permutation of the tiles with non-increasing bins, and no
+"""``htgs_extract_ranges`` also writes the order in which the blend kernels take the tiles: groups of sixteen neighbouring
+tiles (strips of four tile rows, column by column, cut into runs of sixteen), the groups with the longest lists first,
+binned by total length with four bins per power of two, and a group's tiles at the workgroup indices that one
+accelerator die is given (8 (16 p + t) + x).  The order must be a permutation of the tiles with that structure, and no
 result may depend on it."""
 import numpy as np
 import pytest
@@ -20,6 +22,16 @@ def length_bin(length: np.ndarray) -> np.ndarray:
     return np.where(length > 0, 4 * p + sub + 1, 0)
 
 
+def strip_order(grid_w: int, grid_h: int) -> np.ndarray:
+    """the tiles, strip by strip of four tile rows, column by column inside a strip"""
+    out = []
+    for y0 in range(0, grid_h, 4):
+        rows = min(4, grid_h - y0)
+        for x in range(grid_w):
+            out.extend((y0 + r) * grid_w + x for r in range(rows))
+    return np.array(out, np.int64)
+
+
 @pytest.mark.parametrize("config,n,mode", [(0, 10_000, 0), (1, 60_000, 0), (1, 60_000, 2), (3, 40_000, 0), (0, 0, 0)])
 def test_order_is_a_permutation_with_the_longest_lists_first(cuda, config, n, mode):
     print(f"case config={config} n={n} mode={mode}", flush=True)
@@ -33,8 +45,25 @@ def test_order_is_a_permutation_with_the_longest_lists_first(cuda, config, n, mo
     order = u32(fb.tile_order)[:fb.n_tiles].astype(np.int64)
     assert np.array_equal(np.sort(order), np.arange(fb.n_tiles))
     ranges = u32(fb.ranges).astype(np.int64)
-    bins = length_bin(ranges[order, 1] - ranges[order, 0])
-    assert (np.diff(bins) <= 0).all()
+    length = ranges[:, 1] - ranges[:, 0]
+    tile = 16 if mode == 2 else 8
+    grid_w, grid_h = -(-fb.width // tile), -(-fb.height // tile)
+    strip = strip_order(grid_w, grid_h)
+    assert np.array_equal(np.sort(strip), np.arange(fb.n_tiles))
+    n_groups = fb.n_tiles // 16
+    interleaved = n_groups // 8 * 8
+    group_of_tile = np.empty(fb.n_tiles, np.int64)
+    group_of_tile[strip] = np.arange(fb.n_tiles) // 16
+    totals = []
+    for place in range(n_groups):
+        at = (8 * (16 * (place // 8) + np.arange(16)) + place % 8) if place < interleaved else 16 * place + np.arange(16)
+        tiles = order[at]
+        group = group_of_tile[tiles[0]]
+        assert np.array_equal(tiles, strip[16 * group:16 * group + 16])        # one group, its tiles in strip order
+        totals.append(length[tiles].sum())
+    assert np.array_equal(order[16 * n_groups:], strip[16 * n_groups:])          # the tiles that fill no group
+    if totals:
+        assert (np.diff(length_bin(np.array(totals))) <= 0).all()
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
