@@ -246,12 +246,13 @@ enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2, kCullPixels = 3 };
 // With QUADRANTS the result has one bit per 4x4 quadrant of the tile (tile_quadrant_hits) instead of one for the tile.
 // REC4: 16-byte words per record of prim (five; eight in training frames).
 // UNIT: the opacity is staged held to at most 1 (the image-only fast path, whose fragments then need no clamp of their own).
-template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false>
+// POS: the last word of the slot holds the instance's place in the list (fetch) instead of the Gaussian's index.
+template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, bool POS = false>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                     uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes = 0);
 
 // (PixelTerms is complete by the time the template is instantiated)
-template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS, int REC4, bool UNIT>
+template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS, int REC4, bool UNIT, bool POS>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                     uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes)
 {
@@ -305,7 +306,7 @@ __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const floa
     }
     if (UNIT) col.w = col.w < 1.0f ? col.w : 1.0f;
     st.q[4][slot] = make_float4(zxy, zyy, r3.w, col.w);
-    st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(g));
+    st.q[5][slot] = make_float4(col.x, col.y, col.z, bits_to_float(POS ? fetch : g));
     if constexpr (CULL == kCullNone) return QUADRANTS ? 0xfu : 1u;
     else if constexpr (CULL == kCullPixels) {
         static_assert(QUADRANTS, "per quadrant");
@@ -481,14 +482,14 @@ __device__ __forceinline__ void quadrant_list_walk(const QuadrantLists &ql, uint
 // The walk over instances [first, last) of a tile's list (whole batches of 64 from `first` on) by one wave, lanes =
 // pixels by quadrants: every batch is staged (tile_stage_load with the CULL asked for), its quadrant lists are built and
 // turn(addr) is called for every turn.  SOLO: the wave is the whole workgroup (its barriers are the workgroup's).
-template <int MODE, bool DEPTH, int CULL, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, typename Turn>
+template <int MODE, bool DEPTH, int CULL, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, bool POS = false, typename Turn>
 __device__ __forceinline__ void tile_list_walk(TileStageQ &st, QuadrantLists &ql, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                uint32_t first, uint32_t last, uint32_t lane, float cx, float cy, Turn &&turn, uint64_t pixel_lanes = 0)
 {
     stage_dummy_init(st, lane);
     for (uint32_t base = first; base < last; base += 64) {
         if (SOLO) __syncthreads(); else wave_lds_sync();
-        const uint32_t bits = tile_stage_load<MODE, kStageSlots, DEPTH, CULL, true, REC4, UNIT>(st, prim, inst, base + lane, last, lane + 1, cx, cy, pixel_lanes);
+        const uint32_t bits = tile_stage_load<MODE, kStageSlots, DEPTH, CULL, true, REC4, UNIT, POS>(st, prim, inst, base + lane, last, lane + 1, cx, cy, pixel_lanes);
         const uint32_t n_turns = quadrant_lists_build(ql, bits, lane, st);
         if (SOLO) __syncthreads(); else wave_lds_sync();
         // lanes outside the image run along (their results are never stored): the loop stays wave-uniform

@@ -95,6 +95,84 @@ __device__ __forceinline__ void hybrid_walk(TileStageQ &st, QuadrantLists &ql, c
     }, pixel_lanes);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The image-only fast path's core as sorted 64-bit keys (the kernel with one wave per tile).  A slot is one register
+// pair: the high word holds the depth, the low word alpha as a 19-bit fraction (an absolute error of 2^-20) above the
+// instance's place in the tile's list (13 bits: the lists this kernel walks are no longer than the threshold beyond
+// which a tile goes to the other kernel, at most kPackedListMost).  Positive floats order like their bit patterns and
+// so do the doubles made of (depth, low word): one step of the insertion is slot' = min(carried, slot), carried' =
+// max(carried, slot), two instructions without exec masks or moves, and what is pushed out carries the alpha that the
+// tail needs.  The Gaussian's index, which only the final core needs, is looked up from the place in the list when the
+// pixel is composited.  (Which of two fragments of equal depth comes first is decided by the low word here, which this
+// path does not promise to reproduce; depths that are not positive numbers would order differently from floats.)
+// ---------------------------------------------------------------------------------------------
+typedef double CoreKey;
+constexpr uint32_t kPackedListMost = 8192, kPackedAlphaOne = (1u << 19) - 1u;
+__device__ __forceinline__ float key_depth(CoreKey k) { return bits_to_float((uint32_t)__double2hiint(k)); }
+__device__ __forceinline__ uint32_t key_low(CoreKey k) { return (uint32_t)__double2loint(k); }
+__device__ __forceinline__ CoreKey make_key(float depth, uint32_t low) { return __hiloint2double((int)float_to_bits(depth), (int)low); }
+__device__ __forceinline__ uint32_t key_pack(float alpha, uint32_t place)      // alpha in [0, 1]
+{
+    return (uint32_t)__builtin_fmaf(alpha, (float)kPackedAlphaOne, 0.5f) << 13 | place;
+}
+__device__ __forceinline__ float key_alpha(uint32_t low) { return (float)(low >> 13) * (1.0f / (float)kPackedAlphaOne); }
+__device__ __forceinline__ void key_step(CoreKey &carried, CoreKey &slot)
+{
+    CoreKey out;
+    asm("v_max_f64 %0, %2, %1\n\tv_min_f64 %1, %2, %1" : "=&v"(out), "+v"(slot) : "v"(carried));
+    carried = out;
+}
+template <int K>
+__device__ __forceinline__ void core_key_walk(CoreKey &carried, CoreKey (&core)[K])
+{
+#pragma unroll
+    for (int g0 = 0; g0 < K; g0 += kInsertGroup) {
+        const int g1 = g0 + kInsertGroup < K ? g0 + kInsertGroup : K;
+        if (K > kInsertGroup && !__any(key_depth(carried) < key_depth(core[g1 - 1]))) continue;
+#pragma unroll
+        for (int i = g0; i < g1; ++i) key_step(carried, core[i]);
+    }
+}
+template <int K, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4>
+__device__ __forceinline__ void hybrid_fast_key_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+                                                     uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy,
+                                                     CoreKey (&core)[K], HybridTail &tail)
+{
+    constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
+    constexpr int N = kStageSlots;
+    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4, true, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool fragment = tile_frag_fast<MODE, N>(addr, pt, f);
+        const float4 col = stage_row<N, 5>(addr);
+        if (!fragment) return;
+        float depth = tile_frag_depth<N>(addr, pt, f);
+        float p3 = f.alpha;
+        tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
+        tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
+        tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
+        if (depth < key_depth(core[K - 1]) && f.alpha >= kMinAlphaCore) {
+            CoreKey carried = make_key(depth, key_pack(p3, float_to_bits(col.w) - first));
+            core_key_walk<K>(carried, core);
+            depth = key_depth(carried);
+            p3 = key_alpha(key_low(carried));
+        }
+        hybrid_tail_add<true>(tail, depth, p3);
+    });
+}
+// the finished keys as the three arrays the composite takes
+template <int K>
+__device__ __forceinline__ void key_core_unpack(const CoreKey (&core)[K], const uint32_t *__restrict__ inst, uint32_t first, uint32_t last, float (&cd)[K],
+                                                float (&ca)[K], float (&ci)[K])
+{
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const uint32_t low = key_low(core[i]), place = low & (kPackedListMost - 1u);
+        cd[i] = key_depth(core[i]);
+        ca[i] = key_alpha(low);
+        ci[i] = ca[i] > 0.0f && first + place < last ? bits_to_float(inst[first + place]) : 0.0f;
+    }
+}
+
 // core + tail -> pixel (R/include/hybrid_blend/kernels/inference.cuh:172-213)
 template <int K, int REC4 = HTGS_PRIM_FLOATS / 4>
 __device__ __forceinline__ void hybrid_composite(const float4 *__restrict__ prim, float (&cd)[K], float (&ca)[K], float (&ci)[K], HybridTail &tail,
@@ -260,7 +338,8 @@ __device__ __forceinline__ bool long_part_done(const uint32_t *long_tiles, uint3
 }
 
 // One wave per tile; the tiles with very long lists are left to blend_hybrid_long_kernel.
-template <int K, bool FAST>
+// KEYS (the fast path, with long_tiles and a threshold of no more than kPackedListMost): the core as sorted 64-bit keys.
+template <int K, bool FAST, bool KEYS = false>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
@@ -279,9 +358,22 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     HybridTail tail;
     hybrid_tail_init(tail);
     float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
-    hybrid_core_init<K>(cd, ca, ci);
-    hybrid_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
-    if (!px.inside) return;
+    if constexpr (KEYS) {
+        static_assert(FAST, "the image-only path");
+        CoreKey core[K];
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            core[i] = make_key(__FLT_MAX__, 0u);
+            asm volatile("" : "+v"(core[i]));      // one register pair per slot, never a wide tuple
+        }
+        hybrid_fast_key_walk<K, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail);
+        if (!px.inside) return;
+        key_core_unpack<K>(core, inst, first, last, cd, ca, ci);
+    } else {
+        hybrid_core_init<K>(cd, ca, ci);
+        hybrid_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
+        if (!px.inside) return;
+    }
     hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
 }
 
