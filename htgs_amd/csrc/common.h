@@ -110,6 +110,11 @@ inline DepthKeys depth_key_range(const htgs_frame *f)
 // the result is in keys / vals[*selector]
 int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int digit_bits,
                    int *selector);
+// the same in one pass over keys of at most nine bits whose values are 0 .. n - 1 in this order, from keys / vals[0] to
+// keys / vals[1]; the tile rectangles (four 16-bit bounds per value) are written in sorted order as well, with the number
+// of tiles each covers (0 for the key `culled`)
+int sort_u32_pairs_with_rectangles(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int bits,
+                                   const uint16_t *rectangles_in, uint16_t *rectangles_out, uint32_t *counts_out, uint32_t culled);
 
 // host side error reporting (api.hip)
 int fail(int code, const char *fmt, ...);

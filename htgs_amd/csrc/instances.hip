@@ -367,10 +367,16 @@ static int launch_scan(const htgs_frame *f, uint32_t *tile_sums, const char *who
         if ((uintptr_t)f->depth_order & 15) return fail(HTGS_ERR_ARGUMENT, "%s: depth_order must be 16-byte aligned", who);
         const DepthOrder d = depth_order_parts(f);       // (htgs_preprocess has written the pairs to sort)
         const DepthKeys k = depth_key_range(f);
-        int sel = 0;
-        const int rc = sort_u32_pairs(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n, k.end_bit, k.digit_bits, &sel);
-        if (rc != HTGS_OK) return rc;
-        hipLaunchKernelGGL(gather_counts_kernel, dim3(div_up(n, 256)), dim3(256), 0, s, d.vals[sel], d.keys[sel], f->bounds, d.counts, d.bounds, n, k.culled);
+        if (k.passes == 1 && k.digit_bits == 9) {
+            // (one pass: the rectangles and the counts travel with the pairs)
+            const int rc = sort_u32_pairs_with_rectangles(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n, k.end_bit, f->bounds, d.bounds, d.counts, k.culled);
+            if (rc != HTGS_OK) return rc;
+        } else {
+            int sel = 0;
+            const int rc = sort_u32_pairs(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n, k.end_bit, k.digit_bits, &sel);
+            if (rc != HTGS_OK) return rc;
+            hipLaunchKernelGGL(gather_counts_kernel, dim3(div_up(n, 256)), dim3(256), 0, s, d.vals[sel], d.keys[sel], f->bounds, d.counts, d.bounds, n, k.culled);
+        }
         counts = d.counts;
     }
     if (tiles > 0) {

@@ -105,10 +105,16 @@ __global__ void __launch_bounds__(kScanThreads) digit_row_scan_kernel(uint32_t *
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = SortDigit<KeyT>::bits>
+// RECTANGLES (a sort of one pass over the Gaussians, whose values are their indices in the order of the input): the
+// Gaussians' tile rectangles, four 16-bit bounds each, travel with the pairs -- read in the order of the input, which is
+// theirs, written in sorted order, with the number of tiles each covers beside them (none for the key `culled`, whose
+// rectangle was never written).
+template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = SortDigit<KeyT>::bits, bool RECTANGLES = false>
 __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
     const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
-    const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask)
+    const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask,
+    const uint2 *__restrict__ rectangles_in = nullptr, uint2 *__restrict__ rectangles_out = nullptr, uint32_t *__restrict__ counts_out = nullptr,
+    uint32_t culled = 0)
 {
     constexpr int kSortThreads = THREADS, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
     constexpr int kBits = BITS, kRadix = 1 << kBits, kDigitWaves = kRadix / kWave;
@@ -227,8 +233,30 @@ __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
             const uint32_t d = digit_of(k, shift, mask);
             const uint32_t pos = global_base[d] + (i - digit_start[d]);
             keys_out[pos] = k;
-            if (kTwoRounds) digits[r / 2] |= d << (16 * (r % 2));
-            else vals_out[pos] = local_vals[i];
+            if (kTwoRounds || RECTANGLES) digits[r / 2] |= d << (16 * (r % 2));
+            if (!kTwoRounds) vals_out[pos] = local_vals[i];
+        }
+    }
+    if constexpr (RECTANGLES) {
+        static_assert(!kTwoRounds && sizeof(KeyT) == 4, "the rectangles take the room of the keys and the values");
+        uint2 *local_rectangles = reinterpret_cast<uint2 *>(local_raw);
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kSortItems; ++r) {
+            const uint64_t i = wave_base + (uint64_t)r * kWave + lane;
+            if (i < n) local_rectangles[rank[r]] = key[r] == (KeyT)culled ? make_uint2(0u, 0u) : rectangles_in[i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < kSortItems; ++r) {
+            const uint32_t i = (uint32_t)r * kSortThreads + threadIdx.x;
+            if (i < n_local) {
+                const uint32_t d = digits[r / 2] >> (16 * (r % 2)) & 0xffffu;
+                const uint32_t pos = global_base[d] + (i - digit_start[d]);
+                const uint2 b = local_rectangles[i];                 // x0 | x1 << 16, y0 | y1 << 16
+                rectangles_out[pos] = b;
+                counts_out[pos] = ((b.x >> 16) - (b.x & 0xffffu)) * ((b.y >> 16) - (b.y & 0xffffu));
+            }
         }
     }
     if (kTwoRounds) {
@@ -271,6 +299,24 @@ static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2
         cur ^= 1;
     }
     *selector = cur;
+    return check_launch("sort");
+}
+
+int sort_u32_pairs_with_rectangles(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int bits,
+                                   const uint16_t *rectangles_in, uint16_t *rectangles_out, uint32_t *counts_out, uint32_t culled)
+{
+    if (n == 0) return HTGS_OK;
+    if (bits < 1 || bits > 9) return fail(HTGS_ERR_ARGUMENT, "sort: one pass takes at most nine bits");
+    constexpr int kThreads = 512, kBits = 9, kRadix = 1 << kBits, kTile = kThreads * kSortItems;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t n_blocks = (uint32_t)((n + kTile - 1) / kTile);
+    uint32_t *hist = sort_tmp, *totals = sort_tmp + (size_t)kRadix * n_blocks;
+    const uint32_t mask = (1u << bits) - 1u;
+    hipLaunchKernelGGL((digit_histogram_kernel<uint32_t, kThreads, kBits>), dim3(xcd_padded_grid(n_blocks)), dim3(kThreads), 0, s, keys[0], hist, n, n_blocks, 0, mask);
+    hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
+    hipLaunchKernelGGL((digit_scatter_kernel<uint32_t, kThreads, kBits, true>), dim3(xcd_padded_grid(n_blocks)), dim3(kThreads), 0, s, keys[0], vals[0], keys[1],
+                       vals[1], hist, totals, n, n_blocks, 0, mask, reinterpret_cast<const uint2 *>(rectangles_in), reinterpret_cast<uint2 *>(rectangles_out),
+                       counts_out, culled);
     return check_launch("sort");
 }
 
