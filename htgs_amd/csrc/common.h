@@ -76,12 +76,12 @@ inline DepthOrder depth_order_parts(const htgs_frame *f)
 // patterns order like the depths; these are the low 32 bits of the reference's tile | depth keys) less that of the near
 // plane, which no Gaussian that is not culled lies in front of, `culled` for a culled Gaussian (behind all others).  With
 // the far plane as the upper bound the keys of the usual cameras have 27 bits: three passes of 9-bit digits.
-// Coarse keys (frame_coarse_depth_ordered): the same keys shifted down until nine bits are left, one pass.
+// Coarse keys (frame_coarse_depth_ordered): the same keys shifted down until eight bits are left, one pass.
 struct DepthKeys {
     uint32_t base, culled;
     int end_bit, digit_bits, passes, shift;
 };
-constexpr int kCoarseDepthBits = 9;
+constexpr int kCoarseDepthBits = 8;
 inline DepthKeys depth_key_range(const htgs_frame *f)
 {
     DepthKeys k = { 0u, 0xffffffffu, 32, 8, 4, 0 };
@@ -110,7 +110,7 @@ inline DepthKeys depth_key_range(const htgs_frame *f)
 // the result is in keys / vals[*selector]
 int sort_u32_pairs(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int digit_bits,
                    int *selector);
-// the same in one pass over keys of at most nine bits whose values are 0 .. n - 1 in this order, from keys / vals[0] to
+// the same in one pass over keys of at most eight bits whose values are 0 .. n - 1 in this order, from keys / vals[0] to
 // keys / vals[1]; the tile rectangles (four 16-bit bounds per value) are written in sorted order as well, with the number
 // of tiles each covers (0 for the key `culled`)
 int sort_u32_pairs_with_rectangles(void *stream, uint32_t *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int bits,

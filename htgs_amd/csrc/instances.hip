@@ -367,7 +367,7 @@ static int launch_scan(const htgs_frame *f, uint32_t *tile_sums, const char *who
         if ((uintptr_t)f->depth_order & 15) return fail(HTGS_ERR_ARGUMENT, "%s: depth_order must be 16-byte aligned", who);
         const DepthOrder d = depth_order_parts(f);       // (htgs_preprocess has written the pairs to sort)
         const DepthKeys k = depth_key_range(f);
-        if (k.passes == 1 && k.digit_bits == 9) {
+        if (k.passes == 1 && k.end_bit <= 8) {
             // (one pass: the rectangles and the counts travel with the pairs)
             const int rc = sort_u32_pairs_with_rectangles(f->stream, d.keys, d.vals, d.sort_tmp, (uint64_t)n, k.end_bit, f->bounds, d.bounds, d.counts, k.culled);
             if (rc != HTGS_OK) return rc;

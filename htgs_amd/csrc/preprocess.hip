@@ -99,7 +99,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     for (int k = 0; k < kShRegs; ++k) {
         const int q = k * 256 + threadIdx.x;
         float4 t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (q < words / 4) t = src4[q];
+        if (q < words / 4) {
+            // (read once per frame and 576 MB on a scene of 3 M Gaussians: marked as streaming, so that it does not push the
+            // records and lists the later stages come back to out of the last-level cache)
+            typedef float streamed_float4 __attribute__((ext_vector_type(4)));
+            const streamed_float4 v = __builtin_nontemporal_load(reinterpret_cast<const streamed_float4 *>(src4 + q));
+            t = make_float4(v.x, v.y, v.z, v.w);
+        }
         sh_regs[k][0] = t.x; sh_regs[k][1] = t.y; sh_regs[k][2] = t.z; sh_regs[k][3] = t.w;
     }
 

@@ -146,8 +146,9 @@ __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
     for (int r = 0; r < kSortItems; ++r) {
         const uint64_t i = wave_base + (uint64_t)r * kWave + lane;
         const bool valid = i < n;
-        key[r] = valid ? keys_in[i] : (KeyT)0;
-        val[r] = valid ? vals_in[i] : 0u;
+        // (the last reads of these buffers before they are written again: streaming, nothing to keep in the caches)
+        key[r] = valid ? __builtin_nontemporal_load(keys_in + i) : (KeyT)0;
+        val[r] = valid ? __builtin_nontemporal_load(vals_in + i) : 0u;
         const uint32_t d = digit_of(key[r], shift, mask);
         // lanes of this wave holding the same digit: per digit bit, keep the lanes whose bit equals this lane's.
         // (bit as 0 / ~0 by a signed bit-field extract; keep = peers & ~(vote ^ bit) is one three-input operation per half)
@@ -306,8 +307,9 @@ int sort_u32_pairs_with_rectangles(void *stream, uint32_t *const keys[2], uint32
                                    const uint16_t *rectangles_in, uint16_t *rectangles_out, uint32_t *counts_out, uint32_t culled)
 {
     if (n == 0) return HTGS_OK;
-    if (bits < 1 || bits > 9) return fail(HTGS_ERR_ARGUMENT, "sort: one pass takes at most nine bits");
-    constexpr int kThreads = 512, kBits = 9, kRadix = 1 << kBits, kTile = kThreads * kSortItems;
+    if (bits < 1 || bits > 8) return fail(HTGS_ERR_ARGUMENT, "sort: one pass takes at most eight bits");
+    // (blocks of 4096 items, the smallest the kernels take: a few million pairs are three rounds of such blocks)
+    constexpr int kThreads = kSortTileMin / kSortItems, kBits = 8, kRadix = 1 << kBits, kTile = kThreads * kSortItems;
     hipStream_t s = (hipStream_t)stream;
     const uint32_t n_blocks = (uint32_t)((n + kTile - 1) / kTile);
     uint32_t *hist = sort_tmp, *totals = sort_tmp + (size_t)kRadix * n_blocks;

@@ -103,7 +103,7 @@ typedef struct htgs_frame {
                                   (same sorted vals, same ranges) in two passes over 2-byte keys instead of five over
                                   8-byte keys.  NULL: the reference's keys (no counterpart in the reference).
                                   HYBRID_BLEND and ALPHA_BLEND_FIRST_K with fast_math set (htgs_preprocess reads it then):
-                                  the same with the depth keys cut to nine bits, one pass -- every tile's list holds the
+                                  the same with the depth keys cut to eight bits, one pass -- every tile's list holds the
                                   instances of the reference's list, roughly front to back instead of by Gaussian
                                   index, which the image-only blend does not mind and which spares it most insertions
                                   into the sorted core.  Ignored in the other cases */

@@ -140,10 +140,10 @@ def test_depth_that_is_not_a_number_sorts_behind_the_valid_ones(cuda):
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("config,n", [(0, 5000), (1, 60_000), (3, 60_000)])
 def test_fast_path_lists_are_the_reference_lists_roughly_front_to_back(cuda, config, n, mode):
-    """The image-only fast path of the two modes with a sorted core sorts the Gaussians by nine bits of their depth keys
+    """The image-only fast path of the two modes with a sorted core sorts the Gaussians by eight bits of their depth keys
     before the instances are made: every tile's list must hold exactly the instances of the oracle's list, and along a
-    list the depths may fall only by what one step of the coarse keys is worth (a key step is at most 2^18 steps of the
-    depth's bit pattern for near / far planes within the usual nine powers of two, 3.2 % of the depth)."""
+    list the depths may fall only by what one step of the coarse keys is worth (a key step is at most 2^19 steps of the
+    depth's bit pattern for near / far planes within the usual eight powers of two, 6.3 % of the depth)."""
     print(f"case config={config} n={n} mode={mode}", flush=True)
     scene = make_scene(config, n)
     ref = oracle_render(scene, mode, 16)
