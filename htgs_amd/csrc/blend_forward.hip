@@ -78,7 +78,7 @@ struct HybridRecords {
 #pragma unroll
         for (int i = 0; i < K; ++i) {
             const bool skip = !(c3[i] > 0.0f) || T_core < kTransmittanceThreshold;      // an empty slot has alpha 0
-            core_idx[(size_t)i * rnp + rp] = skip ? 0xffffffffu : float_to_bits(ci[i]);
+            __builtin_nontemporal_store(skip ? 0xffffffffu : float_to_bits(ci[i]), core_idx + ((size_t)i * rnp + rp));
             float4 info = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (!skip) {
                 const float bw = T_core * c3[i];
@@ -93,7 +93,10 @@ struct HybridRecords {
                 info.w = bw;
                 T_core *= oma;
             }
-            core_info[(size_t)i * rnp + rp] = info;
+            // (0.7 GB of records per frame at 1080p, read back once by the backward pass: streaming stores)
+            typedef float streamed_float4 __attribute__((ext_vector_type(4)));
+            streamed_float4 packed; packed.x = info.x; packed.y = info.y; packed.z = info.z; packed.w = info.w;
+            __builtin_nontemporal_store(packed, reinterpret_cast<streamed_float4 *>(core_info + ((size_t)i * rnp + rp)));
         }
         image[pix] = r + w0; image[np + pix] = g + w1; image[2 * np + pix] = b + w2;
     }
@@ -162,7 +165,7 @@ struct FirstKRecords {
 #pragma unroll
         for (int i = 0; i < K; ++i) {
             const bool skip = ci[i] == 0xffffffffu || T < kTransmittanceThreshold;
-            core_idx[(size_t)i * rnp + rp] = skip ? 0xffffffffu : ci[i];
+            __builtin_nontemporal_store(skip ? 0xffffffffu : ci[i], core_idx + ((size_t)i * rnp + rp));     // (streaming, as in HybridRecords)
             float4 info = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             if (!skip) {
                 const float bw = T * ca[i];
@@ -177,7 +180,9 @@ struct FirstKRecords {
                 info.w = bw;
                 T *= oma;
             }
-            core_info[(size_t)i * rnp + rp] = info;
+            typedef float streamed_float4 __attribute__((ext_vector_type(4)));
+            streamed_float4 packed; packed.x = info.x; packed.y = info.y; packed.z = info.z; packed.w = info.w;
+            __builtin_nontemporal_store(packed, reinterpret_cast<streamed_float4 *>(core_info + ((size_t)i * rnp + rp)));
         }
         image[pix] = r; image[np + pix] = g; image[2 * np + pix] = b;
     }

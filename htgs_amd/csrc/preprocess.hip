@@ -238,8 +238,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) p
     __syncthreads();
     float4 *dst4 = reinterpret_cast<float4 *>(prim) + (size_t)rec4 * first;
     if (rec4 == HTGS_PRIM_FLOATS / 4) {
+        typedef float streamed_float4 __attribute__((ext_vector_type(4)));
         for (int q = threadIdx.x; q < n_block * (HTGS_PRIM_FLOATS / 4); q += 256)
-            if (s_visible[q / (HTGS_PRIM_FLOATS / 4)]) dst4[q] = lds4[q];
+            if (s_visible[q / (HTGS_PRIM_FLOATS / 4)]) {
+                const float4 v = lds4[q];
+                streamed_float4 w; w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+                __builtin_nontemporal_store(w, reinterpret_cast<streamed_float4 *>(dst4 + q));
+            }
     } else {
         for (int q = threadIdx.x; q < n_block * (HTGS_PRIM_FLOATS_TRAIN / 4); q += 256)
             if (s_visible[q / (HTGS_PRIM_FLOATS_TRAIN / 4)]) dst4[q] = lds4[q];
