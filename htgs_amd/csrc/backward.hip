@@ -751,7 +751,12 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
         for (int k = 0; k < kShRegs; ++k) {
             const int q = k * 256 + threadIdx.x;
             float4 t = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            if (q < words / 4) t = src4[q];
+            if (q < words / 4) {
+                // (read once per step: streaming, as in the forward pass's preprocess)
+                typedef float streamed_float4 __attribute__((ext_vector_type(4)));
+                const streamed_float4 v = __builtin_nontemporal_load(reinterpret_cast<const streamed_float4 *>(src4 + q));
+                t = make_float4(v.x, v.y, v.z, v.w);
+            }
             sh_regs[k][0] = t.x; sh_regs[k][1] = t.y; sh_regs[k][2] = t.z; sh_regs[k][3] = t.w;
         }
     }
@@ -973,7 +978,13 @@ __global__ void __launch_bounds__(256) preprocess_backward_kernel(
         for (int k = 45; k < per; ++k) gsr[k] = 0.0f;
         __syncthreads();
         float4 *dst4 = reinterpret_cast<float4 *>(grad_sh_rest + base_word);
-        for (int q = threadIdx.x; q < words / 4; q += 256) dst4[q] = lds4[q];
+        // (the gradients leave for the optimizer; nothing of this step reads them again: streaming)
+        typedef float streamed_float4 __attribute__((ext_vector_type(4)));
+        for (int q = threadIdx.x; q < words / 4; q += 256) {
+            const float4 v = lds4[q];
+            streamed_float4 w; w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w;
+            __builtin_nontemporal_store(w, reinterpret_cast<streamed_float4 *>(dst4 + q));
+        }
         for (int q = (words & ~3) + threadIdx.x; q < words; q += 256) grad_sh_rest[base_word + q] = lds[q];
     }
 }
