@@ -266,13 +266,20 @@ __device__ __forceinline__ uint32_t strip_order_tile(uint32_t i, uint32_t grid_w
     const uint32_t rows = grid_h % kOrderStrip, r = i - full;
     return (grid_h - rows + r % rows) * grid_w + r / rows;
 }
-__device__ __forceinline__ uint32_t order_group_length(const uint32_t *__restrict__ ranges, uint32_t group, uint32_t grid_w, uint32_t grid_h)
+// A thread per tile, in strip order: sixteen neighbouring lanes are a group and add up its lists' lengths between them.
+// i: the tile's place in strip order; returns the group's total in all of its lanes (0 beyond the last whole group).
+__device__ __forceinline__ uint32_t order_group_length(const uint32_t *__restrict__ ranges, uint32_t i, uint32_t n_tiles, uint32_t grid_w, uint32_t grid_h,
+                                                       uint32_t &tile)
 {
+    static_assert(kOrderGroup == 16, "a group is sixteen lanes");
     uint32_t length = 0;
-    for (uint32_t t = 0; t < kOrderGroup; ++t) {
-        const uint32_t tile = strip_order_tile(kOrderGroup * group + t, grid_w, grid_h);
-        length += ranges[2 * tile + 1] - ranges[2 * tile];
+    tile = 0;
+    if (i < n_tiles / kOrderGroup * kOrderGroup) {
+        tile = strip_order_tile(i, grid_w, grid_h);
+        length = ranges[2 * tile + 1] - ranges[2 * tile];
     }
+#pragma unroll
+    for (int m = 1; m < (int)kOrderGroup; m <<= 1) length += __shfl_xor(length, m, kWave);
     return length;
 }
 __global__ void __launch_bounds__(256) tile_order_count_kernel(const uint32_t *__restrict__ ranges, uint32_t *__restrict__ order, uint32_t grid_w,
@@ -281,8 +288,10 @@ __global__ void __launch_bounds__(256) tile_order_count_kernel(const uint32_t *_
     __shared__ uint32_t count[kOrderBuckets];
     if (threadIdx.x < kOrderBuckets) count[threadIdx.x] = 0;
     __syncthreads();
-    const uint32_t n_tiles = grid_w * grid_h, group = blockIdx.x * 256 + threadIdx.x;
-    if (group < n_tiles / kOrderGroup) atomicAdd(&count[order_bucket(order_group_length(ranges, group, grid_w, grid_h))], 1u);
+    const uint32_t n_tiles = grid_w * grid_h, i = blockIdx.x * 256 + threadIdx.x;
+    uint32_t tile;
+    const uint32_t length = order_group_length(ranges, i, n_tiles, grid_w, grid_h, tile);
+    if (i % kOrderGroup == 0 && i / kOrderGroup < n_tiles / kOrderGroup) atomicAdd(&count[order_bucket(length)], 1u);
     __syncthreads();
     if (threadIdx.x < kOrderBuckets && count[threadIdx.x]) atomicAdd(order + n_tiles + threadIdx.x, count[threadIdx.x]);
 }
@@ -293,12 +302,12 @@ __global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *_
     const uint32_t n_tiles = grid_w * grid_h, n_groups = n_tiles / kOrderGroup;
     if (threadIdx.x < kOrderBuckets) { count[threadIdx.x] = 0; total[threadIdx.x] = order[n_tiles + threadIdx.x]; }
     __syncthreads();
-    const uint32_t group = blockIdx.x * 256 + threadIdx.x;
-    uint32_t bucket = 0, rank = 0;
-    if (group < n_groups) {
-        bucket = order_bucket(order_group_length(ranges, group, grid_w, grid_h));
-        rank = atomicAdd(&count[bucket], 1u);
-    }
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x, group = i / kOrderGroup, t = i % kOrderGroup;
+    uint32_t tile;
+    const uint32_t length = order_group_length(ranges, i, n_tiles, grid_w, grid_h, tile);
+    const uint32_t bucket = order_bucket(length);                   // (the same in the group's lanes)
+    uint32_t rank = 0;
+    if (t == 0 && group < n_groups) rank = atomicAdd(&count[bucket], 1u);
     __syncthreads();
     if (threadIdx.x < kOrderBuckets && count[threadIdx.x]) {
         // where the bin starts (the totals of the bins before it) + what other workgroups have taken of it
@@ -307,14 +316,13 @@ __global__ void __launch_bounds__(256) tile_order_place_kernel(const uint32_t *_
         base[threadIdx.x] = start + atomicAdd(order + n_tiles + kOrderBuckets + threadIdx.x, count[threadIdx.x]);
     }
     __syncthreads();
+    rank = __shfl(rank, (int)((threadIdx.x & (kWave - 1)) & ~(kOrderGroup - 1u)), kWave);      // the group's first lane has it
     if (group < n_groups) {
         const uint32_t place = base[bucket] + rank, interleaved = n_groups / kOrderDies * kOrderDies;
-        for (uint32_t t = 0; t < kOrderGroup; ++t) {
-            const uint32_t at = place < interleaved ? kOrderDies * (kOrderGroup * (place / kOrderDies) + t) + place % kOrderDies : kOrderGroup * place + t;
-            order[at] = strip_order_tile(kOrderGroup * group + t, grid_w, grid_h);
-        }
-    } else if (group == n_groups) {
-        for (uint32_t i = kOrderGroup * n_groups; i < n_tiles; ++i) order[i] = strip_order_tile(i, grid_w, grid_h);
+        const uint32_t at = place < interleaved ? kOrderDies * (kOrderGroup * (place / kOrderDies) + t) + place % kOrderDies : kOrderGroup * place + t;
+        order[at] = tile;
+    } else if (i < n_tiles) {
+        order[i] = strip_order_tile(i, grid_w, grid_h);             // the tiles that fill no group, at the end
     }
 }
 
@@ -508,7 +516,7 @@ extern "C" int htgs_extract_ranges(const htgs_frame *f, int selector)
     }
     if (f->tile_order) {
         const uint32_t grid_w = (uint32_t)div_up(f->width, tile), grid_h = (uint32_t)div_up(f->height, tile);
-        const dim3 grid((unsigned)((n_tiles / kOrderGroup + 1 + 255) / 256)), block(256);
+        const dim3 grid((unsigned)((n_tiles + 255) / 256)), block(256);
         hipLaunchKernelGGL(tile_order_count_kernel, grid, block, 0, s, f->ranges, f->tile_order, grid_w, grid_h);
         hipLaunchKernelGGL(tile_order_place_kernel, grid, block, 0, s, f->ranges, f->tile_order, grid_w, grid_h);
     }
