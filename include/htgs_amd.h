@@ -90,11 +90,14 @@ typedef struct htgs_frame {
                                   NULL: every tile is walked by one wave (no counterpart in the reference, which
                                   does that) */
     int32_t long_list_threshold; /* 0 = the default (8192 instances) */
-    uint32_t *tile_order;      /* htgs_tile_order_words() words or NULL.  Written by htgs_extract_ranges: the n_tiles tiles,
-                                  longest lists first (binned by length, four bins per power of two), then scratch of
-                                  that stage.  Every kernel that walks tile lists takes its tiles in this order, so the long
-                                  lists are not left for the end of the launch; results do not depend on it.  NULL:
-                                  tile order (no counterpart in the reference) */
+    uint32_t *tile_order;      /* htgs_tile_order_words() words or NULL.  Written by htgs_extract_ranges: the n_tiles tiles
+                                  in groups of sixteen neighbours (a 4x4 patch), the groups with the longest lists first
+                                  (binned by total length, four bins per power of two) and a group's tiles at the
+                                  workgroup indices that one accelerator die is given; then scratch of that stage.
+                                  Every kernel that walks tile lists takes its tiles in this order, so the long lists
+                                  are not left for the end of the launch and the tiles that share Gaussians share a
+                                  die's cache; results do not depend on it.  NULL: tile order (no counterpart in the
+                                  reference) */
     uint32_t *depth_order;     /* htgs_depth_order_words(N) words or NULL.  ALPHA_BLEND_GLOBAL_ORDERING, inference entry
                                   points: htgs_scan_offsets first sorts the Gaussians by the depth of their centres
                                   (stable), offsets[] then is the prefix sum in that order and htgs_create_instances emits
