@@ -472,12 +472,17 @@ __device__ __forceinline__ void quadrant_list_walk(const QuadrantLists &ql, uint
     // (the entry of the next turn is read while this turn's slot is evaluated: one LDS round trip per turn, not two)
     uint32_t p = (uint32_t)(uintptr_t)(lds_u32 *)&ql.a[lane >> 4][0];
     uint32_t addr = *(lds_u32 *)(uintptr_t)p;
-    for (uint32_t t = 0; t < n_turns; ++t) {
+    // (two turns per round of the loop, the entry that was read ahead changing registers, so that no turn moves it)
+    uint32_t t = 0;
+    for (; t + 1 < n_turns; t += 2) {
         asm volatile("v_add_u32 %0, 4, %0" : "+v"(p));
         const uint32_t next = *(lds_u32 *)(uintptr_t)p;
         turn(addr);
-        addr = next;
+        asm volatile("v_add_u32 %0, 4, %0" : "+v"(p));
+        addr = *(lds_u32 *)(uintptr_t)p;
+        turn(next);
     }
+    if (t < n_turns) turn(addr);
 }
 // The walk over instances [first, last) of a tile's list (whole batches of 64 from `first` on) by one wave, lanes =
 // pixels by quadrants: every batch is staged (tile_stage_load with the CULL asked for), its quadrant lists are built and

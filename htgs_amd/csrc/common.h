@@ -178,8 +178,11 @@ __device__ __forceinline__ float rcp_refined(float x)
 }
 __device__ __forceinline__ float rcp_exact(float x)
 {
-    if (__builtin_expect(__any(!rcp_in_range(x)), 0)) return 1.0f / x;
-    return rcp_refined(x);
+    // (the short form first and unconditionally, the division over it where a lane needs it: one branch around a side
+    // block instead of two ways that meet again)
+    float r = rcp_refined(x);
+    if (__builtin_expect(__any(!rcp_in_range(x)), 0)) r = 1.0f / x;
+    return r;
 }
 
 __device__ __forceinline__ float clamp_pos(float v) { return v > 0.0f ? v : 0.0f; }
