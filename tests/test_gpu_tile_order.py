@@ -32,16 +32,7 @@ def strip_order(grid_w: int, grid_h: int) -> np.ndarray:
     return np.array(out, np.int64)
 
 
-@pytest.mark.parametrize("config,n,mode", [(0, 10_000, 0), (1, 60_000, 0), (1, 60_000, 2), (3, 40_000, 0), (0, 0, 0)])
-def test_order_is_a_permutation_with_the_longest_lists_first(cuda, config, n, mode):
-    print(f"case config={config} n={n} mode={mode}", flush=True)
-    scene = make_scene(config, max(n, 1))
-    if n == 0:                                     # nothing visible: every list is empty
-        scene.positions[:, 2] = -5.0
-    scene = scene.to(cuda)
-    fb = FrameBuffers(*scene.gaussians(), scene.settings(RasterizerMode(mode), 4), True, False)
-    fb.run()
-    torch.cuda.synchronize()
+def check_order(fb, mode):
     order = u32(fb.tile_order)[:fb.n_tiles].astype(np.int64)
     assert np.array_equal(np.sort(order), np.arange(fb.n_tiles))
     ranges = u32(fb.ranges).astype(np.int64)
@@ -66,6 +57,19 @@ def test_order_is_a_permutation_with_the_longest_lists_first(cuda, config, n, mo
         assert (np.diff(length_bin(np.array(totals))) <= 0).all()
 
 
+@pytest.mark.parametrize("config,n,mode", [(0, 10_000, 0), (1, 60_000, 0), (1, 60_000, 2), (3, 40_000, 0), (0, 0, 0)])
+def test_order_is_a_permutation_with_the_longest_lists_first(cuda, config, n, mode):
+    print(f"case config={config} n={n} mode={mode}", flush=True)
+    scene = make_scene(config, max(n, 1))
+    if n == 0:                                     # nothing visible: every list is empty
+        scene.positions[:, 2] = -5.0
+    scene = scene.to(cuda)
+    fb = FrameBuffers(*scene.gaussians(), scene.settings(RasterizerMode(mode), 4), True, False)
+    fb.run()
+    torch.cuda.synchronize()
+    check_order(fb, mode)
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_results_do_not_depend_on_the_order(cuda, mode):
     print(f"case mode={mode}", flush=True)
@@ -79,3 +83,25 @@ def test_results_do_not_depend_on_the_order(cuda, mode):
     assert with_order.tile_order is not None and in_tile_order.tile_order is None
     assert torch.equal(with_order.image, in_tile_order.image)
     assert torch.equal(with_order.depth, in_tile_order.depth)
+
+
+@pytest.mark.parametrize("width,height", [(8, 8), (24, 16), (100, 52), (130, 70), (33, 200)])
+@pytest.mark.parametrize("mode", [0, 2])
+def test_order_on_grids_that_fill_no_whole_groups_or_strips(cuda, width, height, mode):
+    """Images whose tile grids have fewer than sixteen tiles, leave tiles over after the last whole group, or end in a strip
+    of fewer than four tile rows: the order is still a permutation of the stated structure and changes nothing."""
+    import dataclasses
+    from htgs_amd.synthetic import pinhole
+    print(f"case {width}x{height} mode={mode}", flush=True)
+    scene = make_scene(0, 4000)
+    M, VPM, cam = pinhole(width, height, 0.6 * width, 0.6 * width, width / 2, height / 2, scene.near_plane, scene.far_plane)
+    scene = dataclasses.replace(scene, M=M, VPM=VPM, cam_position=cam, width=width, height=height).to(cuda)
+    settings = scene.settings(RasterizerMode(mode), 4)
+    fb = FrameBuffers(*scene.gaussians(), settings, True, False)
+    fb.run()
+    plain = FrameBuffers(*scene.gaussians(), settings, True, False, pool=None, order_tiles=False)
+    plain.run()
+    torch.cuda.synchronize()
+    check_order(fb, mode)
+    assert float(fb.image.max()) > 0.0
+    assert torch.equal(fb.image, plain.image) and torch.equal(fb.depth, plain.depth)
