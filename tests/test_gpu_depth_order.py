@@ -170,3 +170,39 @@ def test_fast_path_lists_are_the_reference_lists_roughly_front_to_back(cuda, con
     image = fb.image.cpu().numpy()
     diff = np.abs(image - ref["image"])
     assert float((diff > 1e-5).mean()) < 1e-3 and float(diff.max()) <= 5e-2
+
+
+@pytest.mark.parametrize("near,far", [(1e-3, 1e6), (0.0, 100.0), (0.5, float("inf")), (3.0, 5.5)])
+@pytest.mark.parametrize("n", [1, 300, 4097, 9000])
+def test_fast_path_coarse_order_with_other_planes_and_counts(cuda, near, far, n):
+    """The fast path's coarse depth keys for near / far planes that make the full keys wide (or 32 bits: no positive near
+    plane, an infinite far plane) or narrow, and for counts that are no multiple of a sort block: every tile's list holds
+    the oracle's instances, the lists run front to back up to what a key step is worth, the image stays within the fast
+    path's bounds."""
+    import dataclasses
+    from util import u32
+    print(f"case near={near} far={far} n={n}", flush=True)
+    scene = dataclasses.replace(make_scene(0, n), near_plane=near, far_plane=far)
+    ref = oracle_render(scene, 0, 8)
+    sg = scene.to(cuda)
+    fb = FrameBuffers(*sg.gaussians(), sg.settings(RasterizerMode(0), 8), True, False, fast=True)
+    fb.run()
+    torch.cuda.synchronize()
+    ranges = u32(fb.ranges).astype(np.int64)
+    np.testing.assert_array_equal(ranges, ref["ranges"])
+    vals = u32(fb.vals[fb.selector])[:fb.n_instances].astype(np.int64) if fb.n_instances else np.zeros(0, np.int64)
+    depth = ref["pre"]["MT3"][:, 3].astype(np.float64)
+    # what one step of an eight-bit key is worth at most: the keys span the bit patterns from the near plane (or 0) to the far
+    # plane (or the largest pattern), 2^23 patterns per power of two
+    lo = np.float32(near).view(np.uint32) if near > 0.0 and np.isfinite(far) else np.uint32(0)
+    hi = np.float32(far).view(np.uint32) if near > 0.0 and np.isfinite(far) else np.uint32(0xfffffffe)
+    shift = 0
+    while ((int(hi) - int(lo)) >> shift) + 1 >= 256:
+        shift += 1
+    step = 2.0 ** (shift - 23)                                          # relative to the depth, at most
+    for a, b in ranges[ranges[:, 1] > ranges[:, 0]]:
+        assert np.array_equal(np.sort(vals[a:b]), ref["sorted_vals"][a:b].astype(np.int64))
+        d = depth[vals[a:b]]
+        assert float(np.max(np.maximum.accumulate(d) / d)) <= (1.0 + step) * (1.0 + 1e-6) if step < 1.0 else True
+    diff = np.abs(fb.image.cpu().numpy() - ref["image"])
+    assert float((diff > 1e-5).mean()) < 1e-3 and float(diff.max()) <= 5e-2
