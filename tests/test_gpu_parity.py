@@ -115,6 +115,26 @@ def test_fast_rasterize_against_the_oracle(cuda, config, n, mode):
         assert float(diff.max()) <= 5e-2
 
 
+def test_fast_rasterize_with_lists_up_to_the_packing_limit(cuda):
+    """HYBRID_BLEND's fast kernel with one wave per tile packs a core entry's place in its tile's list into 13 bits of a
+    key; on the stress scene dozens of tiles have lists of 4096 to 8192 instances (the longest this kernel walks), and
+    longer ones go to the kernel for long lists, which keeps three registers a slot.  Same bounds as above."""
+    from htgs_amd.torch_bindings import FrameBuffers
+    from util import u32
+    scene = make_scene(3, 200_000)
+    print("case config=3 n=200000 mode=0 (fast, long lists)", flush=True)
+    ref = oracle_render(scene, 0, 16)["image"]
+    sc = scene.to(cuda)
+    fb = FrameBuffers(*sc.gaussians(), sc.settings(0, 16), True, False, fast=True)
+    fb.run()
+    ranges = u32(fb.ranges).astype(np.int64)
+    length = ranges[:, 1] - ranges[:, 0]
+    assert int(((length > 4096) & (length <= 8192)).sum()) > 10 and int((length > 8192).sum()) > 5
+    diff = np.abs(fb.image.cpu().numpy() - ref)
+    assert float((diff > 1e-5).mean()) < 1e-3
+    assert float(diff.max()) <= 5e-2
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_fast_rasterize_reproduces_the_frozen_float64_image(cuda, mode):
     """The same entry point against tests/golden/small_scene.npz (independent float64 evaluator, no CPU oracle in
