@@ -333,8 +333,9 @@ def bench_all_configs(dev, headline_scene):
     scene_cpu, scene = headline_scene
     for mode in (1, 2, 3):
         out[f"cfg2/{MODE_NAMES[mode]}"] = compact(bench_inference(scene_cpu, scene, 2, None, mode, 16, EXTRA_STEPS, EXTRA_WARMUP, cpu_baseline=False))
-    out["cfg2/HYBRID_BLEND/fast_rasterize"] = compact(bench_inference(scene_cpu, scene, 2, None, 0, 16, EXTRA_STEPS, EXTRA_WARMUP, fast=True,
-                                                                      cpu_baseline=False))
+    for mode in (0, 1, 2, 3):
+        out[f"cfg2/{MODE_NAMES[mode]}/fast_rasterize"] = compact(bench_inference(scene_cpu, scene, 2, None, mode, 16, EXTRA_STEPS, EXTRA_WARMUP, fast=True,
+                                                                                 cpu_baseline=False))
     del scene
     release()
     for config, K in ((0, 4), (1, 16), (3, 16)):
