@@ -113,8 +113,8 @@ template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = Sort
 __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
     const KeyT *__restrict__ keys_in, const uint32_t *__restrict__ vals_in, KeyT *__restrict__ keys_out, uint32_t *__restrict__ vals_out,
     const uint32_t *__restrict__ hist, const uint32_t *__restrict__ totals, uint64_t n, uint32_t n_blocks, int shift, uint32_t mask,
-    const uint2 *__restrict__ rectangles_in = nullptr, uint2 *__restrict__ rectangles_out = nullptr, uint32_t *__restrict__ counts_out = nullptr,
-    uint32_t culled = 0)
+    bool last_pass = false, const uint2 *__restrict__ rectangles_in = nullptr, uint2 *__restrict__ rectangles_out = nullptr,
+    uint32_t *__restrict__ counts_out = nullptr, uint32_t culled = 0)
 {
     constexpr int kSortThreads = THREADS, kSortWaves = kSortThreads / kWave, kSortTile = kSortThreads * kSortItems;
     constexpr int kBits = BITS, kRadix = 1 << kBits, kDigitWaves = kRadix / kWave;
@@ -235,7 +235,12 @@ __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
             const uint32_t pos = global_base[d] + (i - digit_start[d]);
             keys_out[pos] = k;
             if (kTwoRounds || RECTANGLES) digits[r / 2] |= d << (16 * (r % 2));
-            if (!kTwoRounds) vals_out[pos] = local_vals[i];
+            if (!kTwoRounds) {
+                // (the sorted values are read once more, by the walk of their tile's list: streaming stores leave the
+                // caches to the records that the tiles share)
+                if (last_pass) __builtin_nontemporal_store(local_vals[i], vals_out + pos);
+                else vals_out[pos] = local_vals[i];
+            }
         }
     }
     if constexpr (RECTANGLES) {
@@ -273,14 +278,18 @@ __global__ void __launch_bounds__(THREADS) digit_scatter_kernel(
             const uint32_t i = (uint32_t)r * kSortThreads + threadIdx.x;
             if (i < n_local) {
                 const uint32_t d = digits[r / 2] >> (16 * (r % 2)) & 0xffffu;
-                vals_out[global_base[d] + (i - digit_start[d])] = local_vals[i];
+                uint32_t *out = vals_out + (global_base[d] + (i - digit_start[d]));
+                if (last_pass) __builtin_nontemporal_store(local_vals[i], out);
+                else *out = local_vals[i];
             }
         }
     }
 }
 
+// streaming_result: the sorted values leave the last pass as streaming stores (the instance lists, which the blend reads once)
 template <typename KeyT, int THREADS = SortShape<KeyT>::threads, int BITS = SortDigit<KeyT>::bits>
-static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int *selector)
+static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2], uint32_t *sort_tmp, uint64_t n, int end_bit, int *selector,
+                      bool streaming_result = false)
 {
     constexpr int kSortThreads = THREADS, kSortTile = kSortThreads * kSortItems;
     const uint32_t n_blocks = (uint32_t)((n + kSortTile - 1) / kSortTile);
@@ -296,7 +305,7 @@ static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2
         hipLaunchKernelGGL((digit_histogram_kernel<KeyT, THREADS, BITS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
         hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
         hipLaunchKernelGGL((digit_scatter_kernel<KeyT, THREADS, BITS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, vals[cur], kout, vals[cur ^ 1],
-                           hist, totals, n, n_blocks, shift, mask);
+                           hist, totals, n, n_blocks, shift, mask, streaming_result && shift + kBits >= end_bit);
         cur ^= 1;
     }
     *selector = cur;
@@ -317,8 +326,8 @@ int sort_u32_pairs_with_rectangles(void *stream, uint32_t *const keys[2], uint32
     hipLaunchKernelGGL((digit_histogram_kernel<uint32_t, kThreads, kBits>), dim3(xcd_padded_grid(n_blocks)), dim3(kThreads), 0, s, keys[0], hist, n, n_blocks, 0, mask);
     hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
     hipLaunchKernelGGL((digit_scatter_kernel<uint32_t, kThreads, kBits, true>), dim3(xcd_padded_grid(n_blocks)), dim3(kThreads), 0, s, keys[0], vals[0], keys[1],
-                       vals[1], hist, totals, n, n_blocks, 0, mask, reinterpret_cast<const uint2 *>(rectangles_in), reinterpret_cast<uint2 *>(rectangles_out),
-                       counts_out, culled);
+                       vals[1], hist, totals, n, n_blocks, 0, mask, false, reinterpret_cast<const uint2 *>(rectangles_in),
+                       reinterpret_cast<uint2 *>(rectangles_out), counts_out, culled);
     return check_launch("sort");
 }
 
@@ -358,8 +367,8 @@ extern "C" int htgs_sort_instances(const htgs_frame *f, int *selector)
     const int end_bit = htgs_frame_end_bit(f);
     hipStream_t s = (hipStream_t)f->stream;
     switch (htgs_frame_key_bytes(f)) {
-        case 8: return sort_pairs<uint64_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector);
-        case 4: return sort_pairs<uint32_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector);
-        default: return sort_pairs<uint16_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector);
+        case 8: return sort_pairs<uint64_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector, true);
+        case 4: return sort_pairs<uint32_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector, true);
+        default: return sort_pairs<uint16_t>(s, f->keys, f->vals, f->sort_tmp, f->n_instances, end_bit, selector, true);
     }
 }
