@@ -181,9 +181,9 @@ static void launch_hybrid(const htgs_frame *f, int selector, uint32_t grid_w, ui
 {
     const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
     // (the fast path packs a core entry's place in its list into 13 bits where no list of the launch can be longer)
-    if (FAST && f->long_tiles != nullptr && threshold <= kPackedListMost)
-        hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
-                           (const float4 *)f->prim, f->image, (float *)nullptr, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
+    if (f->long_tiles != nullptr && threshold <= kPackedListMost)
+        hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST, true>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                           (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
                            f->use_median_depth, f->long_tiles, threshold, long_part_floor(f, selector, n_tiles), f->tile_order);
     else
         hipLaunchKernelGGL((blend_hybrid_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],

@@ -133,31 +133,59 @@ __device__ __forceinline__ void core_key_walk(CoreKey &carried, CoreKey (&core)[
         for (int i = g0; i < g1; ++i) key_step(carried, core[i]);
     }
 }
-template <int K, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4>
-__device__ __forceinline__ void hybrid_fast_key_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
-                                                     uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy,
-                                                     CoreKey (&core)[K], HybridTail &tail)
+// FAST or not is the arithmetic of a fragment alone.  Without FAST, `tie` receives the least depth at which the keys may not
+// have kept what the reference's insertion keeps: an entry left the core that is exactly as deep as the entry that is now
+// last (which of the two stays is the insertion's choice; it matters if the finished core still reaches that deep.  Two
+// such entries that both stay are seen in the finished core, key_core_tied).
+template <int K, bool FAST, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4>
+__device__ __forceinline__ void hybrid_key_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+                                                uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy,
+                                                CoreKey (&core)[K], HybridTail &tail, float &tie)
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
     constexpr int N = kStageSlots;
-    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4, true, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4, FAST, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
         TileFrag f;
-        const bool fragment = tile_frag_fast<MODE, N>(addr, pt, f);
+        bool fragment;
+        if constexpr (FAST) fragment = tile_frag_fast<MODE, N>(addr, pt, f);
+        else {
+            const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+            f.den_rcp = frag_rcp<FAST>(f.den);
+            fragment = tile_frag_alpha<MODE, FAST>(stage_opacity<N>(addr), f) && in_reach;
+        }
         const float4 col = stage_row<N, 5>(addr);
         if (!fragment) return;
         float depth = tile_frag_depth<N>(addr, pt, f);
         float p3 = f.alpha;
-        tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
-        tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
-        tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
         if (depth < key_depth(core[K - 1]) && f.alpha >= kMinAlphaCore) {
-            CoreKey carried = make_key(depth, key_pack(p3, float_to_bits(col.w) - first));
+            // (a fragment that enters the core has the alpha that its key holds from here on: what the colour sums
+            // receive now is what is taken out of them again for the entries of the finished core)
+            const uint32_t low = key_pack(p3, float_to_bits(col.w) - first);
+            p3 = key_alpha(low);
+            tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
+            tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
+            tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
+            CoreKey carried = make_key(depth, low);
             core_key_walk<K>(carried, core);
             depth = key_depth(carried);
             p3 = key_alpha(key_low(carried));
+            if constexpr (!FAST) tie = p3 > 0.0f && depth == key_depth(core[K - 1]) && depth < tie ? depth : tie;
+        } else {
+            tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
+            tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
+            tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
         }
-        hybrid_tail_add<true>(tail, depth, p3);
+        hybrid_tail_add<FAST>(tail, depth, p3);
     });
+}
+// two entries of the finished core are exactly as deep as each other (their order is the reference's insertion's to choose)
+template <int K>
+__device__ __forceinline__ bool key_core_tied(const CoreKey (&core)[K])
+{
+    bool tied = false;
+#pragma unroll
+    for (int i = 0; i + 1 < K; ++i) tied = tied || (key_low(core[i + 1]) >> 13 != 0u && __double2hiint(core[i]) == __double2hiint(core[i + 1]));
+    return tied;
 }
 // the finished keys as the three arrays the composite takes
 template <int K>
@@ -232,6 +260,49 @@ struct HybridImage {
         hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
     }
 };
+
+// One tile by one wave with the core as keys; finish(prim, tile, px, cd, ca, ci, tail) is called once per pixel inside the
+// image.  Without FAST, the pixels at which fragments of exactly equal depth met where they decide the core (a pixel or
+// two in a tile in a hundred) are walked again afterwards, over the instances that reach one of them, with the
+// reference's insertion.
+template <int K, bool FAST, int REC4, typename Finish>
+__device__ __forceinline__ void hybrid_tile_by_keys(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+                                                    uint32_t tile, uint32_t first, uint32_t last, uint32_t lane, const TilePixel &px, uint32_t grid_w,
+                                                    uint32_t width, uint32_t height, const Finish &finish)
+{
+    HybridTail tail;
+    hybrid_tail_init(tail);
+    float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
+    CoreKey core[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        core[i] = make_key(__FLT_MAX__, 0u);
+        asm volatile("" : "+v"(core[i]));      // one register pair per slot, never a wide tuple
+    }
+    float tie = __FLT_MAX__;
+    hybrid_key_walk<K, FAST, true, REC4>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail, tie);
+    if constexpr (FAST) {
+        if (!px.inside) return;
+        key_core_unpack<K>(core, inst, first, last, cd, ca, ci);
+        finish(prim, tile, px, cd, ca, ci, tail);
+    } else {
+        const bool again = px.inside && ((tie < __FLT_MAX__ && tie <= key_depth(core[K - 1])) || key_core_tied<K>(core));
+        const uint64_t again_lanes = __ballot(again);
+        key_core_unpack<K>(core, inst, first, last, cd, ca, ci);
+        if (px.inside && !again) finish(prim, tile, px, cd, ca, ci, tail);
+        if (again_lanes == 0) return;
+        // (the lane and its pixel are worked out afresh, so that nothing the first walk keeps in registers has to
+        // live through the pixels' finish for the sake of this rare second walk)
+        uint32_t lane_again = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        asm volatile("" : "+v"(lane_again));
+        const TilePixel px_again = quadrant_tile_pixel(tile, grid_w, lane_again, width, height);
+        hybrid_tail_init(tail);
+        hybrid_core_init<K>(cd, ca, ci);
+        hybrid_walk<K, false, true, false, true, REC4>(st, ql, inst, prim, first, last, lane_again, px_again.pt, px_again.cx, px_again.cy, cd, ca, ci, tail, nullptr,
+                                                       again_lanes);
+        if ((again_lanes >> lane_again & 1ull) != 0) finish(prim, tile, px_again, cd, ca, ci, tail);
+    }
+}
 
 // ---------------------------------------------------------------------------------------------
 // Tiles with very long lists (HYBRID_BLEND, ALPHA_BLEND_FIRST_K and OIT_BLEND, which walk all of a list): the kernel
@@ -338,7 +409,7 @@ __device__ __forceinline__ bool long_part_done(const uint32_t *long_tiles, uint3
 }
 
 // One wave per tile; the tiles with very long lists are left to blend_hybrid_long_kernel.
-// KEYS (the fast path, with long_tiles and a threshold of no more than kPackedListMost): the core as sorted 64-bit keys.
+// KEYS (with long_tiles and a threshold of no more than kPackedListMost): the core as sorted 64-bit keys, hybrid_tile_by_keys.
 template <int K, bool FAST, bool KEYS = false>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
@@ -355,26 +426,18 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
         return;
     }
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
-    HybridTail tail;
-    hybrid_tail_init(tail);
-    float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
     if constexpr (KEYS) {
-        static_assert(FAST, "the image-only path");
-        CoreKey core[K];
-#pragma unroll
-        for (int i = 0; i < K; ++i) {
-            core[i] = make_key(__FLT_MAX__, 0u);
-            asm volatile("" : "+v"(core[i]));      // one register pair per slot, never a wide tuple
-        }
-        hybrid_fast_key_walk<K, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail);
-        if (!px.inside) return;
-        key_core_unpack<K>(core, inst, first, last, cd, ca, ci);
+        hybrid_tile_by_keys<K, FAST, HTGS_PRIM_FLOATS / 4>(st, ql, inst, prim, tile, first, last, lane, px, grid_w, width, height,
+                                                           HybridImage{ image, depths, width, height, chw, median });
     } else {
+        HybridTail tail;
+        hybrid_tail_init(tail);
+        float cd[K], ca[K], ci[K];                 // ci: the index's bit pattern
         hybrid_core_init<K>(cd, ca, ci);
         hybrid_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci, tail);
         if (!px.inside) return;
+        hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
     }
-    hybrid_composite<K>(prim, cd, ca, ci, tail, image, depths, width, height, px.x, px.y, chw, median);
 }
 
 __device__ __forceinline__ float wave_total(float v)

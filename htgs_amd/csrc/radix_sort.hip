@@ -17,7 +17,7 @@ constexpr int kSortItems = 16;                              // rounds per wave
 // digit width per key type; kRadix digits, the first kRadix threads of a block own one digit each
 template <typename KeyT> struct SortDigit { static constexpr int bits = sizeof(KeyT) == 8 ? 9 : 8; };
 constexpr int kMaxRadix = 512;
-constexpr int kScanThreads = 256;
+constexpr int kScanThreads = 1024;
 // Items per block = threads x 16 = 8192.  Longer blocks give longer runs per digit, i.e. fuller cache lines in the
 // scatter; two blocks fit a CU's LDS for every key width (8-byte keys share one array between keys and values).
 template <typename KeyT> struct SortShape { static constexpr int threads = 512; };
@@ -297,15 +297,18 @@ static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2
     uint32_t *hist = sort_tmp;
     uint32_t *totals = sort_tmp + (size_t)kRadix * n_blocks;
     int cur = 0;
-    for (int shift = 0; shift < end_bit; shift += kBits) {
-        const int bits = end_bit - shift < kBits ? end_bit - shift : kBits;
+    // the passes share the key's bits evenly (13 bits: 7 + 6 rather than 8 + 5): fewer digits per pass are longer runs
+    // per digit in every block's output
+    const int passes = (end_bit + kBits - 1) / kBits, step = passes > 0 ? (end_bit + passes - 1) / passes : kBits;
+    for (int shift = 0; shift < end_bit; shift += step) {
+        const int bits = end_bit - shift < step ? end_bit - shift : step;
         const uint32_t mask = (1u << bits) - 1u;
         const KeyT *kin = (const KeyT *)keys[cur];
         KeyT *kout = (KeyT *)keys[cur ^ 1];
         hipLaunchKernelGGL((digit_histogram_kernel<KeyT, THREADS, BITS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, hist, n, n_blocks, shift, mask);
         hipLaunchKernelGGL(digit_row_scan_kernel, dim3(kRadix), dim3(kScanThreads), 0, s, hist, totals, n_blocks);
         hipLaunchKernelGGL((digit_scatter_kernel<KeyT, THREADS, BITS>), dim3(xcd_padded_grid(n_blocks)), dim3(kSortThreads), 0, s, kin, vals[cur], kout, vals[cur ^ 1],
-                           hist, totals, n, n_blocks, shift, mask, streaming_result && shift + kBits >= end_bit);
+                           hist, totals, n, n_blocks, shift, mask, streaming_result && shift + step >= end_bit);
         cur ^= 1;
     }
     *selector = cur;
