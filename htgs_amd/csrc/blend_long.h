@@ -96,26 +96,44 @@ __device__ __forceinline__ void hybrid_walk(TileStageQ &st, QuadrantLists &ql, c
 }
 
 // ---------------------------------------------------------------------------------------------
-// The image-only fast path's core as sorted 64-bit keys (the kernel with one wave per tile).  A slot is one register
-// pair: the high word holds the depth, the low word alpha as a 19-bit fraction (an absolute error of 2^-20) above the
-// instance's place in the tile's list (13 bits: the lists this kernel walks are no longer than the threshold beyond
-// which a tile goes to the other kernel, at most kPackedListMost).  Positive floats order like their bit patterns and
-// so do the doubles made of (depth, low word): one step of the insertion is slot' = min(carried, slot), carried' =
-// max(carried, slot), two instructions without exec masks or moves, and what is pushed out carries the alpha that the
-// tail needs.  The Gaussian's index, which only the final core needs, is looked up from the place in the list when the
-// pixel is composited.  (Which of two fragments of equal depth comes first is decided by the low word here, which this
-// path does not promise to reproduce; depths that are not positive numbers would order differently from floats.)
+// HYBRID_BLEND's core as sorted 64-bit keys (the kernel with one wave per tile, inference).  A slot is one register pair:
+// the high word holds the depth, the low word alpha as a fraction of 19 to 23 bits (rounded: an absolute error of 2^-20 at
+// most, 2^-24 in the tiles with short lists; KeyFormat) above the instance's place in the tile's list (at most 13 bits: the
+// lists this kernel walks are no longer than the threshold beyond which a tile goes to the other kernel, at most
+// kPackedListMost).  Floats of one sign order like their bit patterns
+// and so do the doubles made of (depth, low word): one step of the insertion is slot' = min(carried, slot), carried' =
+// max(carried, slot), two instructions without exec masks or moves (a third of the exchange of three registers), and what
+// is pushed out carries the alpha that the tail needs.  The Gaussian's index, which only the final core needs, is looked
+// up from the place in the list when the pixel is composited.  Which of two fragments of equal depth comes first is
+// decided by the low word here, not by the reference's insertion: the image-only fast path leaves it at that; with exact
+// arithmetic the walk notes where it can matter (hybrid_key_walk) and such pixels are walked again.
 // ---------------------------------------------------------------------------------------------
 typedef double CoreKey;
-constexpr uint32_t kPackedListMost = 8192, kPackedAlphaOne = (1u << 19) - 1u;
+constexpr uint32_t kPackedListMost = 8192;
+// How a tile's keys divide the low word (the same for every pixel of the tile: scalar registers).  The place takes the bits
+// that the length of the tile's list asks for, nine at least, and alpha the other 19 to 23: a fraction of 23 bits is within
+// 2^-24 of the float, so in the tiles with up to 512 instances a key holds its alpha almost as the float does.
+struct KeyFormat {
+    uint32_t shift, place_mask;     // bits of the place; 2^shift - 1
+    float one, one_rcp;             // 2^(32 - shift) - 1, the fraction that stands for alpha = 1, and its reciprocal
+};
+__device__ __forceinline__ KeyFormat key_format(uint32_t list_length)      // 1 .. kPackedListMost
+{
+    KeyFormat f;
+    f.shift = 32u - (uint32_t)__builtin_clz((list_length - 1u) | 0x1ffu);
+    f.place_mask = (1u << f.shift) - 1u;
+    f.one = (float)((1u << (32u - f.shift)) - 1u);
+    f.one_rcp = 1.0f / f.one;
+    return f;
+}
 __device__ __forceinline__ float key_depth(CoreKey k) { return bits_to_float((uint32_t)__double2hiint(k)); }
 __device__ __forceinline__ uint32_t key_low(CoreKey k) { return (uint32_t)__double2loint(k); }
 __device__ __forceinline__ CoreKey make_key(float depth, uint32_t low) { return __hiloint2double((int)float_to_bits(depth), (int)low); }
-__device__ __forceinline__ uint32_t key_pack(float alpha, uint32_t place)      // alpha in [0, 1]
+__device__ __forceinline__ uint32_t key_pack(float alpha, uint32_t place, const KeyFormat &f)      // alpha in [0, 1]
 {
-    return (uint32_t)__builtin_fmaf(alpha, (float)kPackedAlphaOne, 0.5f) << 13 | place;
+    return (uint32_t)__builtin_fmaf(alpha, f.one, 0.5f) << f.shift | place;
 }
-__device__ __forceinline__ float key_alpha(uint32_t low) { return (float)(low >> 13) * (1.0f / (float)kPackedAlphaOne); }
+__device__ __forceinline__ float key_alpha(uint32_t low, const KeyFormat &f) { return (float)(low >> f.shift) * f.one_rcp; }
 __device__ __forceinline__ void key_step(CoreKey &carried, CoreKey &slot)
 {
     CoreKey out;
@@ -140,7 +158,7 @@ __device__ __forceinline__ void core_key_walk(CoreKey &carried, CoreKey (&core)[
 template <int K, bool FAST, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4>
 __device__ __forceinline__ void hybrid_key_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
                                                 uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy,
-                                                CoreKey (&core)[K], HybridTail &tail, float &tie)
+                                                CoreKey (&core)[K], HybridTail &tail, float &tie, const KeyFormat &fmt)
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
     constexpr int N = kStageSlots;
@@ -160,15 +178,15 @@ __device__ __forceinline__ void hybrid_key_walk(TileStageQ &st, QuadrantLists &q
         if (depth < key_depth(core[K - 1]) && f.alpha >= kMinAlphaCore) {
             // (a fragment that enters the core has the alpha that its key holds from here on: what the colour sums
             // receive now is what is taken out of them again for the entries of the finished core)
-            const uint32_t low = key_pack(p3, float_to_bits(col.w) - first);
-            p3 = key_alpha(low);
+            const uint32_t low = key_pack(p3, float_to_bits(col.w) - first, fmt);
+            p3 = key_alpha(low, fmt);
             tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
             tail.c1 = __builtin_fmaf(p3, col.y, tail.c1);
             tail.c2 = __builtin_fmaf(p3, col.z, tail.c2);
             CoreKey carried = make_key(depth, low);
             core_key_walk<K>(carried, core);
             depth = key_depth(carried);
-            p3 = key_alpha(key_low(carried));
+            p3 = key_alpha(key_low(carried), fmt);
             if constexpr (!FAST) tie = p3 > 0.0f && depth == key_depth(core[K - 1]) && depth < tie ? depth : tie;
         } else {
             tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);
@@ -180,23 +198,23 @@ __device__ __forceinline__ void hybrid_key_walk(TileStageQ &st, QuadrantLists &q
 }
 // two entries of the finished core are exactly as deep as each other (their order is the reference's insertion's to choose)
 template <int K>
-__device__ __forceinline__ bool key_core_tied(const CoreKey (&core)[K])
+__device__ __forceinline__ bool key_core_tied(const CoreKey (&core)[K], const KeyFormat &fmt)
 {
     bool tied = false;
 #pragma unroll
-    for (int i = 0; i + 1 < K; ++i) tied = tied || (key_low(core[i + 1]) >> 13 != 0u && __double2hiint(core[i]) == __double2hiint(core[i + 1]));
+    for (int i = 0; i + 1 < K; ++i) tied = tied || (key_low(core[i + 1]) >> fmt.shift != 0u && __double2hiint(core[i]) == __double2hiint(core[i + 1]));
     return tied;
 }
 // the finished keys as the three arrays the composite takes
 template <int K>
 __device__ __forceinline__ void key_core_unpack(const CoreKey (&core)[K], const uint32_t *__restrict__ inst, uint32_t first, uint32_t last, float (&cd)[K],
-                                                float (&ca)[K], float (&ci)[K])
+                                                float (&ca)[K], float (&ci)[K], const KeyFormat &fmt)
 {
 #pragma unroll
     for (int i = 0; i < K; ++i) {
-        const uint32_t low = key_low(core[i]), place = low & (kPackedListMost - 1u);
+        const uint32_t low = key_low(core[i]), place = low & fmt.place_mask;
         cd[i] = key_depth(core[i]);
-        ca[i] = key_alpha(low);
+        ca[i] = key_alpha(low, fmt);
         ci[i] = ca[i] > 0.0f && first + place < last ? bits_to_float(inst[first + place]) : 0.0f;
     }
 }
@@ -280,15 +298,16 @@ __device__ __forceinline__ void hybrid_tile_by_keys(TileStageQ &st, QuadrantList
         asm volatile("" : "+v"(core[i]));      // one register pair per slot, never a wide tuple
     }
     float tie = __FLT_MAX__;
-    hybrid_key_walk<K, FAST, true, REC4>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail, tie);
+    const KeyFormat fmt = key_format(last > first ? last - first : 1u);
+    hybrid_key_walk<K, FAST, true, REC4>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail, tie, fmt);
     if constexpr (FAST) {
         if (!px.inside) return;
-        key_core_unpack<K>(core, inst, first, last, cd, ca, ci);
+        key_core_unpack<K>(core, inst, first, last, cd, ca, ci, fmt);
         finish(prim, tile, px, cd, ca, ci, tail);
     } else {
-        const bool again = px.inside && ((tie < __FLT_MAX__ && tie <= key_depth(core[K - 1])) || key_core_tied<K>(core));
+        const bool again = px.inside && ((tie < __FLT_MAX__ && tie <= key_depth(core[K - 1])) || key_core_tied<K>(core, fmt));
         const uint64_t again_lanes = __ballot(again);
-        key_core_unpack<K>(core, inst, first, last, cd, ca, ci);
+        key_core_unpack<K>(core, inst, first, last, cd, ca, ci, fmt);
         if (px.inside && !again) finish(prim, tile, px, cd, ca, ci, tail);
         if (again_lanes == 0) return;
         // (the lane and its pixel are worked out afresh, so that nothing the first walk keeps in registers has to

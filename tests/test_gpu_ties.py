@@ -1,8 +1,9 @@
 """The HIP kernels against the hand-computed pixels of tests/test_oracle_ties.py (no oracle in between): fragments of
 exactly equal depth in HYBRID_BLEND's core must come out in the order of the reference's exchange walk
-(R/include/hybrid_blend/kernels/inference.cuh:159-167) -- through the kernel with one wave per tile, through the kernels
-that share a long list between waves (threshold forced down to 2 instances: the cores are merged and the pixel gets the
-second look), and in the core indices the training pass records."""
+(R/include/hybrid_blend/kernels/inference.cuh:159-167) -- through the kernel with one wave per tile (threshold 0, the
+default of 8192: the core as sorted keys, the pixel walked a second time; threshold 2^31 - 1: the exchange insertion
+throughout), through the kernels that share a long list between waves (threshold forced down to 2 instances: the cores
+are merged and the pixel gets the second look), and in the core indices the training pass records."""
 import numpy as np
 import pytest
 import torch
@@ -17,7 +18,7 @@ CASES = [(TWO, [4, 0, 2, 1], [3]), (THREE, [4, 0, 2, 3], [1])]
 
 
 @pytest.mark.parametrize("case,core,tail", CASES)
-@pytest.mark.parametrize("threshold", [0, 2])
+@pytest.mark.parametrize("threshold", [0, 2, 2 ** 31 - 1])
 def test_inference_pixel_with_equal_depths(cuda, case, core, tail, threshold):
     print(f"case depths={case['depths']} threshold={threshold}", flush=True)
     scene = tie_scene(**case).to(cuda)
