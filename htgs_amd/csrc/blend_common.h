@@ -247,17 +247,19 @@ enum { kCullNone = 0, kCullAlpha = 1, kCullCutoff = 2, kCullPixels = 3 };
 // REC4: 16-byte words per record of prim (five; eight in training frames).
 // UNIT: the opacity is staged held to at most 1 (the image-only fast path, whose fragments then need no clamp of their own).
 // POS: the last word of the slot holds the instance's place in the list (fetch) instead of the Gaussian's index.
-template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, bool POS = false>
+// GIVEN: the caller has read inst[fetch] already (`given`).
+template <int MODE, int N, bool DEPTH, int CULL = kCullNone, bool QUADRANTS = false, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, bool POS = false,
+          bool GIVEN = false>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
-                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes = 0);
+                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes = 0, uint32_t given = 0);
 
 // (PixelTerms is complete by the time the template is instantiated)
-template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS, int REC4, bool UNIT, bool POS>
+template <int MODE, int N, bool DEPTH, int CULL, bool QUADRANTS, int REC4, bool UNIT, bool POS, bool GIVEN>
 __device__ __forceinline__ uint32_t tile_stage_load(TileStage<N> &st, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
-                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes)
+                                                    uint32_t fetch, uint32_t last, int slot, float cx, float cy, uint64_t pixel_lanes, uint32_t given)
 {
     if (fetch >= last) return 0;
-    const uint32_t g = inst[fetch];
+    const uint32_t g = GIVEN ? given : inst[fetch];
     const float4 *rec = prim + (size_t)g * REC4;
     // (with CULL the record's colour row is fetched when it is needed, behind a compiler fence: it comes from a cache
     // line the other rows have just brought in, and four registers less at the peak keep the callers' K-buffers out
@@ -487,14 +489,20 @@ __device__ __forceinline__ void quadrant_list_walk(const QuadrantLists &ql, uint
 // The walk over instances [first, last) of a tile's list (whole batches of 64 from `first` on) by one wave, lanes =
 // pixels by quadrants: every batch is staged (tile_stage_load with the CULL asked for), its quadrant lists are built and
 // turn(addr) is called for every turn.  SOLO: the wave is the whole workgroup (its barriers are the workgroup's).
-template <int MODE, bool DEPTH, int CULL, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, bool POS = false, typename Turn>
+// AHEAD: a lane reads the list entry of the next batch before it walks this one (one register more through the walk; the
+// entry is then there when the batch is staged, and the records' fetch does not wait for it).
+template <int MODE, bool DEPTH, int CULL, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4, bool UNIT = false, bool POS = false, bool AHEAD = false, typename Turn>
 __device__ __forceinline__ void tile_list_walk(TileStageQ &st, QuadrantLists &ql, const float4 *__restrict__ prim, const uint32_t *__restrict__ inst,
                                                uint32_t first, uint32_t last, uint32_t lane, float cx, float cy, Turn &&turn, uint64_t pixel_lanes = 0)
 {
     stage_dummy_init(st, lane);
+    uint32_t listed = 0;
+    if (AHEAD) listed = first + lane < last ? inst[first + lane] : 0u;
     for (uint32_t base = first; base < last; base += 64) {
         if (SOLO) __syncthreads(); else wave_lds_sync();
-        const uint32_t bits = tile_stage_load<MODE, kStageSlots, DEPTH, CULL, true, REC4, UNIT, POS>(st, prim, inst, base + lane, last, lane + 1, cx, cy, pixel_lanes);
+        const uint32_t bits = tile_stage_load<MODE, kStageSlots, DEPTH, CULL, true, REC4, UNIT, POS, AHEAD>(st, prim, inst, base + lane, last, lane + 1, cx, cy, pixel_lanes,
+                                                                                                           listed);
+        if (AHEAD) listed = base + 64u + lane < last ? inst[base + 64u + lane] : 0u;
         const uint32_t n_turns = quadrant_lists_build(ql, bits, lane, st);
         if (SOLO) __syncthreads(); else wave_lds_sync();
         // lanes outside the image run along (their results are never stored): the loop stays wave-uniform

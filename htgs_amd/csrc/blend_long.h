@@ -155,14 +155,14 @@ __device__ __forceinline__ void core_key_walk(CoreKey &carried, CoreKey (&core)[
 // have kept what the reference's insertion keeps: an entry left the core that is exactly as deep as the entry that is now
 // last (which of the two stays is the insertion's choice; it matters if the finished core still reaches that deep.  Two
 // such entries that both stay are seen in the finished core, key_core_tied).
-template <int K, bool FAST, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4>
+template <int K, bool FAST, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4, bool AHEAD = false>
 __device__ __forceinline__ void hybrid_key_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
                                                 uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy,
                                                 CoreKey (&core)[K], HybridTail &tail, float &tie, const KeyFormat &fmt)
 {
     constexpr int MODE = HTGS_MODE_HYBRID_BLEND;
     constexpr int N = kStageSlots;
-    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4, FAST, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4, FAST, true, AHEAD>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
         TileFrag f;
         bool fragment;
         if constexpr (FAST) fragment = tile_frag_fast<MODE, N>(addr, pt, f);
@@ -299,7 +299,7 @@ __device__ __forceinline__ void hybrid_tile_by_keys(TileStageQ &st, QuadrantList
     }
     float tie = __FLT_MAX__;
     const KeyFormat fmt = key_format(last > first ? last - first : 1u);
-    hybrid_key_walk<K, FAST, true, REC4>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail, tie, fmt);
+    hybrid_key_walk<K, FAST, true, REC4, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tail, tie, fmt);
     if constexpr (FAST) {
         if (!px.inside) return;
         key_core_unpack<K>(core, inst, first, last, cd, ca, ci, fmt);
