@@ -199,9 +199,14 @@ template <int K, bool FAST>
 static void launch_first_k(const htgs_frame *f, int selector, uint32_t grid_w, uint32_t n_tiles)
 {
     const uint32_t threshold = f->long_list_threshold > 0 ? (uint32_t)f->long_list_threshold : kLongListDefault;
-    hipLaunchKernelGGL((blend_first_k_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
-                       (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
-                       f->use_median_depth, f->long_tiles, threshold, long_part_floor(f, selector, n_tiles), f->tile_order);
+    if (!FAST && f->long_tiles != nullptr && threshold <= kPackedListMost)
+        hipLaunchKernelGGL((blend_first_k_kernel<K, false, true>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                           (const float4 *)f->prim, f->image, f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
+                           f->use_median_depth, f->long_tiles, threshold, long_part_floor(f, selector, n_tiles), f->tile_order);
+    else
+        hipLaunchKernelGGL((blend_first_k_kernel<K, FAST>), dim3(n_tiles), dim3(64), 0, (hipStream_t)f->stream, f->ranges, f->vals[selector],
+                           (const float4 *)f->prim, f->image, FAST ? nullptr : f->depth, (uint32_t)f->width, (uint32_t)f->height, grid_w, f->to_chw,
+                           f->use_median_depth, f->long_tiles, threshold, long_part_floor(f, selector, n_tiles), f->tile_order);
     if (f->long_tiles)
         hipLaunchKernelGGL((blend_first_k_long_kernel<K, FAST, HTGS_PRIM_FLOATS / 4, FirstKImage>), dim3(256 * kLongWaves / long_waves<K>()), dim3(64 * long_waves<K>()), 0,
                            (hipStream_t)f->stream, f->ranges, f->vals[selector], (const float4 *)f->prim, f->long_tiles, (uint32_t)f->width, (uint32_t)f->height, grid_w,

@@ -798,14 +798,15 @@ __device__ __forceinline__ void first_k_core_init(float (&cd)[K], float (&ca)[K]
 // The walk over instances [first, last) of a tile's list by one wave (SOLO: the wave is the whole workgroup).  TIES (the
 // walks of blend_first_k_long_kernel): `tie` receives the least depth at which an entry was pushed out of the core that is
 // exactly as deep as the entry that is now last.
-template <int K, bool FAST, bool SOLO, bool TIES = false, int REC4 = HTGS_PRIM_FLOATS / 4>
+// PIXELS: only the pixels of the lanes in pixel_lanes are wanted; instances that do not reach one of them are left out.
+template <int K, bool FAST, bool SOLO, bool TIES = false, int REC4 = HTGS_PRIM_FLOATS / 4, bool PIXELS = false>
 __device__ __forceinline__ void first_k_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
                                              uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy, float (&cd)[K],
-                                             float (&ca)[K], uint32_t (&ci)[K], float *tie = nullptr)
+                                             float (&ca)[K], uint32_t (&ci)[K], float *tie = nullptr, uint64_t pixel_lanes = 0)
 {
     constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
     constexpr int N = kStageSlots;
-    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+    tile_list_walk<MODE, true, PIXELS ? kCullPixels : kCullAlpha, SOLO, REC4>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
         TileFrag f;
         const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
         f.den_rcp = frag_rcp<FAST>(f.den);
@@ -816,7 +817,42 @@ __device__ __forceinline__ void first_k_walk(TileStageQ &st, QuadrantLists &ql, 
         uint32_t idx = stage_index<N>(addr);
         core_exchange_walk<K>(depth, alpha, idx, cd, ca, ci);
         if (TIES && alpha > 0.0f && depth == cd[K - 1]) *tie = depth < *tie ? depth : *tie;
+    }, pixel_lanes);
+}
+// The same walk with the core as sorted 64-bit keys (above HYBRID_BLEND's: depth | alpha as a fraction | place in the list),
+// exact arithmetic; `tie` as in hybrid_key_walk.
+template <int K, bool SOLO, int REC4 = HTGS_PRIM_FLOATS / 4>
+__device__ __forceinline__ void first_k_key_walk(TileStageQ &st, QuadrantLists &ql, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
+                                                 uint32_t first, uint32_t last, uint32_t lane, const PixelTerms &pt, float cx, float cy,
+                                                 CoreKey (&core)[K], float &tie, const KeyFormat &fmt)
+{
+    constexpr int MODE = HTGS_MODE_ALPHA_BLEND_FIRST_K;
+    constexpr int N = kStageSlots;
+    tile_list_walk<MODE, true, kCullAlpha, SOLO, REC4, false, true, true>(st, ql, prim, inst, first, last, lane, cx, cy, [&](uint32_t addr) {
+        TileFrag f;
+        const bool in_reach = tile_frag_cutoff<N>(addr, pt, f);
+        f.den_rcp = frag_rcp<false>(f.den);
+        float depth = tile_frag_depth<N>(addr, pt, f);
+        if (!(in_reach && depth < key_depth(core[K - 1]))) return;          // depth test before the exponential (:151)
+        if (!tile_frag_alpha<MODE, false>(stage_opacity<N>(addr), f)) return;
+        CoreKey carried = make_key(depth, key_pack(f.alpha, stage_index<N>(addr) - first, fmt));      // (the slot's last word is the place in the list)
+        core_key_walk<K>(carried, core);
+        depth = key_depth(carried);
+        tie = key_low(carried) >> fmt.shift != 0u && depth == key_depth(core[K - 1]) && depth < tie ? depth : tie;
     });
+}
+// the finished keys as the three arrays the composite takes (an empty slot has the index 0xffffffff)
+template <int K>
+__device__ __forceinline__ void first_k_core_unpack(const CoreKey (&core)[K], const uint32_t *__restrict__ inst, uint32_t first, uint32_t last, float (&cd)[K],
+                                                    float (&ca)[K], uint32_t (&ci)[K], const KeyFormat &fmt)
+{
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const uint32_t low = key_low(core[i]), place = low & fmt.place_mask;
+        cd[i] = key_depth(core[i]);
+        ca[i] = key_alpha(low, fmt);
+        ci[i] = low >> fmt.shift != 0u && first + place < last ? inst[first + place] : 0xffffffffu;
+    }
 }
 template <int K, int REC4 = HTGS_PRIM_FLOATS / 4>
 __device__ __forceinline__ void first_k_composite(const float4 *__restrict__ prim, const float (&cd)[K], const float (&ca)[K], const uint32_t (&ci)[K],
@@ -855,12 +891,16 @@ struct FirstKImage {
 };
 // what a workgroup leaves of its part of a list: the core and the depth of a tie
 template <int K> constexpr uint32_t first_k_part_words() { return (3u * K + 1u) * 64u; }
-template <int K, bool FAST>
+// KEYS (exact arithmetic, with long_tiles and a threshold of no more than kPackedListMost): the core as sorted 64-bit keys;
+// the pixels at which fragments of exactly equal depth met where they decide the core are walked again afterwards, over the
+// instances that reach one of them, with the reference's insertion (as in hybrid_tile_by_keys).
+template <int K, bool FAST, bool KEYS = false>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 2))) blend_first_k_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
     uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
 {
+    static_assert(!(KEYS && FAST), "the keys of this mode are for the exact path");
     __shared__ TileStageQ st;
     __shared__ QuadrantLists ql;
     const uint32_t tile = block_tile(tile_order);
@@ -873,10 +913,36 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16
     const TilePixel px = quadrant_tile_pixel(tile, grid_w, lane, width, height);
     float ca[K], cd[K];
     uint32_t ci[K];
-    first_k_core_init<K>(cd, ca, ci);
-    first_k_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
-    if (!px.inside) return;
-    first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+    if constexpr (KEYS) {
+        CoreKey core[K];
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            core[i] = make_key(__FLT_MAX__, 0u);
+            asm volatile("" : "+v"(core[i]));      // one register pair per slot, never a wide tuple
+        }
+        float tie = __FLT_MAX__;
+        const KeyFormat fmt = key_format(last > first ? last - first : 1u);
+        first_k_key_walk<K, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, core, tie, fmt);
+        const bool again = px.inside && ((tie < __FLT_MAX__ && tie <= key_depth(core[K - 1])) || key_core_tied<K>(core, fmt));
+        const uint64_t again_lanes = __ballot(again);
+        first_k_core_unpack<K>(core, inst, first, last, cd, ca, ci, fmt);
+        if (px.inside && !again) first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+        if (again_lanes == 0) return;
+        // (the lane and its pixel are worked out afresh: nothing of the first walk has to live through the composite for this)
+        uint32_t lane_again = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        asm volatile("" : "+v"(lane_again));
+        const TilePixel px_again = quadrant_tile_pixel(tile, grid_w, lane_again, width, height);
+        first_k_core_init<K>(cd, ca, ci);
+        first_k_walk<K, false, true, false, HTGS_PRIM_FLOATS / 4, true>(st, ql, inst, prim, first, last, lane_again, px_again.pt, px_again.cx, px_again.cy, cd, ca, ci,
+                                                                         nullptr, again_lanes);
+        if ((again_lanes >> lane_again & 1ull) != 0)
+            first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px_again.x, px_again.y, chw, median);
+    } else {
+        first_k_core_init<K>(cd, ca, ci);
+        first_k_walk<K, FAST, true>(st, ql, inst, prim, first, last, lane, px.pt, px.cx, px.cy, cd, ca, ci);
+        if (!px.inside) return;
+        first_k_composite<K>(prim, cd, ca, ci, image, depths, width, height, px.x, px.y, chw, median);
+    }
 }
 
 // A core and a tie depth (3K + 1 rows of 64 lanes at from[]) join the running ones: they cover the stretch of the list

@@ -297,7 +297,7 @@ static int sort_pairs(hipStream_t s, void *const keys[2], uint32_t *const vals[2
     uint32_t *hist = sort_tmp;
     uint32_t *totals = sort_tmp + (size_t)kRadix * n_blocks;
     int cur = 0;
-    // the passes share the key's bits evenly (13 bits: 7 + 6 rather than 8 + 5): fewer digits per pass are longer runs
+    // the passes share the key's bits evenly (14 bits: 7 + 7 rather than 8 + 6): fewer digits per pass are longer runs
     // per digit in every block's output
     const int passes = (end_bit + kBits - 1) / kBits, step = passes > 0 ? (end_bit + passes - 1) / passes : kBits;
     for (int shift = 0; shift < end_bit; shift += step) {

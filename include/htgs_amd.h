@@ -212,8 +212,8 @@ int htgs_extract_ranges(const htgs_frame *f, int selector);
  * value buffer vals[1 - selector] as scratch (its content is lost; NULL: a slower path without it, one workgroup per
  * tile).  Without long_tiles the stage reads vals[selector] only.  How a long list is split over workgroups depends on its
  * length and on n_instances alone: results do not depend on the order in which workgroups run.
- * HYBRID_BLEND with f->long_tiles and a threshold of no more than 8192: the kernel with one wave per tile keeps the K
- * nearest fragments of a pixel as sorted 64-bit keys, depth above alpha as a fraction of 19 to 23 bits, the more the
+ * HYBRID_BLEND, and ALPHA_BLEND_FIRST_K without fast_math, with f->long_tiles and a threshold of no more than 8192: the
+ * kernel with one wave per tile keeps the K nearest fragments of a pixel as sorted 64-bit keys, depth above alpha as a fraction of 19 to 23 bits, the more the
  * shorter the tile's list (rounded, 2^-20 at most: the image comes out within 1e-6 of the walk that keeps alphas as floats,
  * which is the one without long_tiles or with a larger threshold), and pixels at which fragments of exactly equal depth met where they decide the K nearest are walked a
  * second time with the reference's insertion, which the keys do not reproduce. */

@@ -1,13 +1,15 @@
-"""HYBRID_BLEND's kernel with one wave per tile keeps the K nearest fragments as sorted 64-bit keys (depth above alpha as a
+"""The kernels of HYBRID_BLEND and ALPHA_BLEND_FIRST_K with one wave per tile keep the K nearest fragments as sorted 64-bit keys (depth above alpha as a
 fraction of 19 to 23 bits above the place in the list) when the frame has the list for long tiles and no list of the launch
 is longer than 8192; pixels at which fragments of exactly equal depth met where they decide the core are walked again with the
-reference's exchange insertion (R/include/hybrid_blend/kernels/inference.cuh:159-167).  Without that list -- or with a
+reference's exchange insertion (R/include/hybrid_blend/kernels/inference.cuh:159-167,
+R/include/alpha_blend_first_k/kernels/inference.cuh:155-163).  Without that list -- or with a
 threshold above 8192 -- the same kernel keeps (depth, alpha, index) triples and inserts by exchange throughout.  The two
 must agree to the rounding of the alphas (2^-20 each), and both with the CPU oracle to the rasterizer's 1e-4."""
 import numpy as np
 import pytest
 
 from htgs_amd.synthetic import make_scene
+from htgs_amd.torch_bindings import RasterizerMode
 from test_gpu_long_tiles import NEVER, render, with_coincident_copies
 from util import oracle_render
 
@@ -60,3 +62,24 @@ def test_keys_with_the_other_output_layouts(cuda, to_chw, median):
     assert float(np.abs(keyed - exchanged).max()) <= BETWEEN
     # (the median depth is one fragment's depth: the same fragment unless two transmittances straddle 1/2 within the alphas' rounding)
     assert float((np.abs(keyed_depth - exchanged_depth) > 1e-5 * max(1.0, float(np.abs(exchanged_depth).max()))).mean()) <= (1e-3 if median else 0.0)
+
+
+FIRST_K = RasterizerMode.ALPHA_BLEND_FIRST_K
+
+
+@pytest.mark.parametrize("config,n,K,copies", [(0, 3000, 4, 1), (0, 3000, 1, 1), (1, 60_000, 16, 1), (2, 100_000, 32, 1), (3, 8_000, 16, 1),
+                                                 (0, 1500, 4, 3), (1, 20_000, 16, 2)])
+def test_first_k_keys_against_the_exchange_walk_and_the_oracle(cuda, config, n, K, copies):
+    """ALPHA_BLEND_FIRST_K has no tail that takes what leaves the core: which of two fragments of equal depth holds the
+    K-th place decides the pixel, so the second walk is what keeps the keyed kernel on the reference's result."""
+    print(f"case config={config} n={n} K={K} copies={copies}", flush=True)
+    scene = make_scene(config, n)
+    if copies > 1: scene = with_coincident_copies(scene, copies)
+    ref = oracle_render(scene, 1, K)
+    keyed, keyed_depth, _ = render(scene.to(cuda), K, 0, mode=FIRST_K)
+    exchanged, exchanged_depth, _ = render(scene.to(cuda), K, NEVER, mode=FIRST_K)
+    scale = max(1.0, float(np.abs(ref["depth"]).max()))
+    between = float(np.abs(keyed - exchanged).max())
+    print(f"  keys against exchange: image {between:.3g}, depth {float(np.abs(keyed_depth - exchanged_depth).max()):.3g} (depths up to {scale:.3g})", flush=True)
+    assert between <= BETWEEN and float(np.abs(keyed_depth - exchanged_depth).max()) <= BETWEEN * scale
+    assert float(np.abs(keyed - ref["image"]).max()) <= TOL and float(np.abs(keyed_depth - ref["depth"]).max()) <= TOL
