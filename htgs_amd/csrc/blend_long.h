@@ -429,8 +429,9 @@ __device__ __forceinline__ bool long_part_done(const uint32_t *long_tiles, uint3
 
 // One wave per tile; the tiles with very long lists are left to blend_hybrid_long_kernel.
 // KEYS (with long_tiles and a threshold of no more than kPackedListMost): the core as sorted 64-bit keys, hybrid_tile_by_keys.
+// (K = 32: two registers a slot leave room for four waves per SIMD instead of three -- cfg2 442 -> 488 FPS)
 template <int K, bool FAST, bool KEYS = false>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : 3))) blend_hybrid_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K <= 16 ? 5 : KEYS ? 4 : 3))) blend_hybrid_kernel(
     const uint32_t *__restrict__ ranges, const uint32_t *__restrict__ inst, const float4 *__restrict__ prim,
     float *__restrict__ image, float *__restrict__ depths, uint32_t width, uint32_t height, uint32_t grid_w, int chw, int median,
     uint32_t *__restrict__ long_tiles, uint32_t long_threshold, uint32_t part_floor, const uint32_t *__restrict__ tile_order)
