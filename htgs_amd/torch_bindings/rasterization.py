@@ -487,7 +487,12 @@ def rasterize(
     use_median_depth: bool,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """Inference render: ``(image, depth)`` with ``image`` ``[3,H,W]`` (``to_chw``) or ``[H,W,3]`` clamped to
-    [0,1] and ``depth`` ``[1,H,W]`` / ``[H,W,1]`` (reference: rasterization.py:140-163)."""
+    [0,1] and ``depth`` ``[1,H,W]`` / ``[H,W,1]`` (reference: rasterization.py:140-163).
+
+    HYBRID_BLEND and ALPHA_BLEND_FIRST_K hold a pixel's K nearest fragments as sorted 64-bit keys, in which alpha is a
+    fraction of 19 to 23 bits (image within 1e-6, depth within 1e-5 of the same walk with alphas kept as floats; every
+    test of a fragment is taken on the float).  ``FrameBuffers(..., long_list_threshold=8193).run()`` is that other
+    walk: any threshold above 8192 selects it, a tenth slower in the blend stage."""
     with torch.no_grad():
         pool = ScratchPool.current(positions.device) if isinstance(positions, torch.Tensor) and positions.is_cuda else None
         image, depth = FrameBuffers(positions, scales, rotations, opacities, sh_0, sh_rest, settings,
