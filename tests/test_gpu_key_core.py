@@ -83,3 +83,14 @@ def test_first_k_keys_against_the_exchange_walk_and_the_oracle(cuda, config, n, 
     print(f"  keys against exchange: image {between:.3g}, depth {float(np.abs(keyed_depth - exchanged_depth).max()):.3g} (depths up to {scale:.3g})", flush=True)
     assert between <= BETWEEN and float(np.abs(keyed_depth - exchanged_depth).max()) <= BETWEEN * scale
     assert float(np.abs(keyed - ref["image"]).max()) <= TOL and float(np.abs(keyed_depth - ref["depth"]).max()) <= TOL
+
+
+@pytest.mark.parametrize("config,n,K,mode", [(0, 3000, 4, 0), (1, 60_000, 16, 0), (1, 60_000, 16, 1)])
+def test_a_threshold_above_8192_keeps_the_alphas_as_floats(cuda, config, n, K, mode):
+    """``long_list_threshold = 8193`` selects the walk with (depth, alpha, index) triples, whose image and depth equal the
+    CPU oracle's bit for bit (both implement one rounding convention)."""
+    scene = make_scene(config, n)
+    ref = oracle_render(scene, mode, K)
+    image, depth, long_tiles = render(scene.to(cuda), K, 8193, mode=RasterizerMode(mode))
+    assert long_tiles == 0
+    assert np.array_equal(image, ref["image"]) and np.array_equal(depth, ref["depth"])
