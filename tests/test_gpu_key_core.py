@@ -36,7 +36,7 @@ def test_keys_against_the_exchange_walk_and_the_oracle(cuda, config, n, K):
     assert float(np.abs(exchanged - ref["image"]).max()) <= TOL and float(np.abs(exchanged_depth - ref["depth"]).max()) <= TOL
 
 
-@pytest.mark.parametrize("config,n,K,copies", [(0, 1500, 4, 3), (1, 20_000, 16, 2), (0, 1500, 1, 2)])
+@pytest.mark.parametrize("config,n,K,copies", [(0, 1500, 4, 3), (1, 20_000, 16, 2), (0, 1500, 1, 2), (0, 1500, 32, 2), (1, 20_000, 8, 3), (0, 1500, 2, 3)])
 def test_keys_where_every_fragment_meets_its_own_depth(cuda, config, n, K, copies):
     """Coincident copies of every Gaussian: every pixel with two fragments in its core is walked a second time."""
     print(f"case config={config} n={n} K={K} copies={copies}", flush=True)
@@ -68,7 +68,7 @@ FIRST_K = RasterizerMode.ALPHA_BLEND_FIRST_K
 
 
 @pytest.mark.parametrize("config,n,K,copies", [(0, 3000, 4, 1), (0, 3000, 1, 1), (1, 60_000, 16, 1), (2, 100_000, 32, 1), (3, 8_000, 16, 1),
-                                                 (0, 1500, 4, 3), (1, 20_000, 16, 2)])
+                                                 (0, 1500, 4, 3), (1, 20_000, 16, 2), (0, 1500, 32, 2), (1, 20_000, 8, 3)])
 def test_first_k_keys_against_the_exchange_walk_and_the_oracle(cuda, config, n, K, copies):
     """ALPHA_BLEND_FIRST_K has no tail that takes what leaves the core: which of two fragments of equal depth holds the
     K-th place decides the pixel, so the second walk is what keeps the keyed kernel on the reference's result."""
