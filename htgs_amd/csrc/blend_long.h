@@ -178,6 +178,9 @@ __device__ __forceinline__ void hybrid_key_walk(TileStageQ &st, QuadrantLists &q
         if (depth < key_depth(core[K - 1]) && f.alpha >= kMinAlphaCore) {
             // (a fragment that enters the core has the alpha that its key holds from here on: what the colour sums
             // receive now is what is taken out of them again for the entries of the finished core)
+            // (the fast path's alpha is opacity * 2^t with the opacity held to 1 and t <= 0 up to the rounding of the staged
+            // quadratic: held to 1 here, the fraction has no room for more; the exact path's is held to 1 when it is evaluated)
+            if constexpr (FAST) p3 = p3 < 1.0f ? p3 : 1.0f;
             const uint32_t low = key_pack(p3, float_to_bits(col.w) - first, fmt);
             p3 = key_alpha(low, fmt);
             tail.c0 = __builtin_fmaf(p3, col.x, tail.c0);

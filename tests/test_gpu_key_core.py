@@ -94,3 +94,18 @@ def test_a_threshold_above_8192_keeps_the_alphas_as_floats(cuda, config, n, K, m
     image, depth, long_tiles = render(scene.to(cuda), K, 8193, mode=RasterizerMode(mode))
     assert long_tiles == 0
     assert np.array_equal(image, ref["image"]) and np.array_equal(depth, ref["depth"])
+
+
+def test_fast_path_holds_a_fully_opaque_fragment(cuda):
+    """alpha = 1 is the largest fraction a key can hold (fragments are held to it): an opaque Gaussian in front of another
+    hides it at the pixel through both centres, on both paths."""
+    from htgs_amd.torch_bindings import fast_rasterize, rasterize
+    from test_oracle_ties import PX
+    from util import tie_scene
+    scene = tie_scene([2.0, 3.0], [1.0, 0.8], [[0.2, 0.5, 0.8], [0.9, 0.1, 0.1]]).to(cuda)
+    settings = scene.settings(RasterizerMode.HYBRID_BLEND, 4)
+    fast = fast_rasterize(*scene.gaussians(), settings, True)
+    image, _ = rasterize(*scene.gaussians(), settings, True, False)
+    want = np.array([0.2, 0.5, 0.8])
+    assert np.abs(image[:, PX, PX].cpu().numpy() - want).max() <= 1e-6
+    assert np.abs(fast[:, PX, PX].cpu().numpy() - want).max() <= 1e-5
